@@ -1,0 +1,480 @@
+"""Pins the CPU oracle (oracle/) against independent formulations.
+
+The reference tree holds no golden vectors for these ops and its kernels cannot
+be built in this image, so each oracle function is checked against what the
+mathematics fixes: brute force, closed forms, invariants and hand-computed tiny
+cases chosen so that a wrong sign, index, tie rule or summation order fails.
+"""
+import numpy as np
+import pytest
+
+from hgcalml_amd import workloads
+
+
+# ------------------------------------------------------------------ helpers
+
+def serial_distsq(a, b):
+    """((0 + d0^2) + d1^2) + ... in fp32; a [M,C], b [C] or [M,C]"""
+    acc = np.zeros(a.shape[0], np.float32)
+    for c in range(a.shape[1]):
+        d = (a[:, c] - (b[c] if b.ndim == 1 else b[:, c])).astype(np.float32)
+        acc = (acc + (d * d).astype(np.float32)).astype(np.float32)
+    return acc
+
+
+def brute_knn_row(coords, lo, hi, i, allowed=None):
+    """all other points of the event, ordered by (d^2, index); returns (idx, d^2)"""
+    j = np.arange(lo, hi)
+    d = serial_distsq(coords[lo:hi], coords[i])
+    keep = j != i
+    if allowed is not None:
+        keep &= allowed[lo:hi]
+    j, d = j[keep], d[keep]
+    o = np.lexsort((j, d))
+    return j[o], d[o]
+
+
+def check_knn_rows(oracle, idx, dist, coords, row_splits, K, rows, direction=None, tf_compatible=False,
+                   radius=None):
+    """every listed row: oracle set == brute-force set unless the K-th boundary
+    is an exact tie, in which case the row must still be a valid kNN set.
+    Returns the number of tie rows."""
+    ties = 0
+    ev = np.searchsorted(row_splits[1:], rows, side="right")
+    allowed = None if direction is None else ~np.isin(direction, (1, 2))
+    for i, e in zip(rows, ev):
+        lo, hi = row_splits[e], row_splits[e + 1]
+        if direction is not None and direction[i] in (0, 2):
+            assert idx[i, 0] == i
+            assert (idx[i, 1:] == (i if tf_compatible else -1)).all()
+            assert (dist[i] == 0).all()
+            continue
+        bj, bd = brute_knn_row(coords, lo, hi, i, allowed)
+        if radius is not None:
+            m = bd <= np.float32(np.float32(radius) * np.float32(radius))
+            bj, bd = bj[m], bd[m]
+        want = min(K - 1, len(bj))
+        got_i, got_d = idx[i, 1:], dist[i, 1:]
+        valid = got_i >= 0 if not tf_compatible else np.arange(1, K) <= want
+        assert idx[i, 0] == i and dist[i, 0] == 0
+        assert valid.sum() == want, (i, valid.sum(), want)
+        gi, gd = got_i[valid], got_d[valid]
+        # padding
+        if not tf_compatible:
+            assert (got_d[~valid] == 0).all()
+        else:
+            assert (got_i[~valid] == i).all() and (got_d[~valid] == 0).all()
+        # distances bitwise per index, all in the same event, no duplicates
+        assert len(set(gi.tolist())) == len(gi)
+        assert ((gi >= lo) & (gi < hi)).all()
+        ref_d = serial_distsq(coords[gi], coords[i])
+        assert (ref_d.view(np.int32) == gd.view(np.int32)).all()
+        if want == 0:
+            continue
+        boundary_tie = want < len(bj) and bd[want - 1] == bd[want]
+        if not boundary_tie:
+            assert set(gi.tolist()) == set(bj[:want].tolist()), i
+        else:
+            ties += 1
+            dk = bd[want - 1]
+            assert (gd <= dk).all()
+            assert set(bj[bd < dk].tolist()) <= set(gi.tolist())
+    return ties
+
+
+# ------------------------------------------------------------------ binning
+
+def test_bin_kernel_matches_closed_form(oracle):
+    rng = np.random.default_rng(1)
+    n = 64
+    coords = (rng.random((n, 3), dtype=np.float32) * np.float32(3.0)).astype(np.float32)
+    bw = np.array([0.5], np.float32)
+    nb = np.array([6, 7, 6], np.int32)
+    coords[5] = [1.0, 1.5, 2.5]          # exactly on bin edges
+    coords[9, 1] = 3.6                   # index 7 -> beyond n_bins[1] -> falls back to 0
+    coords[11, 0] = -0.7                 # negative index -> 0
+    rs = np.array([0, 20, 20, 64], np.int32)   # with an empty event
+    binass, flat, nper, bad = oracle.bin_by_coordinates_kernel(coords, rs, bw, nb)
+    assert bad == 2
+    k = np.trunc(coords / bw[0]).astype(np.int64)
+    k[(k < 0) | (k >= nb[None, :])] = 0
+    ev = np.array([0] * 20 + [2] * 44)
+    want_flat = ((ev * nb[0] + k[:, 0]) * nb[1] + k[:, 1]) * nb[2] + k[:, 2]
+    assert (flat == want_flat).all()
+    assert (binass[:, 0] == ev).all() and (binass[:, 1:] == k).all()
+    assert (binass[5] == [0, 2, 3, 5]).all()
+    assert (nper == np.bincount(want_flat, minlength=6 * 7 * 6 * 3)).all() and nper.sum() == n
+
+
+def test_bin_wrapper_formulas(oracle):
+    rng = np.random.default_rng(2)
+    x = (rng.random((500, 3), dtype=np.float32) * np.array([4., 2., 1.], np.float32)
+         + np.array([-3., 5., 0.], np.float32)).astype(np.float32)
+    rs = np.array([0, 200, 500], np.int32)
+    binass, flat, nb, bw, nper = oracle.BinByCoordinates(x, rs, n_bins=10)
+    ext = (x - x.min(0)).max(0).astype(np.float32) + np.float32(1e-3)
+    assert bw.shape == (1,) and bw[0] == np.max(ext / np.float32(10))
+    assert (nb == (ext / bw[0] + np.float32(1)).astype(np.int32)).all()
+    assert nb.max() in (10, 11) and (nb >= 1).all()
+    assert nper.shape == (int(np.prod(nb)) * 2,) and nper.sum() == 500
+    # every point lies inside its bin (up to the fp32 rounding of the divide)
+    shifted = x - x.min(0)
+    assert (np.abs(shifted / bw[0] - binass[:, 1:] - 0.5) <= 0.5 + 1e-4).all()
+    # a degenerate dimension gets extent 1 + 1e-3
+    x[:, 2] = 7.0
+    _, _, nb2, bw2, _ = oracle.BinByCoordinates(x, rs, n_bins=10)
+    assert nb2[2] == int(np.float32(1.001) / bw2[0] + np.float32(1))
+    # bin_width given instead
+    _, _, nb3, bw3, _ = oracle.BinByCoordinates(x, rs, bin_width=np.array([0.25], np.float32))
+    assert bw3[0] == np.float32(0.25) and nb3[0] == int(ext[0] / np.float32(0.25) + 1)
+
+
+# ------------------------------------------------------------------ shells
+
+@pytest.mark.parametrize("nb", [(4, 5), (3, 4, 5), (6, 2, 3), (2, 3, 2, 3), (2, 2, 3, 2, 2)])
+def test_shells_partition_grid(oracle, nb):
+    rng = np.random.default_rng(3)
+    nb = np.array(nb, np.int32)
+    total = int(np.prod(nb))
+    for _ in range(4):
+        centre = np.array([rng.integers(0, b) for b in nb], np.int32)
+        seen = []
+        for d in range(int(nb.max()) + 1):
+            cells = oracle.shell_enumerate(nb, centre, d)
+            unr = np.array(np.unravel_index(cells, nb)).T.reshape(-1, len(nb))
+            assert (np.abs(unr - centre[None, :]).max(axis=1) == d).all()
+            # dimension 0 is the most significant digit: the flat index rises
+            assert (np.diff(cells) > 0).all()
+            seen.append(cells)
+        seen = np.concatenate(seen)
+        assert len(seen) == total and len(np.unique(seen)) == total
+        assert len(oracle.shell_enumerate(nb, centre, int(nb.max()) + 1)) == 0
+
+
+# ------------------------------------------------------------------ kNN
+
+def test_knn_sets_vs_brute_force_uniform(oracle):
+    cfg = workloads.cfg1(scale=0.1)  # 2000 points, K=16
+    coords = cfg["coords"]
+    rs = np.array([0, 700, 2000], np.int32)
+    idx, dist = oracle.BinnedSelectKnn(16, coords, rs, n_bins=8)
+    ties = check_knn_rows(oracle, idx, dist, coords, rs, 16, np.arange(2000))
+    assert ties == 0
+    # slot order of the reference algorithm is generally not distance sorted
+    assert (np.diff(dist[:, 1:], axis=1) < 0).any()
+
+
+def test_knn_sets_vs_brute_force_clustered_4d(oracle):
+    cfg = workloads.cfg2(scale=0.04)  # 6000 points, 4-D distance over 3 binned dims
+    coords = cfg["coords"]
+    rs = np.array([0, 2500, 6000], np.int32)
+    idx, dist = oracle.BinnedSelectKnn(64, coords, rs, n_bins=12)
+    rows = np.random.default_rng(4).choice(6000, 600, replace=False)
+    assert check_knn_rows(oracle, idx, dist, coords, rs, 64, rows) == 0
+
+
+def test_knn_small_event_padding_direction_and_tf_compat(oracle):
+    rng = np.random.default_rng(5)
+    coords = rng.standard_normal((330, 3)).astype(np.float32)
+    rs = np.array([0, 7, 7, 30, 330], np.int32)  # 7 < K, empty, 23 < K, 300
+    K = 24
+    for tfc in (False, True):
+        idx, dist = oracle.BinnedSelectKnn(K, coords, rs, n_bins=5, tf_compatible=tfc)
+        check_knn_rows(oracle, idx, dist, coords, rs, K, np.arange(330), tf_compatible=tfc)
+    direction = rng.integers(0, 4, size=330).astype(np.int32)
+    idx, dist = oracle.BinnedSelectKnn(K, coords, rs, n_bins=5, direction=direction)
+    check_knn_rows(oracle, idx, dist, coords, rs, K, np.arange(330), direction=direction)
+    # radius mask (select_knn rule: keep d^2 <= r^2)
+    idx, dist = oracle.BinnedSelectKnn(K, coords, rs, n_bins=5, max_radius=0.6)
+    ci, cd = oracle.canonical_knn(idx, dist)
+    check_knn_rows(oracle, ci, cd, coords, rs, K, np.arange(330), radius=0.6)
+    assert (ci[:, 1:] < 0).any() and (np.diff((ci[:, 1:] < 0).astype(int), axis=1) >= 0).all()
+
+
+def test_knn_lattice_ties_are_valid_sets(oracle):
+    g = np.arange(8, dtype=np.float32)
+    coords = np.stack(np.meshgrid(g, g, g, indexing="ij"), -1).reshape(-1, 3)
+    rs = np.array([0, 512], np.int32)
+    idx, dist = oracle.BinnedSelectKnn(8, coords, rs, n_bins=5)
+    ties = check_knn_rows(oracle, idx, dist, coords, rs, 8, np.arange(512))
+    assert ties > 100  # the lattice makes most K-th boundaries exact ties
+
+
+def test_default_n_bins_formula(oracle):
+    assert oracle.default_knn_n_bins(20000, 16, 3) == 30
+    assert oracle.default_knn_n_bins(150000, 64, 3) == 30
+    assert oracle.default_knn_n_bins(1000, 32, 3) == 10   # 1000^(1/3) = 10 (float32 pow)
+    assert oracle.default_knn_n_bins(100, 64, 3) == 5     # clamp below
+    assert oracle.default_knn_n_bins(4000, 32, 2) == 30   # sqrt(4000) = 63 -> clamp
+
+
+# ------------------------------------------------------------------ index replacer
+
+def test_index_replacer(oracle):
+    rep = np.array([10, 11, 12, 13], np.int32)
+    tbr = np.array([[0, 3, -1], [2, -5, 7]], np.int32)
+    out = oracle.IndexReplacer(tbr, rep)
+    assert (out == [[10, 13, -1], [12, -5, 0]]).all()  # 7 is out of range: left at the zero init
+
+
+# ------------------------------------------------------------------ accumulate forward
+
+def np_accumulate(w, x, idx, mean_and_max=True):
+    """gather -> multiply -> slot-serial fp32 sum / K, and max with the
+    reference's rules, vectorised over (vertex, feature)."""
+    n, K = idx.shape
+    F = x.shape[1]
+    s = np.zeros((n, F), np.float32)
+    best = np.zeros((n, F), np.float32)
+    arg = np.zeros((n, F), np.int32)
+    for k in range(K):
+        j = idx[:, k]
+        ok = (j >= 0)[:, None]
+        wf = (x[np.maximum(j, 0)] * w[:, k:k + 1]).astype(np.float32)
+        s = np.where(ok, (s + wf).astype(np.float32), s)
+        take = ok & ((wf >= best) | (k == 0))
+        best = np.where(take, wf, best)
+        arg = np.where(take, j[:, None], arg)
+    mean = (s / np.float32(K)).astype(np.float32)
+    return (np.concatenate([mean, best], 1), arg) if mean_and_max else (mean, arg)
+
+
+def test_accumulate_hand_cases(oracle):
+    x = np.array([[1., -2.], [3., 4.], [-5., 0.5]], np.float32)
+    idx = np.array([[0, 1, 2], [1, 2, -1], [-1, 0, 1]], np.int32)
+    w = np.array([[1., .5, .25], [2., 1., 9.], [7., 1., 1.]], np.float32)
+    out, arg = oracle.AccumulateLinKnn(w, x, idx)
+    # vertex 0: wf = [1,-2],[1.5,2],[-1.25,.125]; mean = sum/3 ; max: slot 0 seeds, then >=
+    assert np.allclose(out[0], [1.25 / 3, 0.125 / 3, 1.5, 2.0])
+    assert (arg[0] == [1, 1]).all()
+    # vertex 1: slots (1,w2) (2,w1) pad: wf=[6,8],[-5,.5]; divides by K=3, not by 2
+    assert np.allclose(out[1], [1. / 3, 8.5 / 3, 6., 8.])
+    assert (arg[1] == [1, 1]).all()
+    # vertex 2: slot 0 is padding -> max floored at 0 with index 0 unless something >= 0 comes
+    # wf slot1 = [1,-2], slot2 = [3,4]
+    assert np.allclose(out[2], [4. / 3, 2. / 3, 3., 4.])
+    assert (arg[2] == [1, 1]).all()
+    # all-negative contributions with slot 0 padded: max stays 0, index 0
+    x2 = -np.abs(x)
+    out2, arg2 = oracle.AccumulateLinKnn(w, x2, idx)
+    assert (out2[2, 2:] == 0).all() and (arg2[2] == 0).all()
+    # exact tie: the later slot wins
+    x3 = np.array([[2.], [2.], [2.]], np.float32)
+    out3, arg3 = oracle.AccumulateLinKnn(np.ones((3, 3), np.float32), x3, np.array([[0, 1, 2]] * 3, np.int32))
+    assert (arg3 == 2).all() and (out3[:, 1] == 2).all()
+    # mean only
+    out4, _ = oracle.AccumulateLinKnn(w, x, idx, mean_and_max=False)
+    assert out4.shape == (3, 2) and np.allclose(out4, out[:, :2])
+
+
+@pytest.mark.parametrize("F", [3, 32])
+def test_accumulate_vs_numpy_composition(oracle, F):
+    rng = np.random.default_rng(6)
+    n, K = 128, 8
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    idx = np.stack([rng.permutation(n)[:K] for _ in range(n)]).astype(np.int32)
+    idx[:, 0] = np.arange(n)
+    idx[10:30, 5:] = -1           # -1 tail
+    idx[40, 0] = -1               # slot 0 missing
+    idx[50, 3:] = 50              # duplicated-self padding
+    d = rng.random((n, K), dtype=np.float32)
+    for mm in (True, False):
+        out, arg = oracle.AccumulateKnn(d, x, idx, mean_and_max=mm)
+        w = np.exp(-d).astype(np.float32)
+        ref, rarg = np_accumulate(w, x, idx, mm)
+        assert (out.view(np.int32) == ref.view(np.int32)).all()
+        if mm:
+            assert (arg == rarg).all()
+
+
+# ------------------------------------------------------------------ accumulate gradient
+
+def test_accumulate_grad_vs_autograd(oracle):
+    import torch
+    rng = np.random.default_rng(7)
+    n, K, F = 96, 8, 5
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    # unique neighbours per row (self only in slot 0), as the op's contract asks
+    idx = np.stack([np.concatenate([[v], rng.permutation(np.delete(np.arange(n), v))[:K - 1]])
+                    for v in range(n)]).astype(np.int32)
+    idx[5:20, 6:] = -1
+    w = (rng.random((n, K)) + 0.1).astype(np.float32)
+    g = rng.standard_normal((n, 2 * F)).astype(np.float32)
+    out, arg = oracle.AccumulateLinKnn(w, x, idx)
+    gw, gx = oracle.accumulate_knn_grad_kernel(g, w, x, idx, arg)
+
+    tw = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tidx = torch.tensor(idx, dtype=torch.int64)
+    valid = (tidx >= 0)
+    gath = tx[tidx.clamp(min=0)] * tw[:, :, None]
+    gath_mean = torch.where(valid[:, :, None], gath, torch.zeros_like(gath))
+    mean = gath_mean.sum(1) / K
+    gath_max = torch.where(valid[:, :, None], gath, torch.full_like(gath, -1e30))
+    mx = gath_max.max(1).values
+    assert np.allclose(torch.cat([mean, mx], 1).detach().numpy(), out, rtol=1e-5, atol=1e-6)
+    (torch.cat([mean, mx], 1) * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    assert np.allclose(gw, tw.grad.numpy(), rtol=1e-5, atol=1e-5)
+    assert np.allclose(gx, tx.grad.numpy(), rtol=1e-5, atol=1e-5)
+    # mean-only mode is detected from the gradient width
+    gw1, gx1 = oracle.accumulate_knn_grad_kernel(g[:, :F], w, x, idx, arg)
+    tw.grad = None
+    tx.grad = None
+    gath = tx[tidx.clamp(min=0)] * tw[:, :, None]
+    mean = torch.where(valid[:, :, None], gath, torch.zeros_like(gath)).sum(1) / K
+    (mean * torch.tensor(g[:, :F], dtype=torch.float64)).sum().backward()
+    assert np.allclose(gw1, tw.grad.numpy(), rtol=1e-5, atol=1e-5)
+    assert np.allclose(gx1, tx.grad.numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_accumulate_grad_summation_order_and_self_rule(oracle):
+    """Feature gradient = ordered scatter of ((g/K)*w + max part); the ordered
+    unbuffered numpy scatter reproduces the ascending (vertex, slot) order."""
+    rng = np.random.default_rng(8)
+    n, K, F = 64, 6, 4
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    idx = np.stack([rng.permutation(n)[:K] for _ in range(n)]).astype(np.int32)
+    idx[:, 0] = np.arange(n)
+    idx[7, 3:] = 7      # repeated self: max part may be counted once only
+    x[7] = 50.0         # make self the arg-max of vertex 7
+    idx[9, 4:] = -1
+    w = (rng.random((n, K)) + 0.5).astype(np.float32)
+    g = rng.standard_normal((n, 2 * F)).astype(np.float32)
+    _, arg = oracle.AccumulateLinKnn(w, x, idx)
+    assert (arg[7] == 7).all()
+    gw, gx = oracle.accumulate_knn_grad_kernel(g, w, x, idx, arg)
+
+    ref = np.zeros((n, F), np.float32)
+    gm = (g[:, :F] / np.float32(K)).astype(np.float32)
+    for v in range(n):
+        first_self = True
+        for k in range(K):
+            m = idx[v, k]
+            if m < 0:
+                continue
+            add = (gm[v] * w[v, k]).astype(np.float32)
+            hit = arg[v] == m
+            if m == v:
+                hit = hit & first_self
+                first_self = False if (arg[v] == m).any() else first_self
+            add = (add + np.where(hit, (g[v, F:] * w[v, k]).astype(np.float32), np.float32(0))).astype(np.float32)
+            ref[m] = (ref[m] + add).astype(np.float32)
+    assert (ref.view(np.int32) == gx.view(np.int32)).all()
+    # weight gradient of the repeated-self slots: every slot gets the max part
+    j = 7
+    want = np.float32(0)
+    acc_m = np.float32(0)
+    acc_x = np.float32(0)
+    for f in range(F):
+        acc_m = np.float32(acc_m + np.float32(g[j, f] * x[j, f]))
+        acc_x = np.float32(acc_x + np.float32(g[j, F + f] * x[j, f]))
+    want = np.float32(np.float32(np.float64(acc_m) * (1.0 / K)) + acc_x)
+    assert (gw[7, [0, 3, 4, 5]] == want).all()
+    assert (gw[9, 4:] == 0).all()
+
+
+# ------------------------------------------------------------------ condensates
+
+def bin_free_greedy(oracle, cfg, by_max_beta):
+    cc = cfg["ccoords"].astype(np.float32)
+    beta = cfg["betas"].reshape(-1)
+    rad = (cfg["dist"].reshape(-1) / np.float32(cfg["distance_threshold"])).astype(np.float32)
+    rs = cfg["row_splits"]
+    n = len(beta)
+    cc = cc - cc.min(0, keepdims=True)
+    # the position tie-break needs the stable bin order; take it from the binning oracle
+    n_bins_sc = max(4, min(int(np.ceil((n / 5) ** (1 / 3))), 25))
+    _, flat, _, _ = oracle.BinByCoordinates(cc[:, :3], rs, n_bins=n_bins_sc, calc_n_per_bin=False,
+                                            pre_normalized=True)
+    pos = np.empty(n, np.int64)
+    pos[np.argsort(flat, kind="stable")] = np.arange(n)
+    assignment = np.full(n, -1, np.int32)
+    asso = np.full(n, -1, np.int32)
+    alphas, ncond = [], [0]
+    for e in range(len(rs) - 1):
+        lo, hi = rs[e], rs[e + 1]
+        members = np.arange(lo, hi)
+        high = members[beta[lo:hi] > np.float32(cfg["beta_threshold"])]
+        order = high[np.lexsort((pos[high], -beta[high].astype(np.float64)))]
+        taken = np.zeros(n, bool)
+        best = np.full(n, np.float32(10e20), np.float32)
+        shower = 0
+        for a in order:
+            if taken[a]:
+                continue
+            taken[a] = True
+            d = np.zeros(hi - lo, np.float32)
+            for c in range(cc.shape[1]):
+                t = (cc[a, c] - cc[lo:hi, c]).astype(np.float32)
+                d = (d + (t * t).astype(np.float32)).astype(np.float32)
+            rsq = np.float32(rad[a] * rad[a])
+            inside = d <= rsq
+            if by_max_beta:
+                claim = inside & (assignment[lo:hi] == -1)
+            else:
+                claim = inside & ((best[lo:hi] * rsq).astype(np.float32) >= d)
+                best[lo:hi] = np.where(claim, d, best[lo:hi])
+            assignment[lo:hi] = np.where(claim, shower, assignment[lo:hi])
+            asso[lo:hi] = np.where(claim, a, asso[lo:hi])
+            taken[lo:hi] |= claim
+            alphas.append(a)
+            shower += 1
+        ncond.append(ncond[-1] + shower)
+    return assignment, asso, np.array(alphas, np.int32), np.array(ncond, np.int32)
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
+@pytest.mark.parametrize("t_d", [0.5, 0.15])
+def test_condensates_vs_bin_free_greedy(oracle, by_max_beta, t_d):
+    cfg = workloads.cfg5(scale=0.024, n_events=3)   # 3 x 1500 hits, many 0.999 beta ties
+    cfg["dist"] = (cfg["dist"] * 0 + t_d).astype(np.float32)
+    # per-hit radii, not just a constant
+    rng = np.random.default_rng(9)
+    cfg["dist"] = (cfg["dist"] * rng.uniform(0.6, 1.4, size=cfg["dist"].shape)).astype(np.float32)
+    b = cfg["betas"].reshape(-1)
+    assert (np.bincount((b * 1000).astype(int))[999] > 5)  # clipped ties are present
+    assignment, asso, alpha, is_cond, ncond = oracle.BuildAndAssignCondensatesBinned(
+        cfg["ccoords"], cfg["betas"], cfg["dist"], cfg["row_splits"], cfg["beta_threshold"],
+        assign_by_max_beta=by_max_beta)
+    r_assignment, r_asso, r_alpha, r_ncond = bin_free_greedy(oracle, cfg, by_max_beta)
+    assert (ncond == r_ncond).all()
+    assert (alpha == r_alpha).all()
+    assert (assignment[:, 0] == r_assignment).all()
+    assert (asso == r_asso).all()
+    # invariants of the reference wrapper / tests
+    assert (asso[alpha] == alpha).all()
+    assert is_cond.sum() == len(alpha) and is_cond[alpha, 0].all()
+    rs = cfg["row_splits"]
+    per_event_max = np.array([assignment[rs[e]:rs[e + 1]].max() + 1 for e in range(len(rs) - 1)])
+    assert (ncond == np.concatenate([[0], np.cumsum(per_event_max)])).all()
+    for e in range(len(rs) - 1):
+        assert (assignment[alpha[ncond[e]:ncond[e + 1]], 0] == np.arange(ncond[e + 1] - ncond[e])).all()
+
+
+@pytest.mark.parametrize("t_b", [1e-5, 0.1, 0.9999])
+def test_condensates_degenerate_coordinates_and_thresholds(oracle, t_b):
+    """4x3 grid x 2 events and all-zero coordinates (the structural cases of the
+    reference's tests/unit/condensate.py:40-128)."""
+    rng = np.random.default_rng(10)
+    gx, gy = np.meshgrid(np.linspace(0, 10, 4), np.linspace(0, 10, 3))
+    x = np.concatenate([np.stack([gx, gy], -1).reshape(-1, 2)] * 2).astype(np.float32)
+    beta = rng.random((24, 1)).astype(np.float32)
+    rs = np.array([0, 12, 24], np.int32)
+    for coords in (x, 0 * x):
+        a, asso, alpha, is_cond, ncond = oracle.BuildAndAssignCondensatesBinned(
+            coords, beta, np.ones_like(beta), rs, t_b, assign_by_max_beta=False)
+        high = beta[:, 0] > np.float32(t_b)
+        if coords.any():
+            # grid spacing 3.33 / 5 > radius 1: every high-beta hit is its own condensate
+            assert set(alpha.tolist()) == set(np.nonzero(high)[0].tolist())
+            assert (asso[high] == np.nonzero(high)[0]).all() and (asso[~high] == -1).all()
+        else:
+            # everything on one spot: one condensate per event that has any high-beta hit
+            for e in range(2):
+                h = np.nonzero(high[rs[e]:rs[e + 1]])[0] + rs[e]
+                n_e = ncond[e + 1] - ncond[e]
+                assert n_e == (1 if len(h) else 0)
+                if len(h):
+                    top = h[np.argmax(beta[h, 0])]
+                    assert (asso[rs[e]:rs[e + 1]] == top).all()
+        assert (a[alpha, 0] >= 0).all()
