@@ -1,0 +1,63 @@
+"""`AccumulateKnn` / `AccumulateLinKnn` — same call signatures and results as
+modules/accknn_op.py:18-89 of the reference, on torch tensors, differentiable
+w.r.t. distances/weights and features.
+
+Indices must be unique in each row, except for repeated self references used
+as padding; -1 entries are skipped (padding at the end of the row).
+"""
+import torch
+
+from . import globals as gl
+from . import ops
+
+
+class _AccumulateFn(torch.autograd.Function):
+    """op + registered gradient (modules/accknn_op.py:71-89)"""
+
+    @staticmethod
+    def forward(ctx, weights, features, indices, mean_and_max):
+        out, maxidx = torch.ops.hgcalml.accumulate_knn(weights, features, indices, 0, mean_and_max)
+        ctx.save_for_backward(weights, features, indices, maxidx)
+        ctx.indices_ref = indices
+        ctx.mark_non_differentiable(maxidx)
+        return out, maxidx
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_maxidx):
+        weights, features, indices, maxidx = ctx.saved_tensors
+        inv_off, inv_slots = ops.cached_inverse_neighbour_index(ctx.indices_ref)
+        gw, gx = torch.ops.hgcalml.accumulate_knn_grad(grad_out.contiguous(), weights, features, indices, maxidx,
+                                                       inv_off, inv_slots)
+        return gw, gx, None, None
+
+
+def _torch_composition(weights, features, indices, mean_and_max):
+    # the reference's pure-TF path (modules/accknn_op.py:27-36): padded slots
+    # contribute 0 to the mean and to the max
+    w = weights.unsqueeze(2)
+    safe = indices.clamp(min=0).to(torch.int64)
+    nfeat = features[safe]
+    nfeat = torch.where((indices < 0)[..., None], torch.zeros_like(nfeat), nfeat)
+    wfeat = w * nfeat
+    fout = wfeat.mean(dim=1)
+    if mean_and_max:
+        fout = torch.cat([fout, wfeat.max(dim=1).values], dim=1)
+    return fout, None
+
+
+def AccumulateLinKnn(weights, features, indices, mean_and_max=True, force_tf=False):
+    """Accumulates neighbour features with linear weights (not exp(-w) as AccumulateKnn)."""
+    if (not gl.acc_ops_use_tf_gradients) and (not force_tf):
+        return _AccumulateFn.apply(weights, features, indices, bool(mean_and_max))
+    return _torch_composition(weights, features, indices, mean_and_max)
+
+
+def AccumulateKnn(distances, features, indices, mean_and_max=True, force_tf=False):
+    """Weighted mean (and max) of neighbour features with weights exp(-distances).
+
+    Returns (out [N, 2F] (mean | max) or [N, F], arg-max neighbour index [N, F]).
+    """
+    weights = torch.exp(-distances)
+    if (not gl.acc_ops_use_tf_gradients) and (not force_tf):
+        return _AccumulateFn.apply(weights, features, indices, bool(mean_and_max))
+    return _torch_composition(weights, features, indices, mean_and_max)

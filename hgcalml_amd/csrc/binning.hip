@@ -1,0 +1,382 @@
+// Spatial binning: grid parameters, per-point bin assignment, stable sort into
+// bin order, bin boundary table, row gather and index replacement.
+//
+// Reference behaviour restated here:
+//   modules/bin_by_coordinates_op.py:46-71            (grid parameters)
+//   modules/compiled/bin_by_coordinates_kernel.cc:46-114 (assignment)
+//   modules/binned_select_knn_op.py:72-84             (sort + boundaries)
+//   modules/compiled/index_replacer_kernel.cc:29-40
+//
+// All of this is HBM-bound integer/byte work over N points (a few bytes per
+// point per pass); the sort and the scans use rocPRIM device primitives.
+#include "hgc_common.hpp"
+
+#include <cstring>
+#include <algorithm>
+
+#include <rocprim/rocprim.hpp>
+
+#include <cfloat>
+#include <cmath>
+
+namespace hgc {
+
+thread_local char g_last_error[512] = "";
+char *last_error_buffer() { return g_last_error; }
+
+namespace {
+
+constexpr int kMaxBinDims = 8;
+
+__global__ void fill_i32_kernel(int *p, int value, long long n) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = value;
+}
+
+__global__ void iota_i32_kernel(int *p, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = i;
+}
+
+// ---- grid parameters --------------------------------------------------------
+
+// stage 1: per-block column minima / maxima of the first n_dims columns
+__global__ __launch_bounds__(256) void column_minmax_kernel(const float *__restrict__ coords, int stride,
+                                                            int n_vert, int n_dims,
+                                                            float *__restrict__ partial /*[blocks][2][8]*/) {
+    float lo[kMaxBinDims], hi[kMaxBinDims];
+#pragma unroll
+    for (int c = 0; c < kMaxBinDims; ++c) {
+        lo[c] = FLT_MAX;
+        hi[c] = -FLT_MAX;
+    }
+    for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < n_vert; p += gridDim.x * blockDim.x) {
+#pragma unroll
+        for (int c = 0; c < kMaxBinDims; ++c) {
+            if (c < n_dims) {
+                float x = coords[(size_t)p * stride + c];
+                lo[c] = fminf(lo[c], x);
+                hi[c] = fmaxf(hi[c], x);
+            }
+        }
+    }
+    __shared__ float s_lo[4][kMaxBinDims], s_hi[4][kMaxBinDims];
+#pragma unroll
+    for (int c = 0; c < kMaxBinDims; ++c) {
+        float a = lo[c], b = hi[c];
+        for (int off = 32; off > 0; off >>= 1) {
+            a = fminf(a, __shfl_xor(a, off, kWave));
+            b = fmaxf(b, __shfl_xor(b, off, kWave));
+        }
+        if (lane_id() == 0) {
+            s_lo[threadIdx.x >> 6][c] = a;
+            s_hi[threadIdx.x >> 6][c] = b;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < kMaxBinDims) {
+        int c = threadIdx.x;
+        float a = fminf(fminf(s_lo[0][c], s_lo[1][c]), fminf(s_lo[2][c], s_lo[3][c]));
+        float b = fmaxf(fmaxf(s_hi[0][c], s_hi[1][c]), fmaxf(s_hi[2][c], s_hi[3][c]));
+        partial[((size_t)blockIdx.x * 2 + 0) * kMaxBinDims + c] = a;
+        partial[((size_t)blockIdx.x * 2 + 1) * kMaxBinDims + c] = b;
+    }
+}
+
+// stage 2: one wave folds the partials and derives shift / bin width / bin counts
+__global__ __launch_bounds__(64) void grid_params_kernel(const float *__restrict__ partial, int n_partial,
+                                                         int n_dims, int pre_normalized, int n_bins_scalar,
+                                                         const float *__restrict__ bin_width_in,
+                                                         float *__restrict__ shift, float *__restrict__ bin_width,
+                                                         int *__restrict__ n_bins) {
+    float lo[kMaxBinDims], hi[kMaxBinDims];
+#pragma unroll
+    for (int c = 0; c < kMaxBinDims; ++c) {
+        float a = FLT_MAX, b = -FLT_MAX;
+        for (int i = threadIdx.x; i < n_partial; i += kWave) {
+            a = fminf(a, partial[((size_t)i * 2 + 0) * kMaxBinDims + c]);
+            b = fmaxf(b, partial[((size_t)i * 2 + 1) * kMaxBinDims + c]);
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            a = fminf(a, __shfl_xor(a, off, kWave));
+            b = fmaxf(b, __shfl_xor(b, off, kWave));
+        }
+        lo[c] = a;
+        hi[c] = b;
+    }
+    if (threadIdx.x != 0) return;
+    float extent[kMaxBinDims];
+    float bw = 0.f;
+    for (int c = 0; c < n_dims; ++c) {
+        const float sh = pre_normalized ? 0.f : lo[c];
+        // the extent is the largest shifted coordinate; subtraction is monotonic,
+        // so that is (column max - shift)
+        float e = hi[c] - sh;
+        const float shifted_min = lo[c] - sh;
+        if (shifted_min == e) e = e + 1.f;
+        e = e + 1e-3f;
+        if (!isfinite(e)) e = 1.f;
+        extent[c] = e;
+        shift[c] = sh;
+        if (n_bins_scalar > 0) bw = fmaxf(bw, e / (float)n_bins_scalar);
+    }
+    if (n_bins_scalar <= 0) bw = bin_width_in[0];
+    bin_width[0] = bw;
+    for (int c = 0; c < n_dims; ++c) {
+        float nb = extent[c] / bw;
+        nb = nb + 1.f;
+        n_bins[c] = (int)nb;
+    }
+}
+
+// ---- per-point assignment ---------------------------------------------------
+
+__global__ __launch_bounds__(256) void bin_points_kernel(
+    const float *__restrict__ coords, int stride, const float *__restrict__ shift,
+    const int *__restrict__ row_splits, const float *__restrict__ bin_width, const int *__restrict__ n_bins,
+    int *__restrict__ binass, int *__restrict__ flat, int *__restrict__ n_per_bin,
+    int *__restrict__ n_out_of_range, int n_vert, int n_dims, int n_rs, int n_total_bins, int calc_n_per_bin) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_vert) return;
+    const float bw = bin_width[0];
+    int mul = 1, cell = 0, bad = 0;
+    for (int c = n_dims - 1; c >= 0; --c) {
+        float x = coords[(size_t)p * stride + c];
+        if (shift) x = x - shift[c];
+        int k = (int)(x / bw);
+        const int nb = n_bins[c];
+        if (k < 0 || k >= nb) {
+            k = 0;
+            ++bad;
+        }
+        binass[(size_t)p * (n_dims + 1) + c + 1] = k;
+        cell += k * mul;
+        mul *= nb;
+    }
+    // event = number of row splits (from the second on) that are <= p; the
+    // splits are non decreasing, so a binary search gives the linear scan's answer
+    int lo = 1, hi = n_rs;
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (row_splits[mid] > p)
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    const int ev = lo - 1;
+    cell += ev * mul;
+    if (bad && n_out_of_range) atomicAdd(n_out_of_range, bad);
+    if (cell >= n_total_bins) return;
+    binass[(size_t)p * (n_dims + 1)] = ev;
+    flat[p] = cell;
+    if (calc_n_per_bin) atomicAdd(&n_per_bin[cell], 1);
+}
+
+// ---- boundaries from the sorted keys -----------------------------------------
+
+__global__ __launch_bounds__(256) void bin_boundaries_kernel(const int *__restrict__ sorted_bins, int n_vert,
+                                                             int *__restrict__ boundaries, int n_total_bins) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b > n_total_bins) return;
+    int lo = 0, hi = n_vert;  // first position whose key is >= b
+    while (lo < hi) {
+        int mid = (lo + hi) >> 1;
+        if (sorted_bins[mid] < b)
+            lo = mid + 1;
+        else
+            hi = mid;
+    }
+    boundaries[b] = lo;
+}
+
+template <int W>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint32_t *__restrict__ in, const int *__restrict__ rows,
+                                                          uint32_t *__restrict__ out, int n_rows, int width) {
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int w = W > 0 ? W : width;
+    if (t >= (long long)n_rows * w) return;
+    const int r = (int)(t / w), c = (int)(t - (long long)r * w);
+    out[t] = in[(size_t)rows[r] * w + c];
+}
+
+__global__ __launch_bounds__(256) void index_replacer_kernel(const int *__restrict__ tbr, const int *__restrict__ repl,
+                                                             int *__restrict__ out, int n, int n_repl) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int v = tbr[i];
+    if (v < 0)
+        out[i] = v;
+    else if (v < n_repl)
+        out[i] = repl[v];
+}
+
+int key_bits(int n_total_bins) {
+    int bits = 1;
+    while (bits < 31 && (1ll << bits) < (long long)n_total_bins) ++bits;
+    return bits;
+}
+
+}  // namespace
+
+int launch_fill_i32(int *p, int value, long long n, hipStream_t s) {
+    if (n <= 0) return HGC_OK;
+    int blocks = (int)std::min<long long>((n + 255) / 256, 4096);
+    fill_i32_kernel<<<blocks, 256, 0, s>>>(p, value, n);
+    return check_launch("fill_i32");
+}
+
+}  // namespace hgc
+
+using namespace hgc;
+
+extern "C" {
+
+int hgc_version(void) { return 100; }
+
+const char *hgc_last_error(void) { return hgc::last_error_buffer(); }
+
+int hgc_bin_by_coordinates_total_bins(const int *h_n_bins, int n_nbins, int n_rs, int *h_out_total_bins) {
+    HGC_REQUIRE(h_n_bins && h_out_total_bins, "null pointer");
+    HGC_REQUIRE(n_nbins >= 1 && n_rs >= 1, "need at least one dimension and one row split entry");
+    long long n = 1;
+    for (int i = 0; i < n_nbins; ++i) {
+        HGC_REQUIRE(h_n_bins[i] > 0, "n_bins[%d] = %d must be positive", i, h_n_bins[i]);
+        n *= h_n_bins[i];
+        HGC_REQUIRE(n < (1ll << 31), "bin count overflows int32");
+    }
+    n *= (n_rs - 1);
+    HGC_REQUIRE(n < (1ll << 31), "bin count overflows int32");
+    *h_out_total_bins = (int)n;
+    return HGC_OK;
+}
+
+int hgc_bin_by_coordinates_strided(const float *d_coords, int coord_stride, const float *d_shift,
+                                   const int *d_rs, const float *d_binswidth, const int *d_n_bins,
+                                   int *d_assigned_bin, int *d_flat_assigned_bin, int *d_n_per_bin,
+                                   int *d_n_out_of_range, int n_vert, int n_bin_dims, int n_rs,
+                                   int n_total_bins, int calc_n_per_bin, hgc_stream_t stream) {
+    HGC_REQUIRE(n_vert >= 0 && n_total_bins >= 0, "negative size");
+    HGC_REQUIRE(n_bin_dims >= 1 && n_bin_dims <= kMaxBinDims, "1 <= binning dimensions <= %d", kMaxBinDims);
+    HGC_REQUIRE(coord_stride >= n_bin_dims, "coordinate stride smaller than the binning dimensions");
+    HGC_REQUIRE(n_rs >= 2, "BinByCoordinatesOp expects at least two row splits entries");
+    HGC_REQUIRE(d_rs && d_binswidth && d_n_bins, "null pointer");
+    hipStream_t s = as_stream(stream);
+    if (d_n_per_bin) {
+        int rc = launch_fill_i32(d_n_per_bin, 0, n_total_bins, s);
+        if (rc) return rc;
+    }
+    if (n_vert == 0) return HGC_OK;
+    HGC_REQUIRE(d_coords && d_assigned_bin && d_flat_assigned_bin, "null pointer");
+    HGC_REQUIRE(!calc_n_per_bin || d_n_per_bin, "calc_n_per_bin needs d_n_per_bin");
+    bin_points_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, coord_stride, d_shift, d_rs, d_binswidth,
+                                                            d_n_bins, d_assigned_bin, d_flat_assigned_bin,
+                                                            d_n_per_bin, d_n_out_of_range, n_vert, n_bin_dims,
+                                                            n_rs, n_total_bins, calc_n_per_bin);
+    return check_launch("bin_points");
+}
+
+int hgc_bin_by_coordinates(const float *d_coords, const int *d_rs, const float *d_binswidth,
+                           const int *d_n_bins, int *d_assigned_bin, int *d_flat_assigned_bin,
+                           int *d_n_per_bin, int n_vert, int n_coords, int n_rs, int n_total_bins,
+                           int calc_n_per_bin, hgc_stream_t stream) {
+    return hgc_bin_by_coordinates_strided(d_coords, n_coords, nullptr, d_rs, d_binswidth, d_n_bins,
+                                          d_assigned_bin, d_flat_assigned_bin, d_n_per_bin, nullptr, n_vert,
+                                          n_coords, n_rs, n_total_bins, calc_n_per_bin, stream);
+}
+
+static int setup_blocks(int n_vert) { return std::max(1, std::min(1024, ceil_div(n_vert, 256 * 4))); }
+
+size_t hgc_bin_setup_workspace_bytes(int n_vert, int n_bin_dims) {
+    (void)n_bin_dims;
+    return align_up((size_t)setup_blocks(n_vert) * 2 * kMaxBinDims * sizeof(float));
+}
+
+int hgc_bin_setup(const float *d_coords, int coord_stride, int n_vert, int n_bin_dims, int pre_normalized,
+                  int n_bins_scalar, const float *d_bin_width_in, float *d_shift, float *d_bin_width,
+                  int *d_n_bins, void *workspace, size_t workspace_bytes, hgc_stream_t stream) {
+    HGC_REQUIRE(n_vert >= 1, "binning needs at least one point");
+    HGC_REQUIRE(n_bin_dims >= 1 && n_bin_dims <= kMaxBinDims, "1 <= binning dimensions <= %d", kMaxBinDims);
+    HGC_REQUIRE(coord_stride >= n_bin_dims, "coordinate stride smaller than the binning dimensions");
+    HGC_REQUIRE(d_coords && d_shift && d_bin_width && d_n_bins, "null pointer");
+    HGC_REQUIRE(n_bins_scalar > 0 || d_bin_width_in, "either n_bins or bin_width must be given");
+    if (!workspace || !aligned256(workspace) ||
+        workspace_bytes < hgc_bin_setup_workspace_bytes(n_vert, n_bin_dims))
+        return fail(HGC_ERR_WORKSPACE, "bin_setup workspace missing, misaligned or too small");
+    hipStream_t s = as_stream(stream);
+    const int blocks = setup_blocks(n_vert);
+    float *partial = static_cast<float *>(workspace);
+    column_minmax_kernel<<<blocks, 256, 0, s>>>(d_coords, coord_stride, n_vert, n_bin_dims, partial);
+    int rc = check_launch("column_minmax");
+    if (rc) return rc;
+    grid_params_kernel<<<1, 64, 0, s>>>(partial, blocks, n_bin_dims, pre_normalized, n_bins_scalar, d_bin_width_in,
+                                        d_shift, d_bin_width, d_n_bins);
+    return check_launch("grid_params");
+}
+
+size_t hgc_sort_by_bin_workspace_bytes(int n_vert, int n_total_bins) {
+    size_t temp = 0;
+    const int n = std::max(n_vert, 1);
+    (void)rocprim::radix_sort_pairs(nullptr, temp, (const unsigned int *)nullptr, (unsigned int *)nullptr,
+                                    (const int *)nullptr, (int *)nullptr, (size_t)n, 0,
+                                    key_bits(std::max(n_total_bins, 2)), (hipStream_t) nullptr);
+    return align_up(temp) + 2 * align_up((size_t)n * sizeof(int));
+}
+
+int hgc_sort_by_bin(const int *d_flat_bin, int n_vert, int n_total_bins, int *d_sorting,
+                    int *d_bin_boundaries, void *workspace, size_t workspace_bytes, hgc_stream_t stream) {
+    HGC_REQUIRE(n_vert >= 0 && n_total_bins >= 1, "bad sizes");
+    HGC_REQUIRE(d_bin_boundaries, "null pointer");
+    hipStream_t s = as_stream(stream);
+    if (n_vert == 0) return launch_fill_i32(d_bin_boundaries, 0, (long long)n_total_bins + 1, s);
+    HGC_REQUIRE(d_flat_bin && d_sorting, "null pointer");
+    if (!workspace || !aligned256(workspace) ||
+        workspace_bytes < hgc_sort_by_bin_workspace_bytes(n_vert, n_total_bins))
+        return fail(HGC_ERR_WORKSPACE, "sort_by_bin workspace missing, misaligned or too small");
+    Carver carve(workspace);
+    int *iota = carve.take<int>(n_vert);
+    unsigned int *keys_out = carve.take<unsigned int>(n_vert);
+    void *temp = carve.base + carve.used;
+    size_t temp_bytes = workspace_bytes - carve.used;
+    iota_i32_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(iota, n_vert);
+    int rc = check_launch("iota");
+    if (rc) return rc;
+    // LSD radix sort: stable, so equal bins keep ascending original index
+    HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, reinterpret_cast<const unsigned int *>(d_flat_bin),
+                                      keys_out, iota, d_sorting, (size_t)n_vert, 0, key_bits(n_total_bins), s));
+    bin_boundaries_kernel<<<ceil_div((long long)n_total_bins + 1, 256), 256, 0, s>>>(
+        reinterpret_cast<const int *>(keys_out), n_vert, d_bin_boundaries, n_total_bins);
+    return check_launch("bin_boundaries");
+}
+
+int hgc_gather_rows(const void *d_in, const int *d_rows, void *d_out, int n_rows, int width,
+                    hgc_stream_t stream) {
+    HGC_REQUIRE(n_rows >= 0 && width >= 1, "bad sizes");
+    if (n_rows == 0) return HGC_OK;
+    HGC_REQUIRE(d_in && d_rows && d_out, "null pointer");
+    hipStream_t s = as_stream(stream);
+    const long long total = (long long)n_rows * width;
+    const int blocks = ceil_div(total, 256);
+    const uint32_t *in = static_cast<const uint32_t *>(d_in);
+    uint32_t *out = static_cast<uint32_t *>(d_out);
+    switch (width) {
+        case 1: gather_rows_kernel<1><<<blocks, 256, 0, s>>>(in, d_rows, out, n_rows, width); break;
+        case 2: gather_rows_kernel<2><<<blocks, 256, 0, s>>>(in, d_rows, out, n_rows, width); break;
+        case 3: gather_rows_kernel<3><<<blocks, 256, 0, s>>>(in, d_rows, out, n_rows, width); break;
+        case 4: gather_rows_kernel<4><<<blocks, 256, 0, s>>>(in, d_rows, out, n_rows, width); break;
+        default: gather_rows_kernel<0><<<blocks, 256, 0, s>>>(in, d_rows, out, n_rows, width); break;
+    }
+    return check_launch("gather_rows");
+}
+
+int hgc_index_replacer(const int *d_to_be_replaced, const int *d_replacements, int *d_replaced,
+                       int n_to_be_replaced, int n_replacements, hgc_stream_t stream) {
+    HGC_REQUIRE(n_to_be_replaced >= 0 && n_replacements >= 0, "negative size");
+    if (n_to_be_replaced == 0) return HGC_OK;
+    HGC_REQUIRE(d_to_be_replaced && d_replaced && (d_replacements || n_replacements == 0), "null pointer");
+    index_replacer_kernel<<<ceil_div(n_to_be_replaced, 256), 256, 0, as_stream(stream)>>>(
+        d_to_be_replaced, d_replacements, d_replaced, n_to_be_replaced, n_replacements);
+    return check_launch("index_replacer");
+}
+
+}  // extern "C"

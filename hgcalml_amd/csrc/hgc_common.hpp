@@ -1,0 +1,119 @@
+// Shared host/device helpers of the gfx950 kernels (wave64 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "hgcalml_amd.h"
+
+namespace hgc {
+
+constexpr int kWave = 64;
+constexpr int kNumXcd = 8;  // MI355X: 8 accelerator complex dies, one L2 each
+
+// ---- error plumbing -------------------------------------------------------
+
+char *last_error_buffer();  // thread local, 512 bytes
+
+inline int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(last_error_buffer(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HGC_REQUIRE(cond, ...)                                         \
+    do {                                                               \
+        if (!(cond)) return ::hgc::fail(HGC_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+    } while (0)
+
+#define HGC_HIP(expr)                                                              \
+    do {                                                                           \
+        hipError_t e_ = (expr);                                                    \
+        if (e_ != hipSuccess)                                                      \
+            return ::hgc::fail(HGC_ERR_LAUNCH, "%s: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+inline int check_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HGC_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+    return HGC_OK;
+}
+
+inline hipStream_t as_stream(hgc_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+
+inline bool aligned256(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 255u) == 0; }
+
+// Carves 256-byte aligned pieces out of a caller supplied workspace.
+struct Carver {
+    char *base;
+    size_t used = 0;
+    explicit Carver(void *p) : base(static_cast<char *>(p)) {}
+    template <typename T>
+    T *take(size_t count) {
+        T *p = reinterpret_cast<T *>(base + used);
+        used += align_up(count * sizeof(T));
+        return p;
+    }
+};
+
+// ---- device helpers -------------------------------------------------------
+
+#ifdef __HIPCC__
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// Consecutive workgroups are dealt round-robin to the 8 XCDs. This maps the
+// hardware block index to a logical tile index such that each XCD works on one
+// contiguous range of tiles (neighbouring tiles then share that XCD's L2).
+__device__ __forceinline__ int xcd_contiguous_block(int bid, int nblocks) {
+    const int per = nblocks / kNumXcd;
+    const int body = per * kNumXcd;
+    if (bid >= body) return bid;  // ragged tail keeps its index
+    return (bid % kNumXcd) * per + bid / kNumXcd;
+}
+
+__device__ __forceinline__ int readlane_i32(int v, int lane) {
+    return __builtin_amdgcn_readlane(v, lane);
+}
+
+__device__ __forceinline__ uint64_t readlane_u64(uint64_t v, int lane) {
+    uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)v, lane);
+    uint32_t hi = __builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), lane);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// lane i receives v from lane i-1; lane 0 receives `into_lane0`
+__device__ __forceinline__ uint32_t wave_shift_up1(uint32_t v, uint32_t into_lane0) {
+    // DPP wave_shr:1 (0x138): whole-wave shift right by one lane; lanes without
+    // a source keep the first operand.
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)into_lane0, (int)v, 0x138, 0xf, 0xf, false);
+}
+
+__device__ __forceinline__ uint64_t wave_shift_up1_u64(uint64_t v, uint64_t into_lane0) {
+    uint32_t lo = wave_shift_up1((uint32_t)v, (uint32_t)into_lane0);
+    uint32_t hi = wave_shift_up1((uint32_t)(v >> 32), (uint32_t)(into_lane0 >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// inclusive prefix sum over the 64 lanes
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        int t = __shfl_up(v, off, kWave);
+        if (lane_id() >= off) v += t;
+    }
+    return v;
+}
+
+#endif  // __HIPCC__
+
+}  // namespace hgc

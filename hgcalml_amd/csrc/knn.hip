@@ -1,0 +1,370 @@
+// Exact binned k-nearest-neighbour search, one wave64 per query point.
+//
+// Reference behaviour restated here:
+//   modules/compiled/binned_select_knn_kernel.cc:19-196 (search, defaults, stop rule)
+//   modules/compiled/binstepper.h:11-97                 (shell of bins at distance d)
+//   modules/binned_select_knn_op.py:92-95               (un-sort, fused when a sorting is given)
+//   modules/compiled/select_knn_kernel.cc:158,244-245   (radius rule)
+//
+// Design (gfx950, wave64):
+//   * Points arrive sorted by bin, so the bins of one row of the grid (last
+//     binned dimension running) are one contiguous range of points. A shell of
+//     half-width d is cut into such ranges ("segments"); the 64 lanes look up 64
+//     segments at once, prefix-sum their lengths, and the wave then walks the
+//     concatenated candidate list 64 points per step, fully coalesced.
+//   * Each lane evaluates one candidate: serial fp32 sum of squared coordinate
+//     differences in coordinate order (no FMA contraction), packed with the
+//     candidate's index into a 64-bit key (distance bits high, index low), so a
+//     single unsigned compare orders by (distance, index).
+//   * The K-1 best keys live in registers, sorted across the lanes (rank r in
+//     lane r%64, register r/64). A ballot finds the candidates that beat the
+//     current K-th key; each is inserted with one DPP wave shift and two
+//     compares, and the new K-th key is read back with a readlane.
+//   * The shell loop stops exactly as the reference does: list full and
+//     ((bw*d)*bw)*d > K-th distance, or no bin of the shell inside the grid.
+//   * No LDS, no atomics, no barriers; every wave exits on its own.
+#include "hgc_common.hpp"
+
+namespace hgc {
+namespace {
+
+constexpr int kMaxBinDims = 5;
+constexpr uint64_t kEmptyKey = ~0ull;
+
+struct KnnParams {
+    const float *coord;
+    const int *bin_idx;
+    const int *direction;
+    const int *dim_bin_idx;
+    const int *bin_boundaries;
+    const int *n_bins;
+    const float *bin_width;
+    const int *sorting;  // may be null
+    int *out_idx;
+    float *out_dist;
+    float radius_sq;  // < 0: no radius
+    int n_vert, K, n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction;
+};
+
+template <int C>
+__device__ __forceinline__ float dist_sq(const float (&q)[C > 0 ? C : 1], const float *__restrict__ coord, int j,
+                                         int n_coords, const float *__restrict__ qrow) {
+    float acc = 0.f;
+    if constexpr (C > 0) {
+        const float *r = coord + (size_t)j * C;
+        float x[C];
+        if constexpr (C == 4) {
+            const float4 v = *reinterpret_cast<const float4 *>(r);
+            x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+        } else if constexpr (C == 2) {
+            const float2 v = *reinterpret_cast<const float2 *>(r);
+            x[0] = v.x; x[1] = v.y;
+        } else {
+#pragma unroll
+            for (int c = 0; c < C; ++c) x[c] = r[c];
+        }
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const float d = q[c] - x[c];
+            acc = acc + d * d;
+        }
+    } else {
+        const float *r = coord + (size_t)j * n_coords;
+        for (int c = 0; c < n_coords; ++c) {
+            const float d = qrow[c] - r[c];
+            acc = acc + d * d;
+        }
+    }
+    return acc;
+}
+
+// insert key c (known to be smaller than the current last key of the list)
+template <int S>
+__device__ __forceinline__ void sorted_insert(uint64_t (&key)[S], uint64_t c) {
+    uint64_t carry = 0;  // what enters lane 0 of the next register level
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const uint64_t old = key[s];
+        const uint64_t last = readlane_u64(old, kWave - 1);
+        if (c < last) {  // wave-uniform: the insertion point is in or before this level
+            const uint64_t prev = wave_shift_up1_u64(old, carry);
+            key[s] = (c < prev) ? prev : ((c < old) ? c : old);
+        }
+        carry = last;
+    }
+}
+
+template <int C, int S, bool MAPPED>
+__global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
+    const int lane = lane_id();
+    const int tile = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    const int q = tile * 4 + (threadIdx.x >> 6);  // one query per wave
+    if (q >= p.n_vert) return;
+
+    const int K = p.K;
+    const int Kn = K - 1;  // neighbours besides the point itself
+    const int self_id = MAPPED ? p.sorting[q] : q;
+    const size_t out_row = (size_t)self_id * K;
+    const int pad_idx = p.tf_compat ? self_id : -1;
+
+    bool searching = Kn > 0;
+    if (p.use_direction) {
+        const int dq = p.direction[q];
+        if (dq == 0 || dq == 2) searching = false;  // may not have neighbours
+    }
+
+    uint64_t key[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) key[s] = kEmptyKey;
+
+    if (searching) {
+        // query coordinates (wave-uniform)
+        float qc[C > 0 ? C : 1];
+        const float *qrow = p.coord + (size_t)q * p.n_coords;
+        if constexpr (C > 0) {
+#pragma unroll
+            for (int c = 0; c < C; ++c) qc[c] = qrow[c];
+        }
+
+        const int B = p.n_bin_dim;
+        int nb[kMaxBinDims], qb[kMaxBinDims];
+        int cells_per_event = 1;
+        int reach_max = 0;  // beyond this shell distance no bin is inside the grid
+#pragma unroll
+        for (int i = 0; i < kMaxBinDims; ++i) {
+            nb[i] = 1;
+            qb[i] = 0;
+            if (i < B) {
+                nb[i] = p.n_bins[i];
+                qb[i] = p.dim_bin_idx[(size_t)q * (B + 1) + 1 + i];
+                cells_per_event *= nb[i];
+                reach_max = max(reach_max, max(qb[i], nb[i] - 1 - qb[i]));
+            }
+        }
+        const int event_base = cells_per_event * (p.bin_idx[q] / cells_per_event);
+        const int nb_last = nb[B - 1], qb_last = qb[B - 1];
+        const float bw = p.bin_width[0];
+
+        // keys at or above `limit` can never enter: the radius cut, if any
+        const bool has_radius = p.radius_sq >= 0.f;
+        const uint64_t limit = has_radius ? ((uint64_t)(__float_as_uint(p.radius_sq) + 1u) << 32) : kEmptyKey;
+        const int kth_lane = (Kn - 1) & (kWave - 1);
+        const int kth_level = (Kn - 1) >> 6;
+        uint64_t thr = limit;  // min(limit, current K-th key)
+
+        for (int d = 0; d <= reach_max; ++d) {
+            const int W = 2 * d + 1;
+            int n_rows = 1;
+            for (int i = 0; i < B - 1; ++i) n_rows *= W;
+            const int n_slots = d == 0 ? 1 : 2 * n_rows;
+
+            for (int slot0 = 0; slot0 < n_slots; slot0 += kWave) {
+                // ---- each lane resolves one segment of the shell ----
+                int seg_start = 0, seg_len = 0;
+                const int slot = slot0 + lane;
+                if (slot < n_slots) {
+                    int row = slot >> 1;
+                    const int second = slot & 1;
+                    bool inside = true, on_face = false;
+                    int off[kMaxBinDims];
+#pragma unroll
+                    for (int i = kMaxBinDims - 2; i >= 0; --i) {
+                        off[i] = 0;
+                        if (i < B - 1) {
+                            const int digit = row % W;
+                            row /= W;
+                            off[i] = digit - d;
+                        }
+                    }
+                    int cell = 0;
+#pragma unroll
+                    for (int i = 0; i < kMaxBinDims - 1; ++i) {
+                        if (i < B - 1) {
+                            const int k = qb[i] + off[i];
+                            inside = inside && k >= 0 && k < nb[i];
+                            on_face = on_face || off[i] == d || off[i] == -d;
+                            cell = cell * nb[i] + k;
+                        }
+                    }
+                    int lo, hi;
+                    if (on_face || d == 0) {  // the whole run of the last dimension
+                        lo = qb_last - d;
+                        hi = second ? lo - 1 : qb_last + d;
+                    } else {  // interior row: only the two end caps
+                        lo = second ? qb_last + d : qb_last - d;
+                        hi = lo;
+                        if (lo < 0 || lo >= nb_last) hi = lo - 1;
+                    }
+                    lo = max(lo, 0);
+                    hi = min(hi, nb_last - 1);
+                    if (inside && lo <= hi) {
+                        const int first = event_base + cell * nb_last + lo;
+                        const int last = event_base + cell * nb_last + hi + 1;
+                        if (last < p.n_bboundaries) {
+                            seg_start = p.bin_boundaries[first];
+                            seg_len = p.bin_boundaries[last] - seg_start;
+                        }
+                    }
+                }
+                const int seg_end_off = wave_inclusive_sum(seg_len);
+                const int seg_off = seg_end_off - seg_len;
+                const int total = readlane_i32(seg_end_off, kWave - 1);
+
+                // ---- walk the concatenated candidates, 64 per step ----
+                for (int t = 0; t < total; t += kWave) {
+                    const int c = t + lane;
+                    // last segment whose offset is <= c (empty ones share the
+                    // offset of their successor, so the last one is the owner)
+                    int s_lo = 0;
+#pragma unroll
+                    for (int step = 32; step > 0; step >>= 1) {
+                        const int probe = s_lo + step;
+                        const int o = __shfl(seg_off, probe, kWave);
+                        if (o <= c) s_lo = probe;
+                    }
+                    const int j = __shfl(seg_start, s_lo, kWave) + (c - __shfl(seg_off, s_lo, kWave));
+                    bool valid = c < total && j != q;
+                    const int jj = valid ? j : q;
+                    if (p.use_direction && valid) {
+                        const int dj = p.direction[jj];
+                        if (dj == 1 || dj == 2) valid = false;  // may not be a neighbour
+                    }
+                    const float dsq = dist_sq<C>(qc, p.coord, jj, p.n_coords, qrow);
+                    const uint32_t id = MAPPED ? (uint32_t)p.sorting[jj] : (uint32_t)jj;
+                    const uint64_t ck = ((uint64_t)__float_as_uint(dsq) << 32) | id;
+                    uint64_t beats = __ballot(valid && ck < thr);
+                    while (beats) {
+                        const int src = __ffsll((long long)beats) - 1;
+                        beats &= beats - 1;
+                        const uint64_t cand = readlane_u64(ck, src);
+                        if (cand < thr) {
+                            sorted_insert<S>(key, cand);
+                            uint64_t kth = kEmptyKey;
+#pragma unroll
+                            for (int s = 0; s < S; ++s)
+                                if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
+                            thr = kth < limit ? kth : limit;
+                        }
+                    }
+                }
+            }
+
+            // stop rule (fp32, evaluated left to right)
+            float reach = bw * (float)d;
+            reach = reach * bw;
+            reach = reach * (float)d;
+            uint64_t kth = kEmptyKey;
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+                if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
+            if (kth != kEmptyKey && reach > __uint_as_float((uint32_t)(kth >> 32))) break;
+            if (has_radius && reach > p.radius_sq) break;
+        }
+    }
+
+    // ---- write the row: slot 0 = self, then ascending (distance, index) ----
+    if (lane == 0) {
+        p.out_idx[out_row] = self_id;
+        p.out_dist[out_row] = 0.f;
+    }
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const int rank = s * kWave + lane;
+        if (rank < Kn) {
+            const bool filled = key[s] != kEmptyKey;
+            p.out_idx[out_row + 1 + rank] = filled ? (int)(uint32_t)key[s] : pad_idx;
+            p.out_dist[out_row + 1 + rank] = filled ? __uint_as_float((uint32_t)(key[s] >> 32)) : 0.f;
+        }
+    }
+}
+
+template <int C, bool MAPPED>
+int launch_levels(const KnnParams &p, hipStream_t s) {
+    const int levels = std::max(1, ceil_div(p.K - 1, kWave));
+    const dim3 grid(ceil_div(p.n_vert, 4)), block(256);
+    switch (levels) {
+        case 1: knn_wave_kernel<C, 1, MAPPED><<<grid, block, 0, s>>>(p); break;
+        case 2: knn_wave_kernel<C, 2, MAPPED><<<grid, block, 0, s>>>(p); break;
+        case 3:
+        case 4: knn_wave_kernel<C, 4, MAPPED><<<grid, block, 0, s>>>(p); break;
+        default: knn_wave_kernel<C, 8, MAPPED><<<grid, block, 0, s>>>(p); break;
+    }
+    return check_launch("knn_wave_kernel");
+}
+
+template <bool MAPPED>
+int launch_coords(const KnnParams &p, hipStream_t s) {
+    switch (p.n_coords) {
+        case 2: return launch_levels<2, MAPPED>(p, s);
+        case 3: return launch_levels<3, MAPPED>(p, s);
+        case 4: return launch_levels<4, MAPPED>(p, s);
+        default: return launch_levels<0, MAPPED>(p, s);
+    }
+}
+
+}  // namespace
+}  // namespace hgc
+
+using namespace hgc;
+
+extern "C" {
+
+int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, const int *d_direction,
+                                const int *d_dim_bin_idx, const int *d_bin_boundaries,
+                                const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
+                                float max_radius, int *d_indices, float *d_dist, int n_vert, int n_neigh,
+                                int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
+                                int use_direction, hgc_stream_t stream) {
+    // same conditions as the reference op (binned_select_knn_kernel.cc:336-352)
+    HGC_REQUIRE(n_bin_dim > 1, "BinnedSelectKnnOp expects at least 2 binning dimensions.");
+    HGC_REQUIRE(n_bin_dim < 6, "BinnedSelectKnnOp expects maximum 5 binning dimensions.");
+    HGC_REQUIRE(n_coords > 1, "BinnedSelectKnnOp expects at least 2 dimensions.");
+    HGC_REQUIRE(n_coords >= n_bin_dim, "fewer coordinates than binning dimensions");
+    HGC_REQUIRE(n_vert >= 0, "negative number of points");
+    HGC_REQUIRE(n_neigh >= 1 && n_neigh <= 8 * kWave + 1, "1 <= n_neighbours <= %d", 8 * kWave + 1);
+    HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neighbours overflows int32");
+    HGC_REQUIRE(n_bboundaries >= 2, "bin boundary table too short");
+    if (n_vert == 0) return HGC_OK;
+    HGC_REQUIRE(d_coord && d_bin_idx && d_dim_bin_idx && d_bin_boundaries && d_n_bins && d_bin_width &&
+                    d_indices && d_dist,
+                "null pointer");
+    HGC_REQUIRE(!use_direction || d_direction,
+                "BinnedSelectKnnOp needs a direction tensor (0,1,2,other) with length nvert if use_direction=True.");
+    HGC_REQUIRE((n_coords != 4 && n_coords != 2) || (reinterpret_cast<uintptr_t>(d_coord) & 15u) == 0,
+                "coordinate matrix must be 16-byte aligned");
+
+    KnnParams p;
+    p.coord = d_coord;
+    p.bin_idx = d_bin_idx;
+    p.direction = d_direction;
+    p.dim_bin_idx = d_dim_bin_idx;
+    p.bin_boundaries = d_bin_boundaries;
+    p.n_bins = d_n_bins;
+    p.bin_width = d_bin_width;
+    p.sorting = d_sorting;
+    p.out_idx = d_indices;
+    p.out_dist = d_dist;
+    p.radius_sq = max_radius > 0.f ? max_radius * max_radius : -1.f;
+    p.n_vert = n_vert;
+    p.K = n_neigh;
+    p.n_coords = n_coords;
+    p.n_bin_dim = n_bin_dim;
+    p.n_bboundaries = n_bboundaries;
+    p.tf_compat = tf_compat;
+    p.use_direction = use_direction;
+    hipStream_t s = as_stream(stream);
+    return d_sorting ? launch_coords<true>(p, s) : launch_coords<false>(p, s);
+}
+
+int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int *d_direction,
+                          const int *d_dim_bin_idx, const int *d_bin_boundaries, const int *d_n_bins,
+                          const float *d_bin_width, int *d_indices, float *d_dist, int n_vert, int n_neigh,
+                          int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat, int use_direction,
+                          hgc_stream_t stream) {
+    return hgc_binned_select_knn_fused(d_coord, d_bin_idx, d_direction, d_dim_bin_idx, d_bin_boundaries,
+                                       d_n_bins, d_bin_width, nullptr, -1.f, d_indices, d_dist, n_vert,
+                                       n_neigh, n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction,
+                                       stream);
+}
+
+}  // extern "C"

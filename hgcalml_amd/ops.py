@@ -1,0 +1,264 @@
+"""Tensor-level entry points of the HIP kernels, registered as PyTorch custom
+ops in the ``hgcalml`` namespace (``torch.ops.hgcalml.*``).
+
+Inputs/outputs follow the reference's REGISTER_OP blocks
+(modules/compiled/*_module.cc): same order, same dtypes. All tensors live on
+the GPU; the work is enqueued on torch's current HIP stream.
+"""
+import weakref
+
+import torch
+
+from . import _lib
+from ._lib import check, f32, i32, lib, p, require_device, stream, workspace
+
+
+# --------------------------------------------------------------------------- binning
+
+@torch.library.custom_op("hgcalml::bin_by_coordinates", mutates_args=())
+def bin_by_coordinates(coordinates: torch.Tensor, row_splits: torch.Tensor, bin_width: torch.Tensor,
+                       nbins: torch.Tensor, n_total_bins: int,
+                       calc_n_per_bin: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """modules/compiled/bin_by_coordinates_module.cc:7-15 (n_total_bins is passed
+    by the caller instead of being copied back from the device)."""
+    dev = require_device(coordinates, row_splits, bin_width, nbins)
+    coordinates, row_splits, bin_width, nbins = f32(coordinates), i32(row_splits), f32(bin_width), i32(nbins)
+    if coordinates.dim() != 2 or row_splits.dim() != 1 or row_splits.numel() < 2:
+        raise ValueError("BinByCoordinatesOp expects coordinates [N,C] and row splits [R+1]")
+    n, c = coordinates.shape
+    if nbins.numel() != c or bin_width.numel() != 1:
+        raise ValueError("BinByCoordinatesOp expects n_bins [C] and a singleton bin width")
+    binass = torch.zeros((n, c + 1), dtype=torch.int32, device=dev)
+    flat = torch.zeros((n,), dtype=torch.int32, device=dev)
+    nper = torch.empty((n_total_bins,), dtype=torch.int32, device=dev)
+    check(lib.hgc_bin_by_coordinates(p(coordinates), p(row_splits), p(bin_width), p(nbins), p(binass), p(flat),
+                                     p(nper), n, c, row_splits.numel(), n_total_bins, int(calc_n_per_bin), stream()))
+    return binass, flat, nper
+
+
+def bin_setup(coords, n_bin_dims, pre_normalized, n_bins=None, bin_width=None):
+    """grid parameters on the device: (shift [B], bin_width [1], n_bins [B])"""
+    dev = require_device(coords, bin_width)
+    n, c = coords.shape
+    shift = torch.empty((n_bin_dims,), dtype=torch.float32, device=dev)
+    bw = torch.empty((1,), dtype=torch.float32, device=dev)
+    nb = torch.empty((n_bin_dims,), dtype=torch.int32, device=dev)
+    ws = workspace(lib.hgc_bin_setup_workspace_bytes(n, n_bin_dims), dev)
+    bw_in = None if bin_width is None else f32(bin_width).reshape(1)
+    check(lib.hgc_bin_setup(p(coords), c, n, n_bin_dims, int(pre_normalized), int(n_bins) if n_bins is not None else 0,
+                            p(bw_in), p(shift), p(bw), p(nb), p(ws), ws.numel(), stream()))
+    return shift, bw, nb
+
+
+def bin_points(coords, n_bin_dims, shift, row_splits, bin_width, nbins, n_total_bins, calc_n_per_bin):
+    """strided binning kernel: bins the first n_bin_dims columns of coords"""
+    dev = require_device(coords)
+    n, c = coords.shape
+    binass = torch.zeros((n, n_bin_dims + 1), dtype=torch.int32, device=dev)
+    flat = torch.zeros((n,), dtype=torch.int32, device=dev)
+    nper = torch.empty((n_total_bins,), dtype=torch.int32, device=dev) if calc_n_per_bin else None
+    check(lib.hgc_bin_by_coordinates_strided(p(coords), c, p(shift), p(row_splits), p(bin_width), p(nbins), p(binass),
+                                             p(flat), p(nper), None, n, n_bin_dims, row_splits.numel(), n_total_bins,
+                                             int(calc_n_per_bin), stream()))
+    return binass, flat, nper
+
+
+def sort_by_bin(flat_bin, n_total_bins):
+    """(sorting [N], bin_boundaries [T+1]) — stable"""
+    dev = require_device(flat_bin)
+    n = flat_bin.numel()
+    sorting = torch.empty((n,), dtype=torch.int32, device=dev)
+    bounds = torch.empty((n_total_bins + 1,), dtype=torch.int32, device=dev)
+    ws = workspace(lib.hgc_sort_by_bin_workspace_bytes(n, n_total_bins), dev)
+    check(lib.hgc_sort_by_bin(p(flat_bin), n, n_total_bins, p(sorting), p(bounds), p(ws), ws.numel(), stream()))
+    return sorting, bounds
+
+
+def gather_rows(t, rows):
+    """t[rows] for 4-byte element tensors of shape [N] or [N, W]"""
+    require_device(t, rows)
+    assert t.element_size() == 4 and t.is_contiguous()
+    width = 1 if t.dim() == 1 else t.shape[1]
+    out = torch.empty((rows.numel(),) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+    check(lib.hgc_gather_rows(p(t), p(rows), p(out), rows.numel(), width, stream()))
+    return out
+
+
+# --------------------------------------------------------------------------- kNN
+
+def _knn_checks(coords, bin_idx, dim_bin_idx, n_bins, bin_width, direction, use_direction):
+    # modules/compiled/binned_select_knn_kernel.cc:336-352
+    n_bin_dims = n_bins.numel()
+    if not 1 < n_bin_dims < 6:
+        raise ValueError("BinnedSelectKnnOp expects between 2 and 5 binning dimensions.")
+    if dim_bin_idx.shape[1] - 1 != n_bin_dims:
+        raise ValueError("BinnedSelectKnnOp expects number of bin dimensions (including row splits) -1 == "
+                         "number of total bin dimensions.")
+    if coords.shape[1] < 2:
+        raise ValueError("BinnedSelectKnnOp expects at least 2 dimensions.")
+    if coords.shape[0] != bin_idx.shape[0]:
+        raise ValueError("BinnedSelectKnnOp expects same first dimension for bin idx and coordinates.")
+    if bin_width.numel() != 1:
+        raise ValueError("BinnedSelectKnnOp expects singleton (dim(1)) for bin width.")
+    if use_direction and direction.shape[0] != coords.shape[0]:
+        raise ValueError("BinnedSelectKnnOp needs a direction tensor (0,1,2,other) with length nvert "
+                         "if use_direction=True.")
+
+
+@torch.library.custom_op("hgcalml::binned_select_knn", mutates_args=())
+def binned_select_knn(coords: torch.Tensor, bin_idx: torch.Tensor, dim_bin_idx: torch.Tensor,
+                      bin_boundaries: torch.Tensor, n_bins: torch.Tensor, bin_width: torch.Tensor,
+                      direction: torch.Tensor, n_neighbours: int, tf_compatible: bool,
+                      use_direction: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    """modules/compiled/binned_select_knn_module.cc:8-20; inputs in bin-sorted order,
+    outputs in the same (sorted) index space."""
+    return binned_select_knn_fused(coords, bin_idx, dim_bin_idx, bin_boundaries, n_bins, bin_width, direction,
+                                   None, -1.0, n_neighbours, tf_compatible, use_direction)
+
+
+def binned_select_knn_fused(coords, bin_idx, dim_bin_idx, bin_boundaries, n_bins, bin_width, direction, sorting,
+                            max_radius, n_neighbours, tf_compatible, use_direction):
+    dev = require_device(coords, bin_idx, dim_bin_idx, bin_boundaries, n_bins, bin_width, sorting)
+    coords, bin_idx, dim_bin_idx = f32(coords), i32(bin_idx), i32(dim_bin_idx)
+    bin_boundaries, n_bins, bin_width = i32(bin_boundaries), i32(n_bins), f32(bin_width)
+    direction = i32(direction) if use_direction else None
+    _knn_checks(coords, bin_idx, dim_bin_idx, n_bins, bin_width, direction, use_direction)
+    n, c = coords.shape
+    idx = torch.empty((n, n_neighbours), dtype=torch.int32, device=dev)
+    dist = torch.empty((n, n_neighbours), dtype=torch.float32, device=dev)
+    check(lib.hgc_binned_select_knn_fused(p(coords), p(bin_idx), p(direction), p(dim_bin_idx), p(bin_boundaries),
+                                          p(n_bins), p(bin_width), p(sorting),
+                                          float(max_radius) if max_radius is not None else -1.0, p(idx), p(dist), n,
+                                          int(n_neighbours), c, n_bins.numel(), bin_boundaries.numel(),
+                                          int(tf_compatible), int(use_direction), stream()))
+    return idx, dist
+
+
+@torch.library.custom_op("hgcalml::index_replacer", mutates_args=())
+def index_replacer(to_be_replaced: torch.Tensor, replacements: torch.Tensor) -> torch.Tensor:
+    """modules/compiled/index_replacer_module.cc:7-10"""
+    require_device(to_be_replaced, replacements)
+    tbr, rep = i32(to_be_replaced), i32(replacements)
+    out = torch.zeros_like(tbr)
+    check(lib.hgc_index_replacer(p(tbr), p(rep), p(out), tbr.numel(), rep.numel(), stream()))
+    return out
+
+
+# --------------------------------------------------------------------------- accumulate
+
+@torch.library.custom_op("hgcalml::accumulate_knn", mutates_args=())
+def accumulate_knn(distances: torch.Tensor, features: torch.Tensor, indices: torch.Tensor, n_moments: int,
+                   mean_and_max: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    """modules/compiled/accumulate_knn_module.cc:7-14 (`distances` are the weights)"""
+    dev = require_device(distances, features, indices)
+    w, x, idx = f32(distances), f32(features), i32(indices)
+    # modules/compiled/accumulate_knn_kernel.cc:107-111
+    if w.dim() != 2 or x.dim() != 2 or idx.dim() != 2:
+        raise ValueError("AccumulateKnnOp expects rank 2 tensors")
+    if idx.shape != w.shape or x.shape[0] != idx.shape[0]:
+        raise ValueError("AccumulateKnnOp expects first dimensions of all inputs to match, and indices and "
+                         "distances to have the same shape")
+    n, k = idx.shape
+    f = x.shape[1]
+    out = torch.empty((n, 2 * f if mean_and_max else f), dtype=torch.float32, device=dev)
+    maxidx = torch.empty((n, f), dtype=torch.int32, device=dev) if mean_and_max else \
+        torch.zeros((n, f), dtype=torch.int32, device=dev)
+    check(lib.hgc_accumulate_knn(p(w), p(x), p(idx), p(out), p(maxidx), n, k, f, out.shape[1], int(n_moments),
+                                 int(mean_and_max), stream()))
+    return out, maxidx
+
+
+def inverse_neighbour_index(indices):
+    """(offsets [N+1], slots [N*K]): who names each vertex, ascending (vertex, slot)"""
+    dev = require_device(indices)
+    idx = i32(indices)
+    n, k = idx.shape
+    offsets = torch.empty((n + 1,), dtype=torch.int32, device=dev)
+    slots = torch.empty((max(n * k, 1),), dtype=torch.int32, device=dev)
+    ws = workspace(lib.hgc_inverse_neighbour_index_workspace_bytes(n, k), dev)
+    check(lib.hgc_inverse_neighbour_index(p(idx), n, k, p(offsets), p(slots), p(ws), ws.numel(), stream()))
+    return offsets, slots
+
+
+_INVERSE_CACHE = {}
+
+
+def cached_inverse_neighbour_index(indices):
+    """The inverse index depends only on the neighbour table; GravNet-style
+    models run several accumulations (and their gradients) over one table, so
+    it is built once per tensor object and version."""
+    key = id(indices)
+    hit = _INVERSE_CACHE.get(key)
+    if hit is not None:
+        ref, version, ptr, value = hit
+        if ref() is indices and version == indices._version and ptr == indices.data_ptr():
+            return value
+    value = inverse_neighbour_index(indices)
+    if len(_INVERSE_CACHE) > 64:
+        for k in [k for k, v in _INVERSE_CACHE.items() if v[0]() is None]:
+            del _INVERSE_CACHE[k]
+        if len(_INVERSE_CACHE) > 64:
+            _INVERSE_CACHE.clear()
+    _INVERSE_CACHE[key] = (weakref.ref(indices), indices._version, indices.data_ptr(), value)
+    return value
+
+
+@torch.library.custom_op("hgcalml::accumulate_knn_grad", mutates_args=())
+def accumulate_knn_grad(grad_from_out_features: torch.Tensor, distances: torch.Tensor, features: torch.Tensor,
+                        neigh_indices: torch.Tensor, max_feat_indices: torch.Tensor, inv_offsets: torch.Tensor,
+                        inv_slots: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """modules/compiled/accumulate_knn_grad_module.cc:7-14 plus the inverse
+    neighbour index of `neigh_indices`"""
+    dev = require_device(grad_from_out_features, distances, features, neigh_indices, max_feat_indices)
+    g, w, x = f32(grad_from_out_features), f32(distances), f32(features)
+    idx, mi = i32(neigh_indices), i32(max_feat_indices)
+    n, k = idx.shape
+    f = x.shape[1]
+    mean_and_max = g.shape[1] > f  # modules/compiled/accumulate_knn_grad_kernel.cc:253
+    gw = torch.empty((n, k), dtype=torch.float32, device=dev)
+    gx = torch.empty((n, f), dtype=torch.float32, device=dev)
+    check(lib.hgc_accumulate_knn_grad(p(g), p(w), p(x), p(mi), p(idx), p(inv_offsets), p(inv_slots), p(gw), p(gx),
+                                      n, k, f, g.shape[1], 0, int(mean_and_max), stream()))
+    return gw, gx
+
+
+# --------------------------------------------------------------------------- condensates
+
+@torch.library.custom_op("hgcalml::binned_assign_to_condensates", mutates_args=())
+def binned_assign_to_condensates(ccoords: torch.Tensor, dist: torch.Tensor, beta: torch.Tensor,
+                                 no_condensation_mask: torch.Tensor, bins_flat: torch.Tensor,
+                                 bin_splits: torch.Tensor, indices_to_filtered: torch.Tensor,
+                                 original_indices: torch.Tensor, row_splits: torch.Tensor, n_bins: torch.Tensor,
+                                 bin_widths: torch.Tensor, ccoords_h: torch.Tensor, dist_h: torch.Tensor,
+                                 beta_h: torch.Tensor, no_condensation_mask_h: torch.Tensor,
+                                 row_splits_h: torch.Tensor, beta_threshold: float, assign_by_max_beta: bool
+                                 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """modules/compiled/binned_assign_to_condensates_module.cc:7-31; returns
+    (assigned_h, assigned, alpha_indices, association, n_condensates)."""
+    dev = require_device(ccoords, dist, beta, no_condensation_mask, bin_splits, indices_to_filtered,
+                         original_indices, row_splits, n_bins, bin_widths, ccoords_h, dist_h, beta_h,
+                         no_condensation_mask_h, row_splits_h)
+    ccoords, ccoords_h = f32(ccoords), f32(ccoords_h)
+    dist, dist_h = f32(dist).reshape(-1), f32(dist_h).reshape(-1)
+    beta_h = f32(beta_h).reshape(-1)
+    mask, mask_h = i32(no_condensation_mask).reshape(-1), i32(no_condensation_mask_h).reshape(-1)
+    bin_splits, to_filtered, orig_h = i32(bin_splits), i32(indices_to_filtered), i32(original_indices)
+    row_splits, row_splits_h, n_bins, bin_widths = i32(row_splits), i32(row_splits_h), i32(n_bins), f32(bin_widths)
+    n, c = ccoords.shape
+    nh = beta_h.numel()
+    num_rows = row_splits.numel() - 1
+    assigned_h = torch.zeros((nh,), dtype=torch.int32, device=dev)
+    assigned = torch.empty((n,), dtype=torch.int32, device=dev)
+    alpha = torch.empty((nh,), dtype=torch.int32, device=dev)
+    asso = torch.empty((n,), dtype=torch.int32, device=dev)
+    ncond = torch.empty((num_rows + 1,), dtype=torch.int32, device=dev)
+    taken_h = torch.empty((max(nh, 1),), dtype=torch.int32, device=dev)
+    best = None if assign_by_max_beta else torch.empty((max(n, 1),), dtype=torch.float32, device=dev)
+    ws = workspace(lib.hgc_binned_assign_to_condensates_workspace_bytes(n, nh, num_rows), dev)
+    check(lib.hgc_binned_assign_to_condensates(c, n_bins.numel(), p(taken_h), p(ccoords_h), p(dist_h), p(beta_h),
+                                               p(mask_h), p(assigned_h), p(orig_h), p(row_splits_h), p(ccoords),
+                                               p(dist), p(mask), p(to_filtered), p(best), p(assigned), p(asso),
+                                               p(ncond), p(alpha), p(bin_splits), p(n_bins), p(bin_widths),
+                                               p(row_splits), num_rows, int(assign_by_max_beta), n, nh, None, p(ws),
+                                               ws.numel(), stream()))
+    return assigned_h, assigned, alpha, asso, ncond

@@ -1,0 +1,253 @@
+/*
+ * hgcalml_amd — C ABI of the MI355X (gfx950) implementation of HGCalML's
+ * custom-op hot path: binned kNN, GravNet neighbour accumulation (forward and
+ * gradient) and object-condensation condensate assignment.
+ *
+ * Conventions
+ *   - Every pointer named d_* is DEVICE memory owned by the caller. Nothing
+ *     user visible is allocated by the library; scratch memory is passed in as
+ *     (workspace, workspace_bytes) and sized by the matching *_workspace_bytes
+ *     query. Workspace pointers must be 256-byte aligned.
+ *   - All tensors are dense row-major, `int` is int32, `float` is fp32.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream). All
+ *     work is enqueued on it; no call synchronises the device.
+ *   - Return value: 0 on success, a negative hgc_status otherwise. Argument
+ *     errors are detected on the host before anything is launched.
+ *   - The library is stateless and re-entrant; calls that share output or
+ *     workspace buffers must be ordered by the caller.
+ *
+ * Each entry point names the reference interface it replaces (paths relative
+ * to the HGCalML tree). The reference boundary is the functor
+ * `XOpFunctor<Device,int>::operator()(device, raw pointers..., sizes...)`
+ * declared in modules/compiled/X_kernel.h; argument order follows it.
+ */
+#ifndef HGCALML_AMD_H_
+#define HGCALML_AMD_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *hgc_stream_t;
+
+enum hgc_status {
+    HGC_OK = 0,
+    HGC_ERR_INVALID_ARGUMENT = -1, /* shape / range / null-pointer check failed */
+    HGC_ERR_WORKSPACE = -2,        /* workspace missing, misaligned or too small */
+    HGC_ERR_LAUNCH = -3,           /* the HIP runtime reported an error */
+    HGC_ERR_UNSUPPORTED = -4       /* valid for the reference, not built here */
+};
+
+/* Library version (major*10000 + minor*100 + patch). */
+int hgc_version(void);
+
+/* Human readable text for the last error raised on the calling thread. */
+const char *hgc_last_error(void);
+
+/* ------------------------------------------------------------------ */
+/* Spatial binning                                                     */
+/* ------------------------------------------------------------------ */
+
+/* Total number of bins = prod(n_bins) * (n_rs - 1); host arithmetic.
+ * Replaces BinByCoordinatesNbinsHelperOpFunctor
+ * (modules/compiled/bin_by_coordinates_kernel.h, _kernel.cc:17-35), without
+ * its device-to-host copy: n_bins is a HOST array here. */
+int hgc_bin_by_coordinates_total_bins(const int *h_n_bins, int n_nbins, int n_rs,
+                                      int *h_out_total_bins);
+
+/* Per point: per-dimension bin index int(coord / bin_width) (fallback 0 when
+ * out of range), event index from the row splits, flat bin index (event
+ * major, last coordinate fastest) and optionally the bin populations.
+ * Replaces BinByCoordinatesOpFunctor
+ * (modules/compiled/bin_by_coordinates_kernel.h, _kernel.cc:46-156).
+ *   d_coords [n_vert, n_coords], d_rs [n_rs], d_binswidth [1], d_n_bins [n_coords]
+ *   d_assigned_bin [n_vert, n_coords+1], d_flat_assigned_bin [n_vert],
+ *   d_n_per_bin [n_total_bins] (zeroed by the call; written only if calc_n_per_bin) */
+int hgc_bin_by_coordinates(const float *d_coords, const int *d_rs,
+                           const float *d_binswidth, const int *d_n_bins,
+                           int *d_assigned_bin, int *d_flat_assigned_bin, int *d_n_per_bin,
+                           int n_vert, int n_coords, int n_rs, int n_total_bins,
+                           int calc_n_per_bin, hgc_stream_t stream);
+
+/* Same kernel with the wrapper's pre-processing fused in: reads the first
+ * n_bin_dims columns of a [n_vert, coord_stride] matrix and subtracts
+ * d_shift[c] (may be NULL) before dividing. Replaces the slice and the
+ * `coordinates -= min` of modules/bin_by_coordinates_op.py:49-52 and
+ * modules/binned_select_knn_op.py:65-69. d_n_out_of_range (may be NULL) counts
+ * coordinates that fell outside the grid (the reference prints them). */
+int hgc_bin_by_coordinates_strided(const float *d_coords, int coord_stride, const float *d_shift,
+                                   const int *d_rs, const float *d_binswidth, const int *d_n_bins,
+                                   int *d_assigned_bin, int *d_flat_assigned_bin, int *d_n_per_bin,
+                                   int *d_n_out_of_range,
+                                   int n_vert, int n_bin_dims, int n_rs, int n_total_bins,
+                                   int calc_n_per_bin, hgc_stream_t stream);
+
+/* Bounding box and grid parameters, entirely on the device (no host sync).
+ * Replaces the TF glue of modules/bin_by_coordinates_op.py:46-71:
+ *   shift = column minimum (0 if pre_normalized), extent = max - shift,
+ *   +1 where the column is constant, +1e-3, non finite -> 1;
+ *   n_bins_scalar > 0: bin_width = max_d(extent_d / n_bins_scalar), else the
+ *   given d_bin_width_in[0]; n_bins_d = int(extent_d / bin_width + 1).
+ *   d_shift [n_bin_dims], d_bin_width [1], d_n_bins [n_bin_dims] are outputs. */
+size_t hgc_bin_setup_workspace_bytes(int n_vert, int n_bin_dims);
+int hgc_bin_setup(const float *d_coords, int coord_stride, int n_vert, int n_bin_dims,
+                  int pre_normalized, int n_bins_scalar, const float *d_bin_width_in,
+                  float *d_shift, float *d_bin_width, int *d_n_bins,
+                  void *workspace, size_t workspace_bytes, hgc_stream_t stream);
+
+/* Stable sort of the points by flat bin index plus the bin boundary table.
+ * Replaces tf.argsort + cumsum of modules/binned_select_knn_op.py:72-84 and
+ * tf.argsort + segment_ids_to_row_splits of modules/assign_condensate_op.py:276-284.
+ *   d_sorting [n_vert]: original index of the i-th point in bin order
+ *   d_bin_boundaries [n_total_bins+1]: start of every bin in that order */
+size_t hgc_sort_by_bin_workspace_bytes(int n_vert, int n_total_bins);
+int hgc_sort_by_bin(const int *d_flat_bin, int n_vert, int n_total_bins,
+                    int *d_sorting, int *d_bin_boundaries,
+                    void *workspace, size_t workspace_bytes, hgc_stream_t stream);
+
+/* out[i, :] = in[d_rows[i], :] for rows of `width` 4-byte elements (the
+ * gather_nd calls of modules/binned_select_knn_op.py:74-79). */
+int hgc_gather_rows(const void *d_in, const int *d_rows, void *d_out, int n_rows, int width,
+                    hgc_stream_t stream);
+
+/* ------------------------------------------------------------------ */
+/* Binned k nearest neighbours                                         */
+/* ------------------------------------------------------------------ */
+
+/* Exact kNN inside each event over bin-sorted points.
+ * Replaces BinnedSelectKnnOpFunctor
+ * (modules/compiled/binned_select_knn_kernel.h, _kernel.cc:47-282).
+ *   d_coord [n_vert, n_coords] (bin-sorted), d_bin_idx [n_vert],
+ *   d_direction [n_vert] (read only if use_direction),
+ *   d_dim_bin_idx [n_vert, n_bin_dim+1], d_bin_boundaries [n_bboundaries],
+ *   d_n_bins [n_bin_dim], d_bin_width [1];
+ *   d_indices, d_dist [n_vert, n_neigh].
+ * Output convention: slot 0 is the point itself; slots 1.. hold the neighbours
+ * in ascending (distance^2, index) order; missing neighbours are (-1, 0.0)
+ * (or (self, 0.0) if tf_compat) at the tail. The reference leaves the slots in
+ * fill/replacement order; the neighbour SET is the same except where the K-th
+ * and (K+1)-th distances are exactly equal, where the lower index is kept.
+ * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, 1 <= n_neigh <= 513. */
+int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int *d_direction,
+                          const int *d_dim_bin_idx, const int *d_bin_boundaries,
+                          const int *d_n_bins, const float *d_bin_width,
+                          int *d_indices, float *d_dist,
+                          int n_vert, int n_neigh, int n_coords, int n_bin_dim,
+                          int n_bboundaries, int tf_compat, int use_direction,
+                          hgc_stream_t stream);
+
+/* Same search with the wrapper's post-processing fused in
+ * (modules/binned_select_knn_op.py:92-95: IndexReplacer, two scatter_nd and the
+ * idx<0 -> distance 0 rule) and the radius cut of
+ * modules/compiled/select_knn_kernel.cc:158,244-245:
+ *   d_sorting (may be NULL) [n_vert]: original index of each sorted point; when
+ *     given, neighbour indices are reported in original index space, rows are
+ *     written at their original position and ties are broken by original index;
+ *   max_radius > 0: neighbours with distance^2 > max_radius^2 are dropped. */
+int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, const int *d_direction,
+                                const int *d_dim_bin_idx, const int *d_bin_boundaries,
+                                const int *d_n_bins, const float *d_bin_width,
+                                const int *d_sorting, float max_radius,
+                                int *d_indices, float *d_dist,
+                                int n_vert, int n_neigh, int n_coords, int n_bin_dim,
+                                int n_bboundaries, int tf_compat, int use_direction,
+                                hgc_stream_t stream);
+
+/* out[i] = v < 0 ? v : replacements[v]; entries with v >= n_replacements are
+ * left untouched. Replaces IndexReplacerOpFunctor
+ * (modules/compiled/index_replacer_kernel.h, _kernel.cc:17-42). */
+int hgc_index_replacer(const int *d_to_be_replaced, const int *d_replacements, int *d_replaced,
+                       int n_to_be_replaced, int n_replacements, hgc_stream_t stream);
+
+/* ------------------------------------------------------------------ */
+/* Neighbour accumulation (GravNet aggregation)                        */
+/* ------------------------------------------------------------------ */
+
+/* out[v, f] = sum_n w[v,n] * feat[idx[v,n], f] / K (slot order, fp32), and if
+ * mean_and_max: out[v, F+f] = max_n (...) with d_out_maxidxs[v,f] = the
+ * neighbour index that attained it (later slot wins ties; slot 0 seeds).
+ * Negative (and out-of-range) indices are skipped.
+ * Replaces AccumulateKnnOpFunctor
+ * (modules/compiled/accumulate_knn_kernel.h, _kernel.cc:27-83).
+ *   d_distances [n_vert, n_neigh] are the WEIGHTS (the wrapper applies exp(-d)),
+ *   d_feat [n_vert, n_feat], d_idxs [n_vert, n_neigh],
+ *   d_out_feat [n_vert, n_out_feat] with n_out_feat = n_feat * (mean_and_max ? 2 : 1),
+ *   d_out_maxidxs [n_vert, n_feat] (written only if mean_and_max). */
+int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int *d_idxs,
+                       float *d_out_feat, int *d_out_maxidxs,
+                       int n_vert, int n_neigh, int n_feat, int n_out_feat,
+                       int n_moments, int mean_and_max, hgc_stream_t stream);
+
+/* Inverse neighbour index: for every vertex m the list of (vertex, slot)
+ * pairs that name m, ascending. Built once per neighbour table and reused by
+ * every gradient call on it.
+ *   d_inv_offsets [n_vert+1], d_inv_slots [n_vert*n_neigh] (flat slot v*K+n) */
+size_t hgc_inverse_neighbour_index_workspace_bytes(int n_vert, int n_neigh);
+int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh,
+                                int *d_inv_offsets, int *d_inv_slots,
+                                void *workspace, size_t workspace_bytes, hgc_stream_t stream);
+
+/* Gradients of hgc_accumulate_knn w.r.t. the weights and the features.
+ * Replaces AccumulateKnnGradOpFunctor
+ * (modules/compiled/accumulate_knn_grad_kernel.h, _kernel.cc:24-227); the
+ * contended atomicAdd of the reference's device path becomes an ordered
+ * gather through the inverse neighbour index, which reproduces the CPU
+ * kernel's summation order for the feature gradient.
+ *   d_grad_from_out_features [n_vert, n_grad_from_out_feat]
+ *     (n_grad_from_out_feat == 2*n_feat selects mean_and_max),
+ *   d_distances (weights), d_feat, d_max_feat_indices [n_vert, n_feat], d_neigh_indices,
+ *   d_inv_offsets / d_inv_slots from hgc_inverse_neighbour_index,
+ *   d_out_grad_distances [n_vert, n_neigh], d_out_grad_features [n_vert, n_feat]. */
+int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *d_distances,
+                            const float *d_feat, const int *d_max_feat_indices,
+                            const int *d_neigh_indices,
+                            const int *d_inv_offsets, const int *d_inv_slots,
+                            float *d_out_grad_distances, float *d_out_grad_features,
+                            int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
+                            int n_moments, int mean_and_max, hgc_stream_t stream);
+
+/* ------------------------------------------------------------------ */
+/* Condensate assignment                                               */
+/* ------------------------------------------------------------------ */
+
+/* Greedy highest-beta-first condensate selection and hit assignment per event.
+ * Replaces BinnedCondensatesFinderOpFunctor
+ * (modules/compiled/binned_assign_to_condensates_kernel.h, _kernel.cc:23-241);
+ * argument order follows the functor, sizes the reference derives from tensor
+ * shapes are explicit. Arrays without suffix hold all hits in bin-sorted order,
+ * *_h the high-beta subset in the same order.
+ *   outputs: d_high_assigned_status_h [n_vert_h] (1 for condensate points),
+ *   d_assignment [n_vert] (shower index inside the event, -1 noise),
+ *   d_association [n_vert] (original index of the condensate point, -1 noise),
+ *   d_n_condensates [num_rows+1] (cumulative), d_alpha_indices [n_vert_h]
+ *   (original indices of the condensate points per event, -1 padded).
+ *   d_condensates_assigned_h [n_vert_h] and d_assignment_min_distance [n_vert]
+ *   (the latter only if !assign_by_max_beta) are caller scratch like in the
+ *   reference. d_error (may be NULL) receives 1 if an event made no progress
+ *   (the reference throws std::runtime_error there). */
+size_t hgc_binned_assign_to_condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows);
+int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning,
+                                     int *d_condensates_assigned_h,
+                                     const float *d_ccoords_h, const float *d_dist_h,
+                                     const float *d_beta_h, const int *d_no_condensation_mask_h,
+                                     int *d_high_assigned_status_h,
+                                     const int *d_original_indices_h, const int *d_row_splits_h,
+                                     const float *d_ccoords, const float *d_dist,
+                                     const int *d_no_condensation_mask,
+                                     const int *d_indices_to_filtered,
+                                     float *d_assignment_min_distance,
+                                     int *d_assignment, int *d_association,
+                                     int *d_n_condensates, int *d_alpha_indices,
+                                     const int *d_bin_splits, const int *d_n_bins,
+                                     const float *d_bin_widths, const int *d_row_splits,
+                                     int num_rows, int assign_by_max_beta,
+                                     int n_vert, int n_vert_h, int *d_error,
+                                     void *workspace, size_t workspace_bytes,
+                                     hgc_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HGCALML_AMD_H_ */

@@ -266,13 +266,14 @@ def BinnedSelectKnn(K, coords, row_splits, direction=None, n_bins=None, max_bin_
 
 def canonical_knn(idx, dist):
     """Slot 0 kept; the other slots ordered by ascending (d^2, index) with the
-    (-1, 0.0) padding at the tail. Used to compare neighbour sets."""
+    padding at the tail. Used to compare neighbour sets."""
     idx = np.asarray(idx)
     dist = np.asarray(dist)
     n, K = idx.shape
     if K <= 1:
         return idx.copy(), dist.copy()
-    pad = idx[:, 1:] < 0
+    # padding is -1, or a repeated self reference in tf_compatible mode
+    pad = (idx[:, 1:] < 0) | (idx[:, 1:] == idx[:, :1])
     dkey = np.where(pad, np.float32(np.inf), dist[:, 1:])
     ikey = np.where(pad, np.iinfo(np.int32).max, idx[:, 1:])
     order = np.lexsort((ikey, dkey), axis=1)

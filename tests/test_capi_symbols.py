@@ -1,0 +1,91 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol that
+include/hgcalml_amd.h declares, and rejects bad arguments on the host before
+anything is launched (no GPU needed for any of this)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hgcalml_amd.h")
+LIB = os.path.join(ROOT, "hgcalml_amd", "libhgcalml_amd.so")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hgc_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def capi():
+    if not os.path.exists(LIB):
+        from hgcalml_amd import build
+        build.build(verbose=False)
+    return ctypes.CDLL(LIB)
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for must in ("hgc_bin_by_coordinates", "hgc_binned_select_knn", "hgc_index_replacer", "hgc_accumulate_knn",
+                 "hgc_accumulate_knn_grad", "hgc_binned_assign_to_condensates"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(capi):
+    for name in declared_symbols():
+        assert hasattr(capi, name), "missing export: " + name
+
+
+def test_python_binding_covers_every_declared_symbol(capi):
+    from hgcalml_amd import _lib
+    assert sorted(_lib.EXPORTED_SYMBOLS) == declared_symbols()
+
+
+def test_host_side_argument_checks(capi):
+    capi.hgc_last_error.restype = ctypes.c_char_p
+    assert capi.hgc_version() >= 100
+    # total bins: host arithmetic
+    nb = (ctypes.c_int * 3)(30, 29, 31)
+    out = ctypes.c_int(0)
+    assert capi.hgc_bin_by_coordinates_total_bins(nb, 3, 17, ctypes.byref(out)) == 0
+    assert out.value == 30 * 29 * 31 * 16
+    nb[1] = 0
+    assert capi.hgc_bin_by_coordinates_total_bins(nb, 3, 17, ctypes.byref(out)) == -1
+    assert b"positive" in capi.hgc_last_error()
+    # kNN shape rules of the reference op: 2 <= binning dims <= 5, >= 2 coordinates
+    null = ctypes.c_void_p(None)
+    args_tail = [null] * 9
+    f = capi.hgc_binned_select_knn
+    f.argtypes = [ctypes.c_void_p] * 9 + [ctypes.c_int] * 7 + [ctypes.c_void_p]
+    assert f(*args_tail, 10, 4, 3, 1, 5, 0, 0, null) == -1
+    assert b"at least 2 binning dimensions" in capi.hgc_last_error()
+    assert f(*args_tail, 10, 4, 3, 6, 5, 0, 0, null) == -1
+    assert b"maximum 5 binning dimensions" in capi.hgc_last_error()
+    assert f(*args_tail, 10, 4, 1, 2, 5, 0, 0, null) == -1
+    assert f(*args_tail, 10, 4, 3, 3, 5, 0, 0, null) == -1 and b"null pointer" in capi.hgc_last_error()
+    assert f(*args_tail, 0, 4, 3, 3, 5, 0, 0, null) == 0  # empty input is fine
+    # accumulate: output width must match mean_and_max
+    g = capi.hgc_accumulate_knn
+    g.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p]
+    assert g(*([null] * 5), 10, 4, 8, 8, 0, 1, null) == -1
+    assert g(*([null] * 5), 0, 4, 8, 16, 0, 1, null) == 0
+    # workspace queries are pure host functions
+    capi.hgc_sort_by_bin_workspace_bytes.restype = ctypes.c_size_t
+    capi.hgc_inverse_neighbour_index_workspace_bytes.restype = ctypes.c_size_t
+    assert capi.hgc_sort_by_bin_workspace_bytes(150000, 27000) >= 2 * 150000 * 4
+    assert capi.hgc_inverse_neighbour_index_workspace_bytes(1000, 64) >= 3 * 64000 * 4
+    # missing workspace is reported, not dereferenced
+    h = capi.hgc_sort_by_bin
+    h.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                  ctypes.c_size_t, ctypes.c_void_p]
+    one = ctypes.c_void_p(256)
+    assert h(one, 10, 10, one, one, null, 0, null) == -2
+
+
+def test_package_refuses_cpu_tensors(capi):
+    import torch
+    from hgcalml_amd import AccumulateLinKnn
+    with pytest.raises(RuntimeError, match="GPU"):
+        AccumulateLinKnn(torch.ones(4, 2), torch.ones(4, 3), torch.zeros(4, 2, dtype=torch.int32))

@@ -1,0 +1,456 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on
+the same seeded inputs.
+
+Bars: integer outputs (bins, neighbour indices, arg-max indices, condensate
+assignment) bit-exact; neighbour distances, accumulate forward and the feature
+gradient bit-exact (same fp32 operation order); the weight gradient within
+1e-5 relative to the magnitude of the summed terms (its dot products are
+reduced in a different order than the oracle's serial loop).
+"""
+import numpy as np
+import pytest
+import torch
+
+from hgcalml_amd import workloads
+from helpers import check_knn_rows
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def t(a, dtype=None):
+    return torch.as_tensor(np.ascontiguousarray(a), dtype=dtype).to(DEV)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.int32)
+
+
+# ------------------------------------------------------------------ binning
+
+@pytest.mark.parametrize("pre_normalized", [False, True])
+def test_bin_by_coordinates_matches_oracle(oracle, pre_normalized):
+    from hgcalml_amd import BinByCoordinates
+    rng = np.random.default_rng(11)
+    x = (rng.random((5000, 3), dtype=np.float32) * np.array([4., 2., 1.], np.float32)).astype(np.float32)
+    if not pre_normalized:
+        x = x + np.array([-3., 5., 0.25], np.float32)
+    rs = np.array([0, 1200, 1200, 3100, 5000], np.int32)
+    for kwargs in (dict(n_bins=13), dict(bin_width=np.array([0.21], np.float32))):
+        ref = oracle.BinByCoordinates(x, rs, pre_normalized=pre_normalized, **kwargs)
+        tk = {k: (int(v) if k == "n_bins" else t(v)) for k, v in kwargs.items()}
+        got = BinByCoordinates(t(x), t(rs), pre_normalized=pre_normalized, **tk)
+        assert len(got) == 5
+        for g, r in zip(got, ref):
+            g = g.cpu().numpy()
+            assert g.shape == np.shape(r)
+            if g.dtype == np.float32:
+                assert (bits(g) == bits(r)).all()
+            else:
+                assert (g == r).all()
+    got4 = BinByCoordinates(t(x), t(rs), n_bins=7, calc_n_per_bin=False, pre_normalized=pre_normalized)
+    ref4 = oracle.BinByCoordinates(x, rs, n_bins=7, calc_n_per_bin=False, pre_normalized=pre_normalized)
+    assert len(got4) == 4 and (got4[1].cpu().numpy() == ref4[1]).all()
+
+
+def test_bin_kernel_out_of_range_and_edges(oracle):
+    rng = np.random.default_rng(12)
+    n = 300
+    coords = (rng.random((n, 3), dtype=np.float32) * np.float32(3.0)).astype(np.float32)
+    coords[5] = [1.0, 1.5, 2.5]
+    coords[9, 1] = 3.6
+    coords[11, 0] = -0.7
+    bw = np.array([0.5], np.float32)
+    nb = np.array([6, 7, 6], np.int32)
+    rs = np.array([0, 100, 100, 300], np.int32)
+    rb, rf, rn, bad = oracle.bin_by_coordinates_kernel(coords, rs, bw, nb)
+    assert bad == 2
+    gb, gf, gn = torch.ops.hgcalml.bin_by_coordinates(t(coords), t(rs), t(bw), t(nb), int(np.prod(nb)) * 3, True)
+    assert (gb.cpu().numpy() == rb).all() and (gf.cpu().numpy() == rf).all() and (gn.cpu().numpy() == rn).all()
+
+
+def test_sort_by_bin_is_stable_and_boundaries_match():
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(13)
+    flat = rng.integers(0, 500, size=20000).astype(np.int32)
+    flat[rng.integers(0, 20000, 3000)] = 17  # one crowded bin
+    sorting, bounds = ops.sort_by_bin(t(flat), 700)
+    want = np.argsort(flat, kind="stable")
+    assert (sorting.cpu().numpy() == want).all()
+    wb = np.concatenate([[0], np.cumsum(np.bincount(flat, minlength=700))])
+    assert (bounds.cpu().numpy() == wb).all()
+    g = ops.gather_rows(t(np.arange(60000, dtype=np.float32).reshape(20000, 3)), sorting).cpu().numpy()
+    assert (g[:, 0] == want * 3).all()
+
+
+def test_index_replacer(oracle):
+    from hgcalml_amd import IndexReplacer
+    rep = np.arange(100, 200, dtype=np.int32)
+    tbr = np.random.default_rng(14).integers(-2, 100, size=(50, 7)).astype(np.int32)
+    tbr[3, 3] = 150  # beyond the table: left untouched (zero initialised output)
+    got = IndexReplacer(t(tbr), t(rep)).cpu().numpy()
+    assert (got == oracle.IndexReplacer(tbr, rep)).all()
+
+
+# ------------------------------------------------------------------ kNN
+
+def compare_knn(oracle, got_idx, got_dist, ref_idx, ref_dist, coords, rs, K, **kw):
+    """bitwise equality of the canonical forms; rows that differ must be exact
+    K-th boundary ties and valid kNN sets. Returns the number of such rows."""
+    gi, gd = got_idx.cpu().numpy(), got_dist.cpu().numpy()
+    # the HIP path already emits the canonical order
+    ci, cd = oracle.canonical_knn(gi, gd)
+    assert (ci == gi).all() and (bits(cd) == bits(gd)).all()
+    ri, rd = oracle.canonical_knn(ref_idx, ref_dist)
+    differ = np.nonzero((ri != gi).any(axis=1) | (bits(rd) != bits(gd)).any(axis=1))[0]
+    if len(differ):
+        ties = check_knn_rows(oracle, gi, gd, coords, rs, K, differ, **kw)
+        assert ties == len(differ), "rows differ from the oracle without an exact tie at the K-th boundary"
+    return len(differ)
+
+
+def run_knn_case(oracle, coords, rs, K, n_bins, direction=None, tf_compatible=False, max_radius=None,
+                 max_ties=0):
+    from hgcalml_amd import BinnedSelectKnn
+    ref_i, ref_d = oracle.BinnedSelectKnn(K, coords, rs, direction=direction, n_bins=n_bins,
+                                          tf_compatible=tf_compatible, max_radius=max_radius)
+    got_i, got_d = BinnedSelectKnn(K, t(coords), t(rs), direction=None if direction is None else t(direction),
+                                   n_bins=n_bins, tf_compatible=tf_compatible, max_radius=max_radius)
+    assert got_i.dtype == torch.int32 and got_d.dtype == torch.float32 and tuple(got_i.shape) == (len(coords), K)
+    kw = dict(direction=direction, tf_compatible=tf_compatible)
+    if max_radius is not None:
+        kw["radius"] = max_radius
+    n_ties = compare_knn(oracle, got_i, got_d, ref_i, ref_d, coords, rs, K, **kw)
+    assert n_ties <= max_ties
+    return got_i, got_d
+
+
+def test_knn_cfg1_full(oracle):
+    c = workloads.cfg1()
+    run_knn_case(oracle, c["coords"], c["row_splits"], c["K"], c["n_bins"])
+
+
+def test_knn_cfg2_full(oracle):
+    c = workloads.cfg2()
+    idx, dist = run_knn_case(oracle, c["coords"], c["row_splits"], c["K"], c["n_bins"])
+    # independent of the oracle: sampled rows against an O(N) brute force
+    rows = np.random.default_rng(15).choice(len(c["coords"]), 300, replace=False)
+    assert check_knn_rows(oracle, idx.cpu().numpy(), dist.cpu().numpy(), c["coords"], c["row_splits"], c["K"],
+                          rows) == 0
+
+
+def test_knn_cfg3_ragged_radius(oracle):
+    c = workloads.cfg3(scale=0.1)
+    idx, dist = run_knn_case(oracle, c["coords"], c["row_splits"], c["K"], c["n_bins"], max_radius=c["max_radius"])
+    i = idx.cpu().numpy()
+    pad = i[:, 1:] < 0
+    assert pad.any() and (np.diff(pad.astype(int), axis=1) >= 0).all()  # -1 only at the tail
+    assert (dist.cpu().numpy()[:, 1:][pad] == 0).all()
+
+
+@pytest.mark.parametrize("C,B", [(2, 2), (3, 3), (3, 2), (4, 3), (5, 3), (6, 4), (5, 5)])
+def test_knn_dimensions(oracle, C, B):
+    from hgcalml_amd import BinnedSelectKnn
+    rng = np.random.default_rng(16 + C * 10 + B)
+    coords = rng.standard_normal((3000, C)).astype(np.float32)
+    rs = np.array([0, 1300, 3000], np.int32)
+    ref_i, ref_d = oracle.BinnedSelectKnn(12, coords, rs, n_bins=6, max_bin_dims=B)
+    got_i, got_d = BinnedSelectKnn(12, t(coords), t(rs), n_bins=6, max_bin_dims=B)
+    assert compare_knn(oracle, got_i, got_d, ref_i, ref_d, coords, rs, 12) == 0
+
+
+@pytest.mark.parametrize("K", [1, 2, 33, 65, 66, 130, 200, 300])
+def test_knn_neighbour_counts(oracle, K):
+    rng = np.random.default_rng(17 + K)
+    coords = rng.random((2500, 3), dtype=np.float32)
+    rs = np.array([0, 2500], np.int32)
+    run_knn_case(oracle, coords, rs, K, 7)
+
+
+def test_knn_small_events_direction_tf_compat(oracle):
+    rng = np.random.default_rng(18)
+    coords = rng.standard_normal((330, 3)).astype(np.float32)
+    rs = np.array([0, 7, 7, 30, 330], np.int32)
+    K = 24
+    for tfc in (False, True):
+        run_knn_case(oracle, coords, rs, K, 5, tf_compatible=tfc)
+    direction = rng.integers(0, 4, size=330).astype(np.int32)
+    run_knn_case(oracle, coords, rs, K, 5, direction=direction)
+    run_knn_case(oracle, coords, rs, K, 5, direction=direction, tf_compatible=True)
+    run_knn_case(oracle, coords, rs, K, 5, max_radius=0.6)
+
+
+def test_knn_lattice_ties_lower_index_wins(oracle):
+    from hgcalml_amd import BinnedSelectKnn
+    g = np.arange(8, dtype=np.float32)
+    coords = np.stack(np.meshgrid(g, g, g, indexing="ij"), -1).reshape(-1, 3)
+    rs = np.array([0, 512], np.int32)
+    got_i, got_d = run_knn_case(oracle, coords, rs, 8, 5, max_ties=512)
+    # the documented tie rule: ascending (distance, original index) brute force
+    gi = got_i.cpu().numpy()
+    from helpers import brute_knn_row
+    for i in range(0, 512, 7):
+        bj, _ = brute_knn_row(coords, 0, 512, i)
+        assert (gi[i, 1:] == bj[:7]).all()
+
+
+def test_knn_functor_level_entry_point(oracle):
+    """the raw op on bin-sorted inputs (ties broken by sorted index)"""
+    from hgcalml_amd.binned_select_knn_op import _BinnedSelectKnn
+    c = workloads.cfg2(scale=0.05)
+    coords, rs = c["coords"], c["row_splits"]
+    dbin, flat, nb, bw, nper = oracle.BinByCoordinates(coords[:, :3], rs, n_bins=12)
+    order = np.argsort(flat, kind="stable")
+    bb = np.concatenate([[0], np.cumsum(nper)]).astype(np.int32)
+    ref_i, ref_d = oracle.binned_select_knn_kernel(20, coords[order], flat[order], dbin[order], bb, nb, bw)
+    got_i, got_d = _BinnedSelectKnn(20, t(coords[order]), t(flat[order]), t(dbin[order]), t(bb), t(nb), t(bw))
+    assert compare_knn(oracle, got_i, got_d, ref_i, ref_d, coords[order], rs, 20) == 0
+
+
+# ------------------------------------------------------------------ accumulate
+
+def make_acc_case(rng, n, K, F, holes=True):
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    idx = np.stack([np.concatenate([[v], rng.permutation(np.delete(np.arange(n), v))[:K - 1]])
+                    for v in range(n)]).astype(np.int32)
+    if holes:
+        idx[n // 8:n // 4, K // 2:] = -1   # -1 tail
+        idx[n // 2, 0] = -1               # slot 0 missing
+        idx[n // 2 + 1, K // 2:] = n // 2 + 1  # duplicated-self padding
+        idx[n // 2 + 2, :] = -1           # no neighbours at all
+    d = rng.random((n, K), dtype=np.float32)
+    return d, x, idx
+
+
+@pytest.mark.parametrize("K,F", [(8, 3), (16, 32), (64, 64), (10, 128), (64, 128), (7, 20)])
+def test_accumulate_forward_bit_exact(oracle, K, F):
+    from hgcalml_amd import AccumulateKnn, AccumulateLinKnn
+    rng = np.random.default_rng(19 + K + F)
+    d, x, idx = make_acc_case(rng, 400, K, F)
+    w = np.exp(-d).astype(np.float32)
+    for mm in (True, False):
+        ref, rarg = oracle.AccumulateLinKnn(w, x, idx, mm)
+        out, arg = AccumulateLinKnn(t(w), t(x), t(idx), mean_and_max=mm)
+        assert (bits(out.cpu().numpy()) == bits(ref)).all()
+        if mm:
+            assert (arg.cpu().numpy() == rarg).all()
+    # exp(-d) in front: within 1e-5 relative (library exp), arg-max identical away from ties
+    ref, _ = oracle.AccumulateKnn(d, x, idx)
+    out, _ = AccumulateKnn(t(d), t(x), t(idx))
+    assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-6)
+
+
+def test_accumulate_forward_ties_and_slot0(oracle):
+    from hgcalml_amd import AccumulateLinKnn
+    x = np.array([[2., -1.], [2., -1.], [2., -3.]], np.float32)
+    idx = np.array([[0, 1, 2], [-1, 0, 2], [-1, 2, -1]], np.int32)
+    w = np.ones((3, 3), np.float32)
+    ref, rarg = oracle.AccumulateLinKnn(w, x, idx)
+    out, arg = AccumulateLinKnn(t(w), t(x), t(idx))
+    assert (bits(out.cpu().numpy()) == bits(ref)).all() and (arg.cpu().numpy() == rarg).all()
+    assert (rarg[0] == [2, 1]).all()      # later slot wins the tie
+    assert (rarg[2] == [2, 0]).all()      # slot 0 missing: max floored at 0, index 0
+
+
+def grad_tolerance(g, x, idx, w, K):
+    """1e-5 relative to the sum of |terms| of each weight-gradient entry"""
+    n, F = x.shape
+    gm, gx = np.abs(g[:, :F]), np.abs(g[:, F:]) if g.shape[1] > F else 0
+    ax = np.abs(x[np.maximum(idx, 0)])                    # [n, K, F]
+    scale = (ax * (gm / K + gx)[:, None, :]).sum(-1)
+    return 1e-5 * scale + 1e-30
+
+
+@pytest.mark.parametrize("K,F", [(8, 4), (16, 32), (64, 64), (12, 128), (5, 7), (64, 96)])
+def test_accumulate_gradient(oracle, K, F):
+    rng = np.random.default_rng(20 + K + F)
+    d, x, idx = make_acc_case(rng, 300, K, F)
+    w = np.exp(-d).astype(np.float32)
+    for mm in (True, False):
+        g = rng.standard_normal((300, 2 * F if mm else F)).astype(np.float32)
+        _, arg = oracle.AccumulateLinKnn(w, x, idx, mm)
+        rgw, rgx = oracle.accumulate_knn_grad_kernel(g, w, x, idx, arg)
+        from hgcalml_amd import ops
+        inv = ops.inverse_neighbour_index(t(idx))
+        gw, gx = torch.ops.hgcalml.accumulate_knn_grad(t(g), t(w), t(x), t(idx), t(arg), *inv)
+        # feature gradient: same addends in the same order -> identical bits
+        assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
+        # weight gradient: tree reduction over the features
+        err = np.abs(gw.cpu().numpy() - rgw)
+        assert (err <= grad_tolerance(g, x, idx, w, K)).all()
+        assert (gw.cpu().numpy()[idx < 0] == 0).all()
+
+
+def test_inverse_neighbour_index_is_ordered():
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(21)
+    idx = rng.integers(-1, 500, size=(500, 9)).astype(np.int32)
+    off, slots = ops.inverse_neighbour_index(t(idx))
+    off, slots = off.cpu().numpy(), slots.cpu().numpy()
+    flat = idx.reshape(-1)
+    assert off[0] == 0 and off[-1] == (flat >= 0).sum()
+    for m in range(500):
+        mine = slots[off[m]:off[m + 1]]
+        assert (mine == np.nonzero(flat == m)[0]).all()
+
+
+def test_accumulate_autograd_chain(oracle):
+    from hgcalml_amd import AccumulateKnn
+    rng = np.random.default_rng(22)
+    d, x, idx = make_acc_case(rng, 200, 16, 32)
+    g = rng.standard_normal((200, 64)).astype(np.float32)
+    td, tx = t(d).requires_grad_(True), t(x).requires_grad_(True)
+    tidx = t(idx)
+    out, arg = AccumulateKnn(td, tx, tidx)
+    out.backward(t(g))
+    _, rarg = oracle.AccumulateKnn(d, x, idx)
+    # second backward on the same table reuses the cached inverse index
+    out2, _ = AccumulateKnn(td, tx, tidx)
+    (out2 * 2).backward(t(g))
+    w = np.exp(-d).astype(np.float32)
+    rgd, rgx = oracle.AccumulateKnnGrad(g, d, x, idx, rarg)
+    tol = grad_tolerance(g, x, idx, w, 16)
+    assert (np.abs(td.grad.cpu().numpy() / 3 - rgd) <= 3 * tol + 1e-6 * np.abs(rgd)).all()
+    assert np.allclose(tx.grad.cpu().numpy() / 3, rgx, rtol=1e-5, atol=1e-6)
+
+
+def test_accumulate_cfg4_scaled(oracle):
+    c = workloads.cfg4(scale=0.03)
+    w = np.exp(-c["distsq"]).astype(np.float32)
+    from hgcalml_amd import AccumulateLinKnn, ops
+    ref, rarg = oracle.AccumulateLinKnn(w, c["features"], c["indices"])
+    out, arg = AccumulateLinKnn(t(w), t(c["features"]), t(c["indices"]))
+    assert (bits(out.cpu().numpy()) == bits(ref)).all() and (arg.cpu().numpy() == rarg).all()
+    rgw, rgx = oracle.accumulate_knn_grad_kernel(c["grad_out"], w, c["features"], c["indices"], rarg)
+    inv = ops.inverse_neighbour_index(t(c["indices"]))
+    gw, gx = torch.ops.hgcalml.accumulate_knn_grad(t(c["grad_out"]), t(w), t(c["features"]), t(c["indices"]), arg, *inv)
+    assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
+    assert (np.abs(gw.cpu().numpy() - rgw) <= grad_tolerance(c["grad_out"], c["features"], c["indices"], w, 64)).all()
+
+
+def test_accumulate_cfg4_full_size_properties(oracle):
+    """N=1M: sampled rows against the oracle (forward) and linearity of the
+    gradient in the upstream gradient."""
+    c = workloads.cfg4()
+    from hgcalml_amd import AccumulateLinKnn, ops
+    w = np.exp(-c["distsq"]).astype(np.float32)
+    tw, tx, ti = t(w), t(c["features"]), t(c["indices"])
+    out, arg = AccumulateLinKnn(tw, tx, ti)
+    rows = np.random.default_rng(23).choice(len(w), 4000, replace=False)
+    ref, rarg = oracle.accumulate_knn_kernel(w[rows], c["features"], c["indices"][rows])
+    assert (bits(out[t(rows)].cpu().numpy()) == bits(ref)).all()
+    assert (arg[t(rows)].cpu().numpy() == rarg).all()
+    inv = ops.inverse_neighbour_index(ti)
+    g = t(c["grad_out"])
+    gw1, gx1 = torch.ops.hgcalml.accumulate_knn_grad(g, tw, tx, ti, arg, *inv)
+    gw2, gx2 = torch.ops.hgcalml.accumulate_knn_grad(g * 2, tw, tx, ti, arg, *inv)
+    # scaling by two is exact in fp32, so both gradients double bit for bit
+    assert torch.equal(gx1 * 2, gx2) and torch.equal(gw1 * 2, gw2)
+    # total feature gradient == total of what the vertices push out (float64 check):
+    # mean part (g/K)*sum_n w[v,n], max part to the arg-max neighbour with that slot's weight
+    per_vertex_w = tw.double().sum(1, keepdim=True)
+    mean_total = ((g[:, :128].double() / 64) * per_vertex_w).sum(0)
+    total = gx1.double().sum(0)
+    max_total = torch.zeros(128, dtype=torch.float64, device=DEV)
+    for s in range(0, len(w), 50000):
+        e = min(len(w), s + 50000)
+        m = (ti[s:e, :, None] == arg[s:e, None, :])
+        max_total += (m * tw[s:e, :, None].double() * g[s:e, None, 128:].double()).sum((0, 1))
+    assert torch.allclose(total, mean_total + max_total, rtol=1e-6, atol=1e-3)
+
+
+# ------------------------------------------------------------------ condensates
+
+def run_condensates(oracle, cfg, by_max_beta, mask=None):
+    from hgcalml_amd import BuildAndAssignCondensatesBinned
+    ref = oracle.BuildAndAssignCondensatesBinned(cfg["ccoords"], cfg["betas"], cfg["dist"], cfg["row_splits"],
+                                                 cfg["beta_threshold"], no_condensation_mask=mask,
+                                                 distance_threshold=cfg["distance_threshold"],
+                                                 assign_by_max_beta=by_max_beta)
+    got = BuildAndAssignCondensatesBinned(t(cfg["ccoords"]), t(cfg["betas"]), t(cfg["dist"]), t(cfg["row_splits"]),
+                                          cfg["beta_threshold"],
+                                          no_condensation_mask=None if mask is None else t(mask),
+                                          distance_threshold=cfg["distance_threshold"],
+                                          assign_by_max_beta=by_max_beta)
+    names = ("assignment", "association", "alpha_idx", "is_cond", "n_condensates")
+    for name, g, r in zip(names, got, ref):
+        g = g.cpu().numpy()
+        assert g.shape == r.shape, name
+        assert (g == r).all(), name
+    return got
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensates_cfg5_scaled(oracle, by_max_beta):
+    cfg = workloads.cfg5(scale=0.1)
+    got = run_condensates(oracle, cfg, by_max_beta)
+    assert int(got[4][-1]) > 50
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensates_cfg5_full(oracle, by_max_beta):
+    run_condensates(oracle, workloads.cfg5(), by_max_beta)
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensates_per_hit_radii_and_ties(oracle, by_max_beta):
+    cfg = workloads.cfg5(scale=0.05, n_events=5)
+    rng = np.random.default_rng(24)
+    cfg["dist"] = (0.15 * rng.uniform(0.6, 1.4, size=cfg["dist"].shape)).astype(np.float32)
+    cfg["distance_threshold"] = 0.7
+    run_condensates(oracle, cfg, by_max_beta)
+
+
+@pytest.mark.parametrize("t_b", [1e-5, 0.1, 0.9999])
+def test_condensates_grid_and_degenerate_coordinates(oracle, t_b):
+    rng = np.random.default_rng(25)
+    gx, gy = np.meshgrid(np.linspace(0, 10, 4), np.linspace(0, 10, 3))
+    x = np.concatenate([np.stack([gx, gy], -1).reshape(-1, 2)] * 2).astype(np.float32)
+    beta = rng.random((24, 1)).astype(np.float32)
+    for coords in (x, 0 * x):
+        cfg = dict(ccoords=coords, betas=beta, dist=np.ones_like(beta), row_splits=np.array([0, 12, 24], np.int32),
+                   beta_threshold=t_b, distance_threshold=1.0)
+        run_condensates(oracle, cfg, False)
+        run_condensates(oracle, cfg, True)
+
+
+def test_condensates_empty_event_and_no_high_beta(oracle):
+    cfg = workloads.cfg5(scale=0.02, n_events=3)
+    n = len(cfg["betas"])
+    per = n // 3
+    cfg["row_splits"] = np.array([0, per, per, 2 * per, n], np.int32)   # an empty event
+    cfg["betas"][per:2 * per] = 0.01                                     # an event without high-beta hits
+    run_condensates(oracle, cfg, True)
+    run_condensates(oracle, cfg, False)
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensates_with_no_condensation_mask(oracle, by_max_beta):
+    cfg = workloads.cfg5(scale=0.03, n_events=2)
+    rng = np.random.default_rng(26)
+    mask = (rng.random(len(cfg["betas"])) < 0.01).astype(np.int32)[:, None]
+    run_condensates(oracle, cfg, by_max_beta, mask=mask)
+
+
+def test_condensates_keep_noise_structure(oracle):
+    """keep_noise: every noise hit becomes its own condensation point, numbered
+    before the real ones; the reference's own sanity relation must hold."""
+    from hgcalml_amd import BuildAndAssignCondensatesBinned
+    cfg = workloads.cfg5(scale=0.02, n_events=3)
+    args = (t(cfg["ccoords"]), t(cfg["betas"]), t(cfg["dist"] * 0.2), t(cfg["row_splits"]), cfg["beta_threshold"])
+    a0, s0, al0, c0, n0 = [x.cpu().numpy() for x in BuildAndAssignCondensatesBinned(*args, assign_by_max_beta=True)]
+    a1, s1, al1, c1, n1 = [x.cpu().numpy() for x in BuildAndAssignCondensatesBinned(*args, assign_by_max_beta=True,
+                                                                                    keep_noise=True)]
+    rs = cfg["row_splits"]
+    assert (a0 < 0).any()
+    assert (a1 >= 0).all() and (s1 >= 0).all()
+    assert (s1[s0 < 0] == np.nonzero(s0 < 0)[0]).all() and (s1[s0 >= 0] == s0[s0 >= 0]).all()
+    for e in range(3):
+        lo, hi = rs[e], rs[e + 1]
+        n_noise = int((a0[lo:hi, 0] < 0).sum())
+        assert n1[e + 1] - n1[e] == n_noise + (n0[e + 1] - n0[e])
+        assert a1[lo:hi, 0].max() + 1 == n1[e + 1] - n1[e]
+        # gathering the assignment at the alpha indices gives 0..n-1 per event
+        assert (a1[al1[n1[e]:n1[e + 1]], 0] == np.arange(n1[e + 1] - n1[e])).all()
+    assert c1.sum() == len(al1)
