@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the custom-op hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One timed "step" is the headline workload (cfg2): BinnedSelectKnn on one
+HGCal-like event of N=150,000 hits with 4-D coordinates and K=64 (bounding box,
+binning, stable sort into bin order, search, un-sort — everything the wrapper
+does), followed by the AccumulateKnn forward over F=64 features with the
+returned squared distances. Inputs are resident in HBM before the timed region.
+`value` is kNN queries per second of the whole step.
+
+The `roofline` object is measured in a second timed loop of the same run (also
+K iterations, HIP events on the stream the kernels are launched on):
+accumulate_knn forward + gradient at cfg4 (N=1,000,000, K=64, F=128, banded
+neighbour table), algorithmic bytes 4*N*(2K+4F) forward and 4*N*(3K+5F)
+gradient against the 8 TB/s HBM peak.
+
+`cpu_baseline` times the CPU oracle (a single-threaded C restatement of the
+reference CPU kernels) on this box's host: the binned kNN kernel over the full
+cfg2 event.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def event_ms(fn, steps, warmup):
+    """average milliseconds per call with HIP events on torch's current stream"""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(steps):
+        a = torch.cuda.Event(enable_timing=True)
+        b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b))
+    return float(np.mean(times)), float(np.median(times)), float(np.min(times))
+
+
+def cpu_baseline_knn(cfg):
+    """the oracle's binned kNN kernel over all queries of cfg2, one thread"""
+    import oracle
+    coords, rs, K = cfg["coords"], cfg["row_splits"], cfg["K"]
+    dbin, flat, nb, bw, nper = oracle.BinByCoordinates(coords[:, :3], rs, n_bins=cfg["n_bins"])
+    order = np.argsort(flat, kind="stable")
+    bb = np.concatenate([[0], np.cumsum(nper)]).astype(np.int32)
+    sc, sf, sd = coords[order], flat[order], dbin[order]
+    t0 = time.perf_counter()
+    oracle.binned_select_knn_kernel(K, sc, sf, sd, bb, nb, bw)
+    dt = time.perf_counter() - t0
+    return len(coords) / dt, dt
+
+
+def cpu_baseline_accumulate(cfg4_small):
+    import oracle
+    w = np.exp(-cfg4_small["distsq"]).astype(np.float32)
+    t0 = time.perf_counter()
+    _, arg = oracle.accumulate_knn_kernel(w, cfg4_small["features"], cfg4_small["indices"])
+    t1 = time.perf_counter()
+    oracle.accumulate_knn_grad_kernel(cfg4_small["grad_out"], w, cfg4_small["features"], cfg4_small["indices"], arg)
+    t2 = time.perf_counter()
+    return t1 - t0, t2 - t1
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--roofline-scale", type=float, default=1.0, help="shrink cfg4 (debugging only)")
+    ap.add_argument("--section", choices=["all", "headline", "roofline"], default="all",
+                    help="run only one part (for profiling); the JSON line is printed for 'all' only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build targets ONE GPU (no collectives, no sharding); run with --gpus 1. "
+                 "Events are independent, so several GPUs would each take whole events.")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    from hgcalml_amd import AccumulateKnn, AccumulateLinKnn, BinnedSelectKnn, BuildAndAssignCondensatesBinned, ops, workloads
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    # ------------------------------------------------------------------ headline: cfg2
+    c2 = workloads.cfg2()
+    n2, K2 = len(c2["coords"]), c2["K"]
+    if args.section != "roofline":
+        coords = torch.from_numpy(c2["coords"]).to(dev)
+        rs = torch.from_numpy(c2["row_splits"]).to(dev)
+        feat = torch.from_numpy(c2["features"]).to(dev)
+        state = {}
+
+        def step():
+            idx, dist = BinnedSelectKnn(K2, coords, rs, n_bins=c2["n_bins"])
+            out, _ = AccumulateKnn(dist, feat, idx)
+            state["idx"], state["dist"], state["out"] = idx, dist, out
+
+        log("bench: warmup + %d timed steps of cfg2 (kNN N=%d 4-D K=%d + accumulate fwd F=64)" % (args.steps, n2, K2))
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ms_per_step = wall / args.steps * 1e3
+        value = n2 / (ms_per_step * 1e-3)
+
+        knn_ms = event_ms(lambda: BinnedSelectKnn(K2, coords, rs, n_bins=c2["n_bins"]), args.steps, 2)
+        idx2, dist2 = state["idx"], state["dist"]
+        acc2_ms = event_ms(lambda: AccumulateKnn(dist2, feat, idx2), args.steps, 2)
+        log("bench: cfg2 step %.3f ms (kNN op %.3f ms, accumulate fwd %.3f ms)" % (ms_per_step, knn_ms[0], acc2_ms[0]))
+
+    if args.section == "headline":
+        return
+    # ------------------------------------------------------------------ roofline: cfg4 accumulate fwd + grad
+    log("bench: generating cfg4 (N=1M, K=64, F=128) ...")
+    c4 = workloads.cfg4(scale=args.roofline_scale)
+    n4, K4, F4 = len(c4["indices"]), c4["K"], c4["F"]
+    w4 = torch.exp(-torch.from_numpy(c4["distsq"]).to(dev))
+    x4 = torch.from_numpy(c4["features"]).to(dev)
+    i4 = torch.from_numpy(c4["indices"]).to(dev)
+    g4 = torch.from_numpy(c4["grad_out"]).to(dev)
+    # known-size device copy (512 MB read + 512 MB write): calibrates FETCH_SIZE / WRITE_SIZE
+    # when this run is profiled with hardware counters
+    copy_dst = torch.empty_like(x4)
+    copy_ms = event_ms(lambda: copy_dst.copy_(x4), 3, 1)
+    log("bench: calibration copy of %.0f MB: %.3f ms (%.0f GB/s read+write)" %
+        (x4.numel() * 4 / 1e6, copy_ms[0], 2 * x4.numel() * 4 / (copy_ms[0] * 1e-3) / 1e9))
+    del copy_dst
+    fwd_ms = event_ms(lambda: torch.ops.hgcalml.accumulate_knn_slots(w4, x4, i4, 0, True), args.steps, args.warmup)
+    _, arg4, slots4 = torch.ops.hgcalml.accumulate_knn_slots(w4, x4, i4, 0, True)
+    inv_ms = event_ms(lambda: ops.inverse_neighbour_index(i4), 3, 1)
+    inv = ops.inverse_neighbour_index(i4)
+    grad_ms = event_ms(lambda: torch.ops.hgcalml.accumulate_knn_grad_slots(g4, w4, x4, i4, arg4, slots4, *inv),
+                       args.steps, args.warmup)
+    bytes_fwd = 4.0 * n4 * (2 * K4 + 4 * F4)
+    bytes_bwd = 4.0 * n4 * (3 * K4 + 5 * F4)
+    achieved = (bytes_fwd + bytes_bwd) / ((fwd_ms[0] + grad_ms[0]) * 1e-3) / 1e9
+    log("bench: cfg4 fwd %.3f ms, grad %.3f ms, inverse index (one-off) %.3f ms -> %.1f GB/s" %
+        (fwd_ms[0], grad_ms[0], inv_ms[0], achieved))
+
+    if args.section == "roofline":
+        return
+    # ------------------------------------------------------------------ information: cfg3, cfg5
+    extra = {}
+    try:
+        c3 = workloads.cfg3()
+        co3, rs3 = torch.from_numpy(c3["coords"]).to(dev), torch.from_numpy(c3["row_splits"]).to(dev)
+        m3 = event_ms(lambda: BinnedSelectKnn(c3["K"], co3, rs3, n_bins=c3["n_bins"], max_radius=c3["max_radius"]), 5, 2)
+        extra["cfg3_knn_ms"] = round(m3[0], 3)
+        extra["cfg3_queries_per_s"] = round(len(c3["coords"]) / (m3[0] * 1e-3), 1)
+        c5 = workloads.cfg5()
+        a5 = [torch.from_numpy(c5[k]).to(dev) for k in ("ccoords", "betas", "dist", "row_splits")]
+        for mode in (True, False):
+            m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode), 5, 2)
+            extra["cfg5_condensates_ms_max_beta" if mode else "cfg5_condensates_ms_min_dist"] = round(m5[0], 3)
+    except Exception as e:  # information only; never hide the headline numbers
+        extra["info_error"] = repr(e)
+
+    # ------------------------------------------------------------------ CPU baseline
+    cpu = None
+    if not args.skip_cpu_baseline:
+        log("bench: CPU baseline (oracle, 1 thread): binned kNN kernel over cfg2 ...")
+        qps, secs = cpu_baseline_knn(c2)
+        small = workloads.cfg4(scale=0.02)
+        f_s, b_s = cpu_baseline_accumulate(small)
+        ns = len(small["indices"])
+        cpu = {"value": round(qps, 1), "unit": "queries/s", "cores": 1, "kind": "port",
+               "sample": "all %d queries of cfg2 through the oracle's binned_select_knn kernel (gcc -O2, one run, "
+                         "%.1f s); binning/sort glue not included" % (n2, secs),
+               "accumulate_fwd_grad_GBps": round((4.0 * ns * (2 * K4 + 4 * F4) + 4.0 * ns * (3 * K4 + 5 * F4)) /
+                                                 (f_s + b_s) / 1e9, 4),
+               "accumulate_sample": "cfg4 at N=%d (fwd %.2f s, grad %.2f s)" % (ns, f_s, b_s),
+               "host_cpus": os.cpu_count()}
+        log("bench: CPU oracle kNN %.0f queries/s (%.1f s)" % (qps, secs))
+
+    line = {
+        "metric": "kNN queries/s at N=150k,4D,K=64; accumulate_knn fwd+grad achieved HBM GB/s",
+        "value": round(value, 1),
+        "unit": "queries/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cfg2: one event, N=150000 hits, 4-D clusters+noise, BinnedSelectKnn K=64 "
+                               "(3 binned dims, n_bins=30) + AccumulateKnn forward F=64",
+                   "knn_op_ms": round(knn_ms[0], 4), "accumulate_fwd_ms": round(acc2_ms[0], 4)},
+        "accumulate_fwd_grad_GBps": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "accumulate_knn forward + gradient, cfg4 (N=%d, K=%d, F=%d)" % (n4, K4, F4),
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": bytes_fwd + bytes_bwd,
+                     "fwd_ms": round(fwd_ms[0], 4), "grad_ms": round(grad_ms[0], 4),
+                     "fwd_GBps": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9, 1),
+                     "grad_GBps": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9, 1),
+                     "inverse_index_build_ms": round(inv_ms[0], 3)},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    if cpu:
+        line["speedup_vs_cpu_kernel"] = round(n2 / (knn_ms[0] * 1e-3) / cpu["value"], 1)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -32,9 +32,11 @@ _SIGNATURES = {
     "hgc_binned_select_knn_fused": (_c_int, [_ptr] * 8 + [_c_float] + [_ptr] * 2 + [_c_int] * 7 + [_ptr]),
     "hgc_index_replacer": (_c_int, [_ptr, _ptr, _ptr, _c_int, _c_int, _ptr]),
     "hgc_accumulate_knn": (_c_int, [_ptr] * 5 + [_c_int] * 6 + [_ptr]),
+    "hgc_accumulate_knn_slots": (_c_int, [_ptr] * 6 + [_c_int] * 6 + [_ptr]),
     "hgc_inverse_neighbour_index_workspace_bytes": (_c_size, [_c_int, _c_int]),
     "hgc_inverse_neighbour_index": (_c_int, [_ptr, _c_int, _c_int, _ptr, _ptr, _ptr, _c_size, _ptr]),
     "hgc_accumulate_knn_grad": (_c_int, [_ptr] * 9 + [_c_int] * 6 + [_ptr]),
+    "hgc_accumulate_knn_grad_slots": (_c_int, [_ptr] * 10 + [_c_int] * 6 + [_ptr]),
     "hgc_binned_assign_to_condensates_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
     "hgc_binned_assign_to_condensates": (_c_int, [_c_int, _c_int] + [_ptr] * 21 + [_c_int] * 4 + [_ptr, _ptr, _c_size, _ptr]),
 }

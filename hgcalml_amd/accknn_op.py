@@ -16,18 +16,18 @@ class _AccumulateFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, weights, features, indices, mean_and_max):
-        out, maxidx = torch.ops.hgcalml.accumulate_knn(weights, features, indices, 0, mean_and_max)
-        ctx.save_for_backward(weights, features, indices, maxidx)
+        out, maxidx, slots = torch.ops.hgcalml.accumulate_knn_slots(weights, features, indices, 0, mean_and_max)
+        ctx.save_for_backward(weights, features, indices, maxidx, slots)
         ctx.indices_ref = indices
         ctx.mark_non_differentiable(maxidx)
         return out, maxidx
 
     @staticmethod
     def backward(ctx, grad_out, _grad_maxidx):
-        weights, features, indices, maxidx = ctx.saved_tensors
+        weights, features, indices, maxidx, slots = ctx.saved_tensors
         inv_off, inv_slots = ops.cached_inverse_neighbour_index(ctx.indices_ref)
-        gw, gx = torch.ops.hgcalml.accumulate_knn_grad(grad_out.contiguous(), weights, features, indices, maxidx,
-                                                       inv_off, inv_slots)
+        gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(grad_out.contiguous(), weights, features, indices,
+                                                             maxidx, slots, inv_off, inv_slots)
         return gw, gx, None, None
 
 

@@ -45,9 +45,15 @@ def _compile(src):
 
 
 def build(verbose=True, sources=None):
+    """Compile `sources` (default: all) and link every object into the library."""
     sources = sources or SOURCES
     with ThreadPoolExecutor(max_workers=min(4, len(sources))) as pool:
-        objs = list(pool.map(_compile, sources))
+        list(pool.map(_compile, sources))
+    objs = [os.path.join(CSRC, os.path.splitext(src)[0] + ".o") for src in SOURCES]
+    missing = [o for o in objs if not os.path.exists(o)]
+    if missing:
+        with ThreadPoolExecutor(max_workers=4) as pool:
+            list(pool.map(_compile, [os.path.basename(o)[:-2] + ".hip" for o in missing]))
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:

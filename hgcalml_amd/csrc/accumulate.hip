@@ -47,6 +47,22 @@ __device__ __forceinline__ void load_vec(const float *p, float (&x)[VEC]) {
     if constexpr (VEC == 4) {
         const float4 v = *reinterpret_cast<const float4 *>(p);
         x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    } else if constexpr (VEC == 2) {
+        const float2 v = *reinterpret_cast<const float2 *>(p);
+        x[0] = v.x; x[1] = v.y;
+    } else {
+        x[0] = *p;
+    }
+}
+
+template <int VEC>
+__device__ __forceinline__ void load_vec_i(const int *p, int (&x)[VEC]) {
+    if constexpr (VEC == 4) {
+        const int4 v = *reinterpret_cast<const int4 *>(p);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    } else if constexpr (VEC == 2) {
+        const int2 v = *reinterpret_cast<const int2 *>(p);
+        x[0] = v.x; x[1] = v.y;
     } else {
         x[0] = *p;
     }
@@ -56,6 +72,8 @@ template <int VEC>
 __device__ __forceinline__ void store_vec(float *p, const float (&x)[VEC]) {
     if constexpr (VEC == 4) {
         *reinterpret_cast<float4 *>(p) = make_float4(x[0], x[1], x[2], x[3]);
+    } else if constexpr (VEC == 2) {
+        *reinterpret_cast<float2 *>(p) = make_float2(x[0], x[1]);
     } else {
         *p = x[0];
     }
@@ -65,6 +83,8 @@ template <int VEC>
 __device__ __forceinline__ void store_vec_i(int *p, const int (&x)[VEC]) {
     if constexpr (VEC == 4) {
         *reinterpret_cast<int4 *>(p) = make_int4(x[0], x[1], x[2], x[3]);
+    } else if constexpr (VEC == 2) {
+        *reinterpret_cast<int2 *>(p) = make_int2(x[0], x[1]);
     } else {
         *p = x[0];
     }
@@ -77,8 +97,9 @@ constexpr int kUnroll = 8;
 template <int VEC, bool MAX>
 __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__restrict__ w, const float *__restrict__ feat,
                                                              const int *__restrict__ idx, float *__restrict__ out,
-                                                             int *__restrict__ out_maxidx, int n_vert, int K, int F,
-                                                             int out_cols) {
+                                                             int *__restrict__ out_maxidx,
+                                                             unsigned char *__restrict__ out_maxslot, int n_vert, int K,
+                                                             int F, int out_cols) {
     const int tpv = F / VEC;  // threads per vertex
     const long long t = (long long)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
     const int v = (int)(t / tpv);
@@ -88,12 +109,13 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
     const int *irow = idx + (size_t)v * K;
     const float *wrow = w + (size_t)v * K;
     float sum[VEC], best[VEC];
-    int arg[VEC];
+    int arg[VEC], aslot[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
         sum[e] = 0.f;
         best[e] = 0.f;
         arg[e] = 0;
+        aslot[e] = -1;
     }
 
     for (int n0 = 0; n0 < K; n0 += kUnroll) {
@@ -124,6 +146,7 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
                     const bool take = ok && (wf >= best[e] || first);
                     best[e] = take ? wf : best[e];
                     arg[e] = take ? j[u] : arg[e];
+                    aslot[e] = take ? n0 + u : aslot[e];
                 }
             }
         }
@@ -137,6 +160,449 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
     if (MAX) {
         store_vec<VEC>(out + (size_t)v * out_cols + F + f0, best);
         store_vec_i<VEC>(out_maxidx + (size_t)v * F + f0, arg);
+        if (out_maxslot) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                int sl = aslot[e];
+                if (sl > 0 && arg[e] == v) {  // repeated self reference: report its first slot
+                    for (int n = 0; n < sl; ++n)
+                        if (irow[n] == v) {
+                            sl = n;
+                            break;
+                        }
+                }
+                out_maxslot[(size_t)v * F + f0 + e] = (unsigned char)(sl < 0 ? 255 : sl);
+            }
+        }
+    }
+}
+
+
+// ================================================================== wave-per-vertex kernels (F >= 64)
+//
+// One wave64 owns one vertex; lane l owns features [l*VEC, l*VEC+VEC) of every
+// block of 64*VEC features. The vertex index is wave-uniform, so the neighbour
+// indices and weights of its row come in through scalar loads, and gathered
+// rows are fetched with buffer loads whose address is
+//   descriptor base + scalar row offset + per-lane column offset,
+// i.e. no vector ALU is spent on addressing and the hardware range-checks every
+// access against the size of the matrix. Chunks of U neighbour slots without
+// padding take a branch-free path with all U row loads in flight.
+
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int wave_vertex() {
+    const int tile = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    return __builtin_amdgcn_readfirstlane(tile * 4 + (int)(threadIdx.x >> 6));
+}
+
+// A dense [rows, cols] matrix of 4-byte elements seen through a raw buffer
+// descriptor (stride 0, num_records = size in bytes, gfx9 data format word).
+struct RowMatrix {
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t row_bytes;
+    __device__ __forceinline__ RowMatrix(const void *base, size_t rows, size_t cols)
+        : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)(uint32_t)(rows * cols * 4u),
+                                                 0x00020000)),
+          row_bytes((uint32_t)cols * 4u) {}
+
+    // x[0..VEC) = M[row, col .. col+VEC) with col = lane_bytes/4 (+ col_bytes/4)
+    template <int VEC>
+    __device__ __forceinline__ void load(int row, uint32_t lane_bytes, uint32_t (&x)[VEC]) const {
+        const int soff = (int)((uint32_t)row * row_bytes);
+        if constexpr (VEC == 4) {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_bytes, soff, 0);
+            x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+        } else if constexpr (VEC == 2) {
+            const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_bytes, soff, 0);
+            x[0] = v.x; x[1] = v.y;
+        } else {
+            x[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_bytes, soff, 0);
+        }
+    }
+    template <int VEC>
+    __device__ __forceinline__ void load(int row, uint32_t lane_bytes, float (&x)[VEC]) const {
+        uint32_t r[VEC];
+        load<VEC>(row, lane_bytes, r);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[e] = __uint_as_float(r[e]);
+    }
+    template <int VEC>
+    __device__ __forceinline__ void load(int row, uint32_t lane_bytes, int (&x)[VEC]) const {
+        uint32_t r[VEC];
+        load<VEC>(row, lane_bytes, r);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[e] = (int)r[e];
+    }
+};
+
+// one slot of the forward recurrence for the VEC features of this lane
+template <int VEC, bool MAX, bool SEED>
+__device__ __forceinline__ void fwd_slot(const float (&x)[VEC], float wn, int slot, float (&sum)[VEC],
+                                         float (&best)[VEC], int (&arg)[VEC]) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        const float wf = x[e] * wn;
+        sum[e] = sum[e] + wf;
+        if (MAX) {
+            if (SEED) {  // slot 0 always seeds the maximum
+                best[e] = wf;
+                arg[e] = slot;
+            } else {
+                const bool take = wf >= best[e];  // ">=": a later slot wins ties
+                best[e] = take ? wf : best[e];
+                arg[e] = take ? slot : arg[e];
+            }
+        }
+    }
+}
+
+template <int VEC, bool MAX>
+__global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *__restrict__ w,
+                                                                  const float *__restrict__ feat,
+                                                                  const int *__restrict__ idx, float *__restrict__ out,
+                                                                  int *__restrict__ out_maxidx,
+                                                                  unsigned char *__restrict__ out_maxslot, int n_vert,
+                                                                  int K, int F, int out_cols) {
+    constexpr int U = VEC == 4 ? 8 : 16;
+    const int v = wave_vertex();
+    if (v >= n_vert) return;
+    const int *irow = idx + (size_t)v * K;
+    const float *wrow = w + (size_t)v * K;
+    const float kf = (float)K;
+    const RowMatrix X(feat, n_vert, F);
+    int first_self = -1;  // first slot that names the vertex itself (wave-uniform)
+    if (MAX && out_maxslot) {
+        for (int n = K - 1; n >= 0; --n)
+            if (irow[n] == v) first_self = n;
+    }
+
+    for (int fb = lane_id() * VEC; fb < F; fb += kWave * VEC) {
+        const uint32_t lane_bytes = (uint32_t)fb * 4u;
+        float sum[VEC], best[VEC];
+        int arg[VEC];  // SLOT of the maximum, -1: none (translated to an index at the end)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            sum[e] = 0.f;
+            best[e] = 0.f;
+            arg[e] = -1;
+        }
+        int n0 = 0;
+        for (; n0 + U <= K; n0 += U) {
+            int j[U];
+            float wn[U];
+            float x[U][VEC];
+            bool all_valid = true;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                j[u] = irow[n0 + u];
+                wn[u] = wrow[n0 + u];
+                all_valid = all_valid && (unsigned)j[u] < (unsigned)n_vert;
+            }
+            if (all_valid) {  // wave-uniform: the common, padding-free chunk
+#pragma unroll
+                for (int u = 0; u < U; ++u) X.load<VEC>(j[u], lane_bytes, x[u]);
+                if (n0 == 0) {
+                    fwd_slot<VEC, MAX, true>(x[0], wn[0], 0, sum, best, arg);
+#pragma unroll
+                    for (int u = 1; u < U; ++u) fwd_slot<VEC, MAX, false>(x[u], wn[u], u, sum, best, arg);
+                } else {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) fwd_slot<VEC, MAX, false>(x[u], wn[u], n0 + u, sum, best, arg);
+                }
+            } else {
+                for (int u = 0; u < U; ++u) {
+                    const int jj = irow[n0 + u];
+                    if ((unsigned)jj >= (unsigned)n_vert) continue;
+                    float xs[VEC];
+                    X.load<VEC>(jj, lane_bytes, xs);
+                    if (n0 + u == 0)
+                        fwd_slot<VEC, MAX, true>(xs, wrow[0], 0, sum, best, arg);
+                    else
+                        fwd_slot<VEC, MAX, false>(xs, wrow[n0 + u], n0 + u, sum, best, arg);
+                }
+            }
+        }
+        for (; n0 < K; ++n0) {  // K not a multiple of U
+            const int jj = irow[n0];
+            if ((unsigned)jj >= (unsigned)n_vert) continue;
+            float xs[VEC];
+            X.load<VEC>(jj, lane_bytes, xs);
+            if (n0 == 0)
+                fwd_slot<VEC, MAX, true>(xs, wrow[0], 0, sum, best, arg);
+            else
+                fwd_slot<VEC, MAX, false>(xs, wrow[n0], n0, sum, best, arg);
+        }
+        float mean[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) mean[e] = sum[e] / kf;
+        store_vec<VEC>(out + (size_t)v * out_cols + fb, mean);
+        if (MAX) {
+            store_vec<VEC>(out + (size_t)v * out_cols + F + fb, best);
+            int argidx[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) argidx[e] = arg[e] < 0 ? 0 : irow[arg[e]];
+            store_vec_i<VEC>(out_maxidx + (size_t)v * F + fb, argidx);
+            if (out_maxslot) {
+                // slot of the maximum; for a repeated self reference its first slot,
+                // which is the one the reference's gradient credits
+                uint32_t packed = 0;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    int sl = arg[e];
+                    if (sl >= 0 && argidx[e] == v) sl = first_self;
+                    packed |= (uint32_t)(sl < 0 ? 255 : sl) << (8 * e);
+                }
+                unsigned char *dst = out_maxslot + (size_t)v * F + fb;
+                if constexpr (VEC == 4) *reinterpret_cast<uint32_t *>(dst) = packed;
+                else if constexpr (VEC == 2) *reinterpret_cast<uint16_t *>(dst) = (uint16_t)packed;
+                else *dst = (unsigned char)packed;
+            }
+        }
+    }
+}
+
+// x / K for 0 <= x < 2^31 without an integer divide
+struct FastDiv {
+    uint32_t magic;  // 0: K is a power of two
+    int shift;
+};
+
+__device__ __forceinline__ int fast_div(int x, const FastDiv d) {
+    return d.magic == 0 ? (int)((uint32_t)x >> d.shift) : (int)(__umulhi((uint32_t)x, d.magic) >> d.shift);
+}
+
+// one inverse-list entry of the feature gradient for the VEC features of this lane;
+// `mi` holds arg-max indices compared with `key` = target vertex, or (SLOTS)
+// arg-max slots compared with `key` = slot of this entry
+template <int VEC, bool MAX, bool POW2K>
+__device__ __forceinline__ void fgrad_entry(const float (&gm)[VEC], const float (&gx)[VEC], const int (&mi)[VEC],
+                                            float wv, int key, bool count_max, float kf, float inv_k,
+                                            float (&acc)[VEC]) {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        float part = POW2K ? gm[e] * inv_k : gm[e] / kf;
+        part = part * wv;
+        float part_max = 0.f;
+        if (MAX) {
+            const float pmx = gx[e] * wv;
+            part_max = (mi[e] == key && count_max) ? pmx : 0.f;
+        }
+        const float add = part + part_max;
+        acc[e] = acc[e] + add;
+    }
+}
+
+// VEC arg-max slot bytes of row `row`, columns lane_col .. lane_col+VEC
+template <int VEC>
+__device__ __forceinline__ void load_slots(__amdgpu_buffer_rsrc_t rsrc, int row, uint32_t row_bytes, uint32_t lane_col,
+                                           int (&x)[VEC]) {
+    const int soff = (int)((uint32_t)row * row_bytes);
+    uint32_t packed;
+    if constexpr (VEC == 4) packed = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_col, soff, 0);
+    else if constexpr (VEC == 2) packed = __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int)lane_col, soff, 0);
+    else packed = __builtin_amdgcn_raw_buffer_load_b8(rsrc, (int)lane_col, soff, 0);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) x[e] = (int)((packed >> (8 * e)) & 255u);
+}
+
+// Feature slicing across XCDs: the rows this kernel gathers (gradient row +
+// arg-max row of every vertex that names the target) span a window of the
+// neighbour band times ~1.5 KB, more than one XCD's 4 MB L2 holds. With
+// n_slices == 2 even XCDs work on the even 64*VEC-feature blocks of every row
+// and odd XCDs on the odd ones, so each L2 caches only half of every row.
+// (Workgroups are dealt round-robin to the 8 XCDs; a different dispatch order
+// would only cost speed, not correctness.)
+template <int VEC, bool MAX, bool POW2K, bool SLOTS>
+__global__ __launch_bounds__(256) void feature_grad_wave_kernel(const float *__restrict__ g, const float *__restrict__ w,
+                                                                const int *__restrict__ maxidx,
+                                                                const unsigned char *__restrict__ maxslot,
+                                                                const int *__restrict__ inv_off,
+                                                                const int *__restrict__ inv_slots,
+                                                                float *__restrict__ gfeat, int n_vert, int K, int F,
+                                                                int g_cols, const FastDiv div_k, int n_slices) {
+    constexpr int U = VEC == 4 ? 4 : 8;
+    int m, first_block = 0;
+    if (n_slices == 1) {
+        m = wave_vertex();
+    } else {
+        const int xcd = blockIdx.x % kNumXcd, seq = blockIdx.x / kNumXcd;
+        const int per_xcd = gridDim.x / kNumXcd;
+        first_block = xcd % n_slices;
+        const int tile = (xcd / n_slices) * per_xcd + seq;
+        m = __builtin_amdgcn_readfirstlane(tile * 4 + (int)(threadIdx.x >> 6));
+    }
+    if (m >= n_vert) return;
+    const float kf = (float)K;
+    const float inv_k = 1.f / kf;  // exact when K is a power of two
+    const int begin = inv_off[m], end = inv_off[m + 1];
+    const RowMatrix G(g, n_vert, g_cols);
+    const RowMatrix MI(maxidx, (MAX && !SLOTS) ? n_vert : 0, F);
+    const __amdgpu_buffer_rsrc_t MS = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<unsigned char *>(maxslot), 0, (MAX && SLOTS) ? (int)(uint32_t)((size_t)n_vert * F) : 0, 0x00020000);
+    const uint32_t max_col_bytes = (uint32_t)F * 4u;
+
+    for (int fb = (first_block * kWave + lane_id()) * VEC; fb < F; fb += n_slices * kWave * VEC) {
+        const uint32_t lane_bytes = (uint32_t)fb * 4u;
+        float acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+        bool self_seen = false;  // repeated self references carry the max part once
+        int e0 = begin;
+        for (; e0 + U <= end; e0 += U) {
+            int v[U], key[U];
+            float wv[U];
+            float gm[U][VEC], gx[U][VEC];
+            int mi[U][VEC];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int slot = inv_slots[e0 + u];
+                v[u] = fast_div(slot, div_k);
+                key[u] = SLOTS ? slot - v[u] * K : m;
+                wv[u] = w[slot];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                G.load<VEC>(v[u], lane_bytes, gm[u]);
+                if (MAX) {
+                    if (SLOTS) {
+                        load_slots<VEC>(MS, v[u], (uint32_t)F, (uint32_t)fb, mi[u]);
+                    } else {
+                        MI.load<VEC>(v[u], lane_bytes, mi[u]);
+                        G.load<VEC>(v[u], lane_bytes + max_col_bytes, gx[u]);
+                    }
+                }
+            }
+            if (MAX && SLOTS) {
+                // the max half of a gradient row is fetched only by the lanes whose
+                // feature has its maximum at this entry (about F/K lanes per row)
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    bool any = false;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        any = any || mi[u][e] == key[u];
+                        gx[u][e] = 0.f;
+                    }
+                    if (any) G.load<VEC>(v[u], lane_bytes + max_col_bytes, gx[u]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                bool count_max = true;
+                if (!SLOTS && v[u] == m) {  // (the slot table already points at the first self slot)
+                    count_max = !self_seen;
+                    self_seen = true;
+                }
+                fgrad_entry<VEC, MAX, POW2K>(gm[u], gx[u], mi[u], wv[u], key[u], count_max, kf, inv_k, acc);
+            }
+        }
+        for (; e0 < end; ++e0) {
+            const int slot = inv_slots[e0];
+            const int vv = fast_div(slot, div_k);
+            const int key = SLOTS ? slot - vv * K : m;
+            float gm[VEC], gx[VEC];
+            int mi[VEC];
+            G.load<VEC>(vv, lane_bytes, gm);
+            if (MAX) {
+                if (SLOTS)
+                    load_slots<VEC>(MS, vv, (uint32_t)F, (uint32_t)fb, mi);
+                else
+                    MI.load<VEC>(vv, lane_bytes, mi);
+                G.load<VEC>(vv, lane_bytes + max_col_bytes, gx);
+            }
+            bool count_max = true;
+            if (!SLOTS && vv == m) {
+                count_max = !self_seen;
+                self_seen = true;
+            }
+            fgrad_entry<VEC, MAX, POW2K>(gm, gx, mi, w[slot], key, count_max, kf, inv_k, acc);
+        }
+        store_vec<VEC>(gfeat + (size_t)m * F + fb, acc);
+    }
+}
+
+// After the call lane L holds the sum over all 64 lanes of value index L.
+__device__ __forceinline__ float transpose_reduce_64(float (&val)[64]) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int h = 32; h >= 1; h >>= 1) {
+        const bool upper = (lane & h) != 0;
+#pragma unroll
+        for (int i = 0; i < h; ++i) {
+            const float a = val[i], b = val[i + h];
+            const float send = upper ? a : b;
+            const float keep = upper ? b : a;
+            val[i] = keep + __shfl_xor(send, h, kWave);
+        }
+    }
+    return val[0];
+}
+
+template <int VEC, bool MAX>
+__global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__restrict__ g, const float *__restrict__ feat,
+                                                               const int *__restrict__ maxidx, const int *__restrict__ idx,
+                                                               float *__restrict__ gw, int n_vert, int K, int F,
+                                                               int g_cols) {
+    constexpr int U = 8;
+    constexpr int G = 32;  // slots per reduction group: 32 mean sums + 32 max sums = 64 values
+    const int m = wave_vertex();
+    if (m >= n_vert) return;
+    const int lane = lane_id();
+    const int *irow = idx + (size_t)m * K;
+    const double inv_k = 1.0 / (double)(float)K;
+    const RowMatrix X(feat, n_vert, F);
+
+    for (int l0 = 0; l0 < K; l0 += G) {
+        float val[64];
+#pragma unroll
+        for (int i = 0; i < 64; ++i) val[i] = 0.f;
+        for (int fb = lane * VEC; fb < F; fb += kWave * VEC) {
+            const uint32_t lane_bytes = (uint32_t)fb * 4u;
+            float gm[VEC], gx[VEC];
+            int mi[VEC];
+            load_vec<VEC>(g + (size_t)m * g_cols + fb, gm);
+            if (MAX) {
+                load_vec<VEC>(g + (size_t)m * g_cols + F + fb, gx);
+                load_vec_i<VEC>(maxidx + (size_t)m * F + fb, mi);
+            }
+#pragma unroll
+            for (int u0 = 0; u0 < G; u0 += U) {
+                int j[U];
+                float x[U][VEC];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int l = l0 + u0 + u;
+                    j[u] = l < K ? irow[l] : -1;
+                }
+                // rows outside [0, n_vert) read as zeros (hardware range check) and
+                // can never equal an arg-max index of a valid row; their result is
+                // overwritten with 0 below
+#pragma unroll
+                for (int u = 0; u < U; ++u) X.load<VEC>(j[u], lane_bytes, x[u]);
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        val[u0 + u] = __builtin_fmaf(gm[e], x[u][e], val[u0 + u]);
+                        if (MAX) {
+                            const float t = __builtin_fmaf(gx[e], x[u][e], val[G + u0 + u]);
+                            val[G + u0 + u] = (mi[e] == j[u]) ? t : val[G + u0 + u];
+                        }
+                    }
+                }
+            }
+        }
+        const float r = transpose_reduce_64(val);        // lane < 32: mean sum of slot l0+lane; else max sum
+        const float r_max = __shfl_xor(r, 32, kWave);    // lane < 32 receives its max sum
+        const int l = l0 + lane;
+        if (lane < G && l < K) {
+            const int j = irow[l];
+            const bool ok = (unsigned)j < (unsigned)n_vert;
+            const float mean = (float)((double)r * inv_k);
+            gw[(size_t)m * K + l] = ok ? mean + r_max : 0.f;
+        }
     }
 }
 
@@ -340,6 +806,29 @@ int inverse_key_bits(int n_vert) {
 
 bool is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
 
+// features per lane of the wave-per-vertex kernels: all 64 lanes busy and
+// every access naturally aligned
+int wave_vec(int n_feat, uintptr_t align_or) {
+    if (n_feat % 256 == 0 && (align_or & 15u) == 0) return 4;
+    if (n_feat % 128 == 0 && (align_or & 7u) == 0) return 2;
+    return 1;
+}
+
+FastDiv make_fast_div(int k) {
+    FastDiv d;
+    if (is_pow2(k)) {
+        d.magic = 0;
+        d.shift = 0;
+        while ((1 << d.shift) < k) ++d.shift;
+        return d;
+    }
+    int s = 0;
+    while ((1ll << s) < k) ++s;  // ceil(log2 k) >= 2
+    d.magic = (uint32_t)((1ull << (31 + s)) / (uint32_t)k + 1);
+    d.shift = s - 1;
+    return d;
+}
+
 }  // namespace
 }  // namespace hgc
 
@@ -347,8 +836,8 @@ using namespace hgc;
 
 extern "C" {
 
-int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
-                       int *d_out_maxidxs, int n_vert, int n_neigh, int n_feat, int n_out_feat, int n_moments,
+int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
+                             int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat, int n_out_feat, int n_moments,
                        int mean_and_max, hgc_stream_t stream) {
     (void)n_moments;  // carried by the reference op, never used by its kernels
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
@@ -357,27 +846,52 @@ int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int 
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_distances && d_feat && d_idxs && d_out_feat, "null pointer");
     HGC_REQUIRE(!mean_and_max || d_out_maxidxs, "mean_and_max needs d_out_maxidxs");
+    HGC_REQUIRE(!d_out_maxslots || n_neigh <= 254, "arg-max slots are bytes: n_neigh <= 254");
     hipStream_t s = as_stream(stream);
-    const bool vec4 = (n_feat % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_feat) | reinterpret_cast<uintptr_t>(d_out_feat) |
-                                             reinterpret_cast<uintptr_t>(d_out_maxidxs)) & 15u) == 0;
+    const uintptr_t align_or = reinterpret_cast<uintptr_t>(d_feat) | reinterpret_cast<uintptr_t>(d_out_feat) |
+                              reinterpret_cast<uintptr_t>(d_out_maxidxs);
+    // the wave kernels address rows through 32-bit buffer offsets
+    const bool fits_32bit = (unsigned long long)n_vert * (unsigned long long)n_out_feat * 4ull < (1ull << 32);
+    if (n_feat >= kWave && fits_32bit) {  // one wave per vertex
+        const int vec = wave_vec(n_feat, align_or);
+        const dim3 grid(ceil_div(n_vert, 4)), block(256);
+#define HGC_FWD(VEC, MAX)                                                                                         \
+    accumulate_fwd_wave_kernel<VEC, MAX><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, \
+                                                               d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat)
+        if (mean_and_max) {
+            if (vec == 4) HGC_FWD(4, true); else if (vec == 2) HGC_FWD(2, true); else HGC_FWD(1, true);
+        } else {
+            if (vec == 4) HGC_FWD(4, false); else if (vec == 2) HGC_FWD(2, false); else HGC_FWD(1, false);
+        }
+#undef HGC_FWD
+        return check_launch("accumulate_fwd_wave_kernel");
+    }
+    const bool vec4 = (n_feat % 4 == 0) && (align_or & 15u) == 0;
     const long long threads = (long long)n_vert * (vec4 ? n_feat / 4 : n_feat);
     const dim3 grid(ceil_div(threads, 256)), block(256);
     if (vec4) {
         if (mean_and_max)
             accumulate_fwd_kernel<4, true><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                  n_vert, n_neigh, n_feat, n_out_feat);
+                                                                  d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
         else
             accumulate_fwd_kernel<4, false><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                   n_vert, n_neigh, n_feat, n_out_feat);
+                                                                   d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
     } else {
         if (mean_and_max)
             accumulate_fwd_kernel<1, true><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                  n_vert, n_neigh, n_feat, n_out_feat);
+                                                                  d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
         else
             accumulate_fwd_kernel<1, false><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                   n_vert, n_neigh, n_feat, n_out_feat);
+                                                                   d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
     }
     return check_launch("accumulate_fwd_kernel");
+}
+
+int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
+                       int *d_out_maxidxs, int n_vert, int n_neigh, int n_feat, int n_out_feat, int n_moments,
+                       int mean_and_max, hgc_stream_t stream) {
+    return hgc_accumulate_knn_slots(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, nullptr, n_vert, n_neigh,
+                                    n_feat, n_out_feat, n_moments, mean_and_max, stream);
 }
 
 size_t hgc_inverse_neighbour_index_workspace_bytes(int n_vert, int n_neigh) {
@@ -417,11 +931,12 @@ int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh, int 
     return check_launch("inverse_offsets");
 }
 
-int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
-                            const int *d_max_feat_indices, const int *d_neigh_indices, const int *d_inv_offsets,
-                            const int *d_inv_slots, float *d_out_grad_distances, float *d_out_grad_features,
-                            int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat, int n_moments,
-                            int mean_and_max, hgc_stream_t stream) {
+int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
+                                  const int *d_max_feat_indices, const unsigned char *d_max_slots,
+                                  const int *d_neigh_indices, const int *d_inv_offsets, const int *d_inv_slots,
+                                  float *d_out_grad_distances, float *d_out_grad_features, int n_vert, int n_neigh,
+                                  int n_feat, int n_grad_from_out_feat, int n_moments, int mean_and_max,
+                                  hgc_stream_t stream) {
     (void)n_moments;
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_grad_from_out_feat == n_feat * (mean_and_max ? 2 : 1),
@@ -436,8 +951,48 @@ int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *
     const uintptr_t align_or = reinterpret_cast<uintptr_t>(d_grad_from_out_features) | reinterpret_cast<uintptr_t>(d_feat) |
                                reinterpret_cast<uintptr_t>(d_max_feat_indices) |
                                reinterpret_cast<uintptr_t>(d_out_grad_features);
-    const bool vec4 = (n_feat % 4 == 0) && (align_or & 15u) == 0;
     const bool pow2k = is_pow2(n_neigh);
+
+    const bool fits_32bit = (unsigned long long)n_vert * (unsigned long long)(2 * n_feat) * 4ull < (1ull << 32);
+    if (n_feat >= kWave && fits_32bit) {  // one wave per vertex, rows addressed through 32-bit buffer offsets
+        const int vec = wave_vec(n_feat, align_or);
+        const dim3 grid(ceil_div(n_vert, 4)), block(256);
+        const FastDiv div_k = make_fast_div(n_neigh);
+#define HGC_FGW(VEC, MAX, P2, SL)                                                                                      \
+    feature_grad_wave_kernel<VEC, MAX, P2, SL><<<fg_grid, block, 0, s>>>(                                              \
+        d_grad_from_out_features, d_distances, d_max_feat_indices, d_max_slots, d_inv_offsets, d_inv_slots,            \
+        d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat, div_k, n_slices)
+#define HGC_FGW_V(VEC)                                                                                   \
+    do {                                                                                                 \
+        if (mean_and_max && use_slots) { if (pow2k) HGC_FGW(VEC, true, true, true); else HGC_FGW(VEC, true, false, true); } \
+        else if (mean_and_max) { if (pow2k) HGC_FGW(VEC, true, true, false); else HGC_FGW(VEC, true, false, false); } \
+        else { if (pow2k) HGC_FGW(VEC, false, true, false); else HGC_FGW(VEC, false, false, false); }       \
+    } while (0)
+        const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
+        // two feature slices as soon as a row has two or more 64-feature blocks
+        const int n_slices = n_feat >= 2 * kWave ? 2 : 1;
+        const int fg_vec = n_slices == 1 ? vec : wave_vec(n_feat / 2, align_or);
+        const int tiles = ceil_div(n_vert, 4);
+        const dim3 fg_grid(n_slices == 1 ? tiles : kNumXcd * ceil_div(tiles, kNumXcd / n_slices));
+        if (fg_vec == 4) HGC_FGW_V(4); else if (fg_vec == 2) HGC_FGW_V(2); else HGC_FGW_V(1);
+#undef HGC_FGW_V
+#undef HGC_FGW
+        int rc = check_launch("feature_grad_wave_kernel");
+        if (rc) return rc;
+#define HGC_WGW(VEC, MAX)                                                                                       \
+    weight_grad_wave_kernel<VEC, MAX><<<grid, block, 0, s>>>(d_grad_from_out_features, d_feat, d_max_feat_indices, \
+                                                            d_neigh_indices, d_out_grad_distances, n_vert, n_neigh, \
+                                                            n_feat, n_grad_from_out_feat)
+        if (mean_and_max) {
+            if (vec == 4) HGC_WGW(4, true); else if (vec == 2) HGC_WGW(2, true); else HGC_WGW(1, true);
+        } else {
+            if (vec == 4) HGC_WGW(4, false); else if (vec == 2) HGC_WGW(2, false); else HGC_WGW(1, false);
+        }
+#undef HGC_WGW
+        return check_launch("weight_grad_wave_kernel");
+    }
+
+    const bool vec4 = (n_feat % 4 == 0) && (align_or & 15u) == 0;
 
     // ---- feature gradient ----
     {
@@ -488,6 +1043,17 @@ int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *
         }
         return check_launch("weight_grad_kernel");
     }
+}
+
+int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
+                            const int *d_max_feat_indices, const int *d_neigh_indices, const int *d_inv_offsets,
+                            const int *d_inv_slots, float *d_out_grad_distances, float *d_out_grad_features,
+                            int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat, int n_moments,
+                            int mean_and_max, hgc_stream_t stream) {
+    return hgc_accumulate_knn_grad_slots(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices, nullptr,
+                                         d_neigh_indices, d_inv_offsets, d_inv_slots, d_out_grad_distances,
+                                         d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat, n_moments,
+                                         mean_and_max, stream);
 }
 
 }  // extern "C"

@@ -146,10 +146,7 @@ def index_replacer(to_be_replaced: torch.Tensor, replacements: torch.Tensor) -> 
 
 # --------------------------------------------------------------------------- accumulate
 
-@torch.library.custom_op("hgcalml::accumulate_knn", mutates_args=())
-def accumulate_knn(distances: torch.Tensor, features: torch.Tensor, indices: torch.Tensor, n_moments: int,
-                   mean_and_max: bool) -> tuple[torch.Tensor, torch.Tensor]:
-    """modules/compiled/accumulate_knn_module.cc:7-14 (`distances` are the weights)"""
+def _accumulate_forward(distances, features, indices, n_moments, mean_and_max, with_slots):
     dev = require_device(distances, features, indices)
     w, x, idx = f32(distances), f32(features), i32(indices)
     # modules/compiled/accumulate_knn_kernel.cc:107-111
@@ -163,9 +160,32 @@ def accumulate_knn(distances: torch.Tensor, features: torch.Tensor, indices: tor
     out = torch.empty((n, 2 * f if mean_and_max else f), dtype=torch.float32, device=dev)
     maxidx = torch.empty((n, f), dtype=torch.int32, device=dev) if mean_and_max else \
         torch.zeros((n, f), dtype=torch.int32, device=dev)
-    check(lib.hgc_accumulate_knn(p(w), p(x), p(idx), p(out), p(maxidx), n, k, f, out.shape[1], int(n_moments),
-                                 int(mean_and_max), stream()))
+    slots = None
+    if with_slots and mean_and_max and k <= 254:
+        slots = torch.empty((n, f), dtype=torch.uint8, device=dev)
+    check(lib.hgc_accumulate_knn_slots(p(w), p(x), p(idx), p(out), p(maxidx), p(slots), n, k, f, out.shape[1],
+                                       int(n_moments), int(mean_and_max), stream()))
+    return out, maxidx, slots
+
+
+@torch.library.custom_op("hgcalml::accumulate_knn", mutates_args=())
+def accumulate_knn(distances: torch.Tensor, features: torch.Tensor, indices: torch.Tensor, n_moments: int,
+                   mean_and_max: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    """modules/compiled/accumulate_knn_module.cc:7-14 (`distances` are the weights)"""
+    out, maxidx, _ = _accumulate_forward(distances, features, indices, n_moments, mean_and_max, False)
     return out, maxidx
+
+
+@torch.library.custom_op("hgcalml::accumulate_knn_slots", mutates_args=())
+def accumulate_knn_slots(distances: torch.Tensor, features: torch.Tensor, indices: torch.Tensor, n_moments: int,
+                         mean_and_max: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """accumulate_knn plus the arg-max SLOT per (vertex, feature) as uint8 (an
+    empty tensor when it does not apply), which lets the gradient gather one
+    byte instead of four per (neighbour, feature)."""
+    out, maxidx, slots = _accumulate_forward(distances, features, indices, n_moments, mean_and_max, True)
+    if slots is None:
+        slots = torch.empty((0,), dtype=torch.uint8, device=out.device)
+    return out, maxidx, slots
 
 
 def inverse_neighbour_index(indices):
@@ -203,23 +223,41 @@ def cached_inverse_neighbour_index(indices):
     return value
 
 
-@torch.library.custom_op("hgcalml::accumulate_knn_grad", mutates_args=())
-def accumulate_knn_grad(grad_from_out_features: torch.Tensor, distances: torch.Tensor, features: torch.Tensor,
-                        neigh_indices: torch.Tensor, max_feat_indices: torch.Tensor, inv_offsets: torch.Tensor,
-                        inv_slots: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """modules/compiled/accumulate_knn_grad_module.cc:7-14 plus the inverse
-    neighbour index of `neigh_indices`"""
+def _accumulate_backward(grad_from_out_features, distances, features, neigh_indices, max_feat_indices, max_slots,
+                         inv_offsets, inv_slots):
     dev = require_device(grad_from_out_features, distances, features, neigh_indices, max_feat_indices)
     g, w, x = f32(grad_from_out_features), f32(distances), f32(features)
     idx, mi = i32(neigh_indices), i32(max_feat_indices)
     n, k = idx.shape
     f = x.shape[1]
     mean_and_max = g.shape[1] > f  # modules/compiled/accumulate_knn_grad_kernel.cc:253
+    if max_slots is not None and max_slots.numel() != n * f:
+        max_slots = None
     gw = torch.empty((n, k), dtype=torch.float32, device=dev)
     gx = torch.empty((n, f), dtype=torch.float32, device=dev)
-    check(lib.hgc_accumulate_knn_grad(p(g), p(w), p(x), p(mi), p(idx), p(inv_offsets), p(inv_slots), p(gw), p(gx),
-                                      n, k, f, g.shape[1], 0, int(mean_and_max), stream()))
+    check(lib.hgc_accumulate_knn_grad_slots(p(g), p(w), p(x), p(mi), p(max_slots), p(idx), p(inv_offsets),
+                                            p(inv_slots), p(gw), p(gx), n, k, f, g.shape[1], 0, int(mean_and_max),
+                                            stream()))
     return gw, gx
+
+
+@torch.library.custom_op("hgcalml::accumulate_knn_grad", mutates_args=())
+def accumulate_knn_grad(grad_from_out_features: torch.Tensor, distances: torch.Tensor, features: torch.Tensor,
+                        neigh_indices: torch.Tensor, max_feat_indices: torch.Tensor, inv_offsets: torch.Tensor,
+                        inv_slots: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """modules/compiled/accumulate_knn_grad_module.cc:7-14 plus the inverse
+    neighbour index of `neigh_indices`"""
+    return _accumulate_backward(grad_from_out_features, distances, features, neigh_indices, max_feat_indices, None,
+                                inv_offsets, inv_slots)
+
+
+@torch.library.custom_op("hgcalml::accumulate_knn_grad_slots", mutates_args=())
+def accumulate_knn_grad_slots(grad_from_out_features: torch.Tensor, distances: torch.Tensor, features: torch.Tensor,
+                              neigh_indices: torch.Tensor, max_feat_indices: torch.Tensor, max_slots: torch.Tensor,
+                              inv_offsets: torch.Tensor, inv_slots: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """accumulate_knn_grad fed with the slot table of accumulate_knn_slots"""
+    return _accumulate_backward(grad_from_out_features, distances, features, neigh_indices, max_feat_indices,
+                                max_slots, inv_offsets, inv_slots)
 
 
 # --------------------------------------------------------------------------- condensates

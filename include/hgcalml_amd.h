@@ -180,6 +180,19 @@ int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int 
                        int n_vert, int n_neigh, int n_feat, int n_out_feat,
                        int n_moments, int mean_and_max, hgc_stream_t stream);
 
+/* hgc_accumulate_knn that also reports, as one byte per (vertex, feature), the
+ * neighbour SLOT that attained the maximum (255: none; for a repeated self
+ * reference the first slot naming the vertex, which is the one the reference's
+ * gradient credits). Has no counterpart in the reference, which re-derives the
+ * slot in the gradient by comparing indices; it exists so that the gradient
+ * gathers 1 byte instead of 4 per (neighbour, feature). Needs n_neigh <= 254
+ * and, like the reference, indices that are unique in a row apart from
+ * repeated self references. d_out_maxslots [n_vert, n_feat] may be NULL. */
+int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, const int *d_idxs,
+                             float *d_out_feat, int *d_out_maxidxs, unsigned char *d_out_maxslots,
+                             int n_vert, int n_neigh, int n_feat, int n_out_feat,
+                             int n_moments, int mean_and_max, hgc_stream_t stream);
+
 /* Inverse neighbour index: for every vertex m the list of (vertex, slot)
  * pairs that name m, ascending. Built once per neighbour table and reused by
  * every gradient call on it.
@@ -207,6 +220,17 @@ int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *
                             float *d_out_grad_distances, float *d_out_grad_features,
                             int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
                             int n_moments, int mean_and_max, hgc_stream_t stream);
+
+/* hgc_accumulate_knn_grad with the arg-max slot table of
+ * hgc_accumulate_knn_slots (d_max_slots [n_vert, n_feat], may be NULL: then
+ * identical to hgc_accumulate_knn_grad). Same results, less gather traffic. */
+int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const float *d_distances,
+                                  const float *d_feat, const int *d_max_feat_indices,
+                                  const unsigned char *d_max_slots, const int *d_neigh_indices,
+                                  const int *d_inv_offsets, const int *d_inv_slots,
+                                  float *d_out_grad_distances, float *d_out_grad_features,
+                                  int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
+                                  int n_moments, int mean_and_max, hgc_stream_t stream);
 
 /* ------------------------------------------------------------------ */
 /* Condensate assignment                                               */

@@ -282,6 +282,41 @@ def test_accumulate_gradient(oracle, K, F):
         assert (gw.cpu().numpy()[idx < 0] == 0).all()
 
 
+@pytest.mark.parametrize("K,F", [(16, 32), (64, 64), (64, 128), (20, 192), (12, 256)])
+def test_accumulate_slot_table_path(oracle, K, F):
+    """forward with arg-max slots + gradient fed with them: same bits as the
+    index-comparing path and as the oracle, including repeated self references"""
+    rng = np.random.default_rng(30 + K + F)
+    n = 300
+    d, x, idx = make_acc_case(rng, n, K, F)
+    idx[7, K // 2:] = 7
+    x[7] = 50.0      # self is the arg-max of vertex 7: the max part goes to its FIRST slot
+    idx[9, 1:4] = 9
+    x[9] = -50.0
+    w = np.exp(-d).astype(np.float32)
+    g = rng.standard_normal((n, 2 * F)).astype(np.float32)
+    from hgcalml_amd import ops
+    out, arg, slots = torch.ops.hgcalml.accumulate_knn_slots(t(w), t(x), t(idx), 0, True)
+    ref, rarg = oracle.AccumulateLinKnn(w, x, idx)
+    assert (bits(out.cpu().numpy()) == bits(ref)).all() and (arg.cpu().numpy() == rarg).all()
+    sl = slots.cpu().numpy()
+    assert sl.shape == (n, F) and sl.dtype == np.uint8
+    # the slot names the arg-max index (first occurrence), 255 where nothing was taken
+    first_occurrence = np.array([[next((s_ for s_ in range(K) if idx[v, s_] == rarg[v, f]), 255) for f in range(F)]
+                                 for v in (7, 9, 0, 1, n // 2, n // 2 + 2)])
+    got = sl[[7, 9, 0, 1, n // 2, n // 2 + 2]]
+    taken = got != 255
+    assert (got[taken] == first_occurrence[taken]).all()
+    assert (sl[n // 2 + 2] == 255).all()      # a row without any neighbour
+    rgw, rgx = oracle.accumulate_knn_grad_kernel(g, w, x, idx, rarg)
+    inv = ops.inverse_neighbour_index(t(idx))
+    gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(g), t(w), t(x), t(idx), arg, slots, *inv)
+    gw0, gx0 = torch.ops.hgcalml.accumulate_knn_grad(t(g), t(w), t(x), t(idx), arg, *inv)
+    assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
+    assert torch.equal(gx, gx0) and torch.equal(gw, gw0)
+    assert (np.abs(gw.cpu().numpy() - rgw) <= grad_tolerance(g, x, idx, w, K)).all()
+
+
 def test_inverse_neighbour_index_is_ordered():
     from hgcalml_amd import ops
     rng = np.random.default_rng(21)
