@@ -18,6 +18,7 @@
 // no float atomics anywhere.
 #include "hgc_common.hpp"
 
+#include <cstdlib>
 #include <cstring>
 #include <algorithm>
 
@@ -272,11 +273,7 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
     const float *wrow = w + (size_t)v * K;
     const float kf = (float)K;
     const RowMatrix X(feat, n_vert, F);
-    int first_self = -1;  // first slot that names the vertex itself (wave-uniform)
-    if (MAX && out_maxslot) {
-        for (int n = K - 1; n >= 0; --n)
-            if (irow[n] == v) first_self = n;
-    }
+    int first_self = -1;  // first slot that names the vertex itself (wave-uniform, scalar ALU)
 
     for (int fb = lane_id() * VEC; fb < F; fb += kWave * VEC) {
         const uint32_t lane_bytes = (uint32_t)fb * 4u;
@@ -299,6 +296,13 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                 j[u] = irow[n0 + u];
                 wn[u] = wrow[n0 + u];
                 all_valid = all_valid && (unsigned)j[u] < (unsigned)n_vert;
+            }
+            if (MAX) {
+                int fs = -1;
+#pragma unroll
+                for (int u = U - 1; u >= 0; --u)
+                    if (j[u] == v) fs = n0 + u;
+                if (first_self < 0) first_self = fs;
             }
             if (all_valid) {  // wave-uniform: the common, padding-free chunk
 #pragma unroll
@@ -327,6 +331,7 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
         for (; n0 < K; ++n0) {  // K not a multiple of U
             const int jj = irow[n0];
             if ((unsigned)jj >= (unsigned)n_vert) continue;
+            if (jj == v && first_self < 0) first_self = n0;
             float xs[VEC];
             X.load<VEC>(jj, lane_bytes, xs);
             if (n0 == 0)
@@ -449,85 +454,92 @@ __global__ __launch_bounds__(256) void feature_grad_wave_kernel(const float *__r
 #pragma unroll
         for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
         bool self_seen = false;  // repeated self references carry the max part once
-        int e0 = begin;
-        for (; e0 + U <= end; e0 += U) {
-            int v[U], key[U];
-            float wv[U];
-            float gm[U][VEC], gx[U][VEC];
-            int mi[U][VEC];
+        if (begin < end) {
+            // The scalar side (inverse-list slots, then the weights they address) runs
+            // one chunk ahead of the vector side so that its latency is hidden behind
+            // the row gathers. Entries past the end are clamped to the last one and
+            // skipped in the arithmetic.
+            const int last = end - 1;
+            int slot_cur[U], slot_nxt[U];
+            float w_cur[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int slot = inv_slots[e0 + u];
-                v[u] = fast_div(slot, div_k);
-                key[u] = SLOTS ? slot - v[u] * K : m;
-                wv[u] = w[slot];
-            }
+            for (int u = 0; u < U; ++u) slot_cur[u] = inv_slots[min(begin + u, last)];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                G.load<VEC>(v[u], lane_bytes, gm[u]);
-                if (MAX) {
-                    if (SLOTS) {
-                        load_slots<VEC>(MS, v[u], (uint32_t)F, (uint32_t)fb, mi[u]);
-                    } else {
-                        MI.load<VEC>(v[u], lane_bytes, mi[u]);
-                        G.load<VEC>(v[u], lane_bytes + max_col_bytes, gx[u]);
-                    }
-                }
-            }
-            if (MAX && SLOTS) {
-                // the max half of a gradient row is fetched only by the lanes whose
-                // feature has its maximum at this entry (about F/K lanes per row)
+            for (int u = 0; u < U; ++u) w_cur[u] = w[slot_cur[u]];
+#pragma unroll
+            for (int u = 0; u < U; ++u) slot_nxt[u] = inv_slots[min(begin + U + u, last)];
+
+            for (int e0 = begin; e0 < end; e0 += U) {
+                int v[U], key[U];
+                float gm[U][VEC], gx[U][VEC];
+                int mi[U][VEC];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    bool any = false;
+                    v[u] = fast_div(slot_cur[u], div_k);
+                    key[u] = SLOTS ? slot_cur[u] - v[u] * K : m;
+                }
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        any = any || mi[u][e] == key[u];
-                        gx[u][e] = 0.f;
+                for (int u = 0; u < U; ++u) {
+                    G.load<VEC>(v[u], lane_bytes, gm[u]);
+                    if (MAX) {
+                        if (SLOTS) {
+                            load_slots<VEC>(MS, v[u], (uint32_t)F, (uint32_t)fb, mi[u]);
+                        } else {
+                            MI.load<VEC>(v[u], lane_bytes, mi[u]);
+                            G.load<VEC>(v[u], lane_bytes + max_col_bytes, gx[u]);
+                        }
                     }
-                    if (any) G.load<VEC>(v[u], lane_bytes + max_col_bytes, gx[u]);
                 }
-            }
+                // scalar prefetch for the next two chunks
+                float w_nxt[U];
+                int slot_nn[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                bool count_max = true;
-                if (!SLOTS && v[u] == m) {  // (the slot table already points at the first self slot)
-                    count_max = !self_seen;
-                    self_seen = true;
+                for (int u = 0; u < U; ++u) w_nxt[u] = w[slot_nxt[u]];
+#pragma unroll
+                for (int u = 0; u < U; ++u) slot_nn[u] = inv_slots[min(e0 + 2 * U + u, last)];
+
+                if (MAX && SLOTS) {
+                    // the max half of a gradient row is fetched only by the lanes whose
+                    // feature has its maximum at this entry (about F/K lanes per row)
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        bool any = false;
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) {
+                            any = any || mi[u][e] == key[u];
+                            gx[u][e] = 0.f;
+                        }
+                        if (any) G.load<VEC>(v[u], lane_bytes + max_col_bytes, gx[u]);
+                    }
                 }
-                fgrad_entry<VEC, MAX, POW2K>(gm[u], gx[u], mi[u], wv[u], key[u], count_max, kf, inv_k, acc);
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (e0 + u >= end) break;  // wave-uniform
+                    bool count_max = true;
+                    if (!SLOTS && v[u] == m) {  // (the slot table already points at the first self slot)
+                        count_max = !self_seen;
+                        self_seen = true;
+                    }
+                    fgrad_entry<VEC, MAX, POW2K>(gm[u], gx[u], mi[u], w_cur[u], key[u], count_max, kf, inv_k, acc);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    slot_cur[u] = slot_nxt[u];
+                    w_cur[u] = w_nxt[u];
+                    slot_nxt[u] = slot_nn[u];
+                }
             }
-        }
-        for (; e0 < end; ++e0) {
-            const int slot = inv_slots[e0];
-            const int vv = fast_div(slot, div_k);
-            const int key = SLOTS ? slot - vv * K : m;
-            float gm[VEC], gx[VEC];
-            int mi[VEC];
-            G.load<VEC>(vv, lane_bytes, gm);
-            if (MAX) {
-                if (SLOTS)
-                    load_slots<VEC>(MS, vv, (uint32_t)F, (uint32_t)fb, mi);
-                else
-                    MI.load<VEC>(vv, lane_bytes, mi);
-                G.load<VEC>(vv, lane_bytes + max_col_bytes, gx);
-            }
-            bool count_max = true;
-            if (!SLOTS && vv == m) {
-                count_max = !self_seen;
-                self_seen = true;
-            }
-            fgrad_entry<VEC, MAX, POW2K>(gm, gx, mi, w[slot], key, count_max, kf, inv_k, acc);
         }
         store_vec<VEC>(gfeat + (size_t)m * F + fb, acc);
     }
 }
 
-// After the call lane L holds the sum over all 64 lanes of value index L.
-__device__ __forceinline__ float transpose_reduce_64(float (&val)[64]) {
+// 32 partial sums per lane in, after the call lane L holds the sum over all 64
+// lanes of value index (L & 31). Fixed butterfly: deterministic summation order.
+__device__ __forceinline__ float transpose_reduce_32(float (&val)[32]) {
     const int lane = lane_id();
 #pragma unroll
-    for (int h = 32; h >= 1; h >>= 1) {
+    for (int h = 16; h >= 1; h >>= 1) {
         const bool upper = (lane & h) != 0;
 #pragma unroll
         for (int i = 0; i < h; ++i) {
@@ -537,7 +549,7 @@ __device__ __forceinline__ float transpose_reduce_64(float (&val)[64]) {
             val[i] = keep + __shfl_xor(send, h, kWave);
         }
     }
-    return val[0];
+    return val[0] + __shfl_xor(val[0], 32, kWave);
 }
 
 template <int VEC, bool MAX>
@@ -546,7 +558,7 @@ __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__re
                                                                float *__restrict__ gw, int n_vert, int K, int F,
                                                                int g_cols) {
     constexpr int U = 8;
-    constexpr int G = 32;  // slots per reduction group: 32 mean sums + 32 max sums = 64 values
+    constexpr int G = 16;  // slots per reduction group: 16 mean sums + 16 max sums = 32 values
     const int m = wave_vertex();
     if (m >= n_vert) return;
     const int lane = lane_id();
@@ -555,9 +567,9 @@ __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__re
     const RowMatrix X(feat, n_vert, F);
 
     for (int l0 = 0; l0 < K; l0 += G) {
-        float val[64];
+        float val[2 * G];
 #pragma unroll
-        for (int i = 0; i < 64; ++i) val[i] = 0.f;
+        for (int i = 0; i < 2 * G; ++i) val[i] = 0.f;
         for (int fb = lane * VEC; fb < F; fb += kWave * VEC) {
             const uint32_t lane_bytes = (uint32_t)fb * 4u;
             float gm[VEC], gx[VEC];
@@ -576,9 +588,9 @@ __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__re
                     const int l = l0 + u0 + u;
                     j[u] = l < K ? irow[l] : -1;
                 }
-                // rows outside [0, n_vert) read as zeros (hardware range check) and
-                // can never equal an arg-max index of a valid row; their result is
-                // overwritten with 0 below
+                // rows outside [0, n_vert) read as arbitrary in-range data or zeros
+                // (hardware range check) and can never equal an arg-max index of a
+                // valid row; their result is overwritten with 0 below
 #pragma unroll
                 for (int u = 0; u < U; ++u) X.load<VEC>(j[u], lane_bytes, x[u]);
 #pragma unroll
@@ -594,8 +606,8 @@ __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__re
                 }
             }
         }
-        const float r = transpose_reduce_64(val);        // lane < 32: mean sum of slot l0+lane; else max sum
-        const float r_max = __shfl_xor(r, 32, kWave);    // lane < 32 receives its max sum
+        const float r = transpose_reduce_32(val);        // lanes 0..15 (mod 32): mean sums, 16..31: max sums
+        const float r_max = __shfl_xor(r, 16, kWave);    // lane < 16 receives its max sum
         const int l = l0 + lane;
         if (lane < G && l < K) {
             const int j = irow[l];
@@ -958,6 +970,7 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
         const int vec = wave_vec(n_feat, align_or);
         const dim3 grid(ceil_div(n_vert, 4)), block(256);
         const FastDiv div_k = make_fast_div(n_neigh);
+        const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
 #define HGC_FGW(VEC, MAX, P2, SL)                                                                                      \
     feature_grad_wave_kernel<VEC, MAX, P2, SL><<<fg_grid, block, 0, s>>>(                                              \
         d_grad_from_out_features, d_distances, d_max_feat_indices, d_max_slots, d_inv_offsets, d_inv_slots,            \
@@ -968,9 +981,13 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
         else if (mean_and_max) { if (pow2k) HGC_FGW(VEC, true, true, false); else HGC_FGW(VEC, true, false, false); } \
         else { if (pow2k) HGC_FGW(VEC, false, true, false); else HGC_FGW(VEC, false, false, false); }       \
     } while (0)
-        const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
         // two feature slices as soon as a row has two or more 64-feature blocks
-        const int n_slices = n_feat >= 2 * kWave ? 2 : 1;
+        // Without the slot table a gathered row is 1.5 KB (gradient row + arg-max
+        // indices) and the neighbour window overflows one XCD's L2: slice. With it
+        // the row shrinks to 640 B plus a few lanes of the max half and the wider
+        // unsliced loads win.
+        int n_slices = (n_feat >= 2 * kWave && !(mean_and_max && use_slots)) ? 2 : 1;
+        if (const char *env = getenv("HGC_FGRAD_SLICES")) n_slices = atoi(env) == 2 && n_feat >= 2 * kWave ? 2 : 1;  // tuning aid
         const int fg_vec = n_slices == 1 ? vec : wave_vec(n_feat / 2, align_or);
         const int tiles = ceil_div(n_vert, 4);
         const dim3 fg_grid(n_slices == 1 ? tiles : kNumXcd * ceil_div(tiles, kNumXcd / n_slices));
