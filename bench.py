@@ -35,6 +35,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per forward+gradient pass at full cfg4, from two hardware-counter
+# runs of this file's roofline section (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB,
+# both scaled by what the counters read for the 512 MB calibration copy below);
+# summary in profiles/accumulate_knn_cfg4_hbm_counters.txt. Counters cannot be
+# read from inside the timed run, so this is the last profiled value.
+CFG4_MEASURED_HBM_BYTES = 18.9e9
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -218,7 +225,8 @@ def main():
         "accumulate_fwd_grad_GBps": round(achieved, 1),
         "roofline": {"bound": "hbm", "kernel": "accumulate_knn forward + gradient, cfg4 (N=%d, K=%d, F=%d)" % (n4, K4, F4),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": CFG4_MEASURED_HBM_BYTES if args.roofline_scale == 1.0 else None,
                      "algorithmic_bytes": bytes_fwd + bytes_bwd,
                      "fwd_ms": round(fwd_ms[0], 4), "grad_ms": round(grad_ms[0], 4),
                      "fwd_GBps": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9, 1),
