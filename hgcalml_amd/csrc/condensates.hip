@@ -100,19 +100,50 @@ __global__ __launch_bounds__(256) void selection_keys_kernel(const float *__rest
     values[q] = q;
 }
 
-__global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondParams p) {
+// claimed flags of the event's high-beta hits: one bit each, in LDS when they
+// fit (LDS_FLAGS), else the caller's int array in global memory
+template <bool LDS_FLAGS>
+struct TakenFlags {
+    uint32_t *bits;  // LDS
+    int *global;     // taken_h + first_h
+    __device__ __forceinline__ bool test(int local) const {
+        if (LDS_FLAGS) return (bits[local >> 5] >> (local & 31)) & 1u;
+        return global[local] != 0;
+    }
+    __device__ __forceinline__ void set(int local) const {
+        if (LDS_FLAGS)
+            atomicOr(&bits[local >> 5], 1u << (local & 31));
+        else
+            global[local] = 1;
+    }
+};
+
+constexpr int kHitsPerThread = 4;
+
+template <bool LDS_FLAGS>
+__global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondParams p, int flag_words) {
+    extern __shared__ uint32_t s_bits[];
+    __shared__ int s_first[kWavesPerBlock];
+    __shared__ int s_pick, s_alpha;
+    __shared__ int s_row_off[kBlock + 1];
+    __shared__ int s_row_start[kBlock];
+    __shared__ int s_wave_tot[kWavesPerBlock];
+
     const int r = blockIdx.x;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
     const int first = p.row_splits[r], last = p.row_splits[r + 1];
     const int first_h = p.row_splits_h[r], last_h = p.row_splits_h[r + 1];
+    const TakenFlags<LDS_FLAGS> taken{s_bits, p.taken_h + first_h};
 
     for (int q = first_h + tid; q < last_h; q += kBlock) {
         p.is_alpha_h[q] = 0;
         p.taken_h[q] = 0;
         p.alpha_indices[q] = -1;
     }
+    if (LDS_FLAGS)
+        for (int i = tid; i < flag_words; i += kBlock) s_bits[i] = 0;
     for (int i = first + tid; i < last; i += kBlock) {
         p.assignment[i] = -1;
         p.association[i] = -1;
@@ -129,21 +160,23 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
     }
     const int *bin_splits = p.bin_splits + (size_t)cells * r;
     const float bw = p.bin_widths[0];
-
-    __shared__ int s_first[kWavesPerBlock];
-    __shared__ int s_pick;
+    const float edge_slack = 1e-3f * bw;  // bins are cut by a rounded fp32 divide
     __syncthreads();
 
-    int cursor = first_h;  // everything before it in the order is claimed
+    int cursor = first_h;  // everything before it in the selection order is claimed
+    int window = -1;       // start of the 1024 order entries cached in registers
+    int my_q = -1;
+    bool my_selectable = false;
     int shower = 0;
     while (cursor < last_h) {
         // ---- next unclaimed hit in selection order ----
-        const int pos = cursor + tid;
-        bool open = false;
-        if (pos < last_h) {
-            const int q = p.order_h[pos];
-            open = p.taken_h[q] == 0 && (always_first(p.mask_h, p.n_vert_h, q) || p.beta_h[q] > -1.f);
+        if (window < 0 || cursor >= window + kBlock) {
+            window = cursor;
+            const int pos = window + tid;
+            my_q = pos < last_h ? p.order_h[pos] : -1;
+            my_selectable = my_q >= 0 && (always_first(p.mask_h, p.n_vert_h, my_q) || p.beta_h[my_q] > -1.f);
         }
+        const bool open = my_selectable && window + tid >= cursor && !taken.test(my_q - first_h);
         const uint64_t b = __ballot(open);
         if (lane == 0) s_first[wave] = b ? wave * kWave + (__ffsll((long long)b) - 1) : kBlock;
         __syncthreads();
@@ -155,14 +188,16 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         __syncthreads();
         const int pick = s_pick;
         if (pick == kBlock) {  // nothing open in this window
-            cursor += kBlock;
+            cursor = window + kBlock;
             __syncthreads();
             continue;
         }
-        cursor += pick;
-        const int alpha = p.order_h[cursor];
+        if (tid == pick) s_alpha = my_q;
+        __syncthreads();
+        cursor = window + pick;
+        const int alpha = s_alpha;
 
-        // ---- claim step: all threads test the hits of alpha's box of bins ----
+        // ---- claim step ----
         float centre[kMaxDims];
 #pragma unroll
         for (int c = 0; c < kMaxDims; ++c) centre[c] = c < C ? p.ccoords_h[(size_t)alpha * C + c] : 0.f;
@@ -170,6 +205,7 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         const float radius_sq = radius * radius;
         const bool solitary = p.mask_h[alpha] > 0;
         if (solitary) radius = 0.f;
+        const float reach_sq = radius * radius * 1.0001f;  // pruning bound, slightly generous
 
         int lo_bin[kMaxBinDims], width[kMaxBinDims];
         int n_rows = 1;
@@ -193,46 +229,122 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         const int run_lo = lo_bin[B - 1], run_hi = lo_bin[B - 1] + width[B - 1] - 1;
         const int shower_orig = p.orig_h[alpha];
 
-        for (int row = wave; row < n_rows; row += kWavesPerBlock) {
-            // per-dimension indices are not range checked (only the flat index
-            // is), like the reference
-            long long base = 0;
-            int rem = row;
-            long long stride = nb[B - 1];
-            for (int d = B - 2; d >= 0; --d) {
-                const int k = lo_bin[d] + rem % width[d];
-                rem /= width[d];
-                base += (long long)k * stride;
-                stride *= nb[d];
-            }
-            long long a = base + run_lo, z = base + run_hi;
-            if (a < 0) a = 0;
-            if (z > cells - 1) z = cells - 1;
-            if (a > z) continue;
-            const int hit_lo = bin_splits[a], hit_hi = bin_splits[z + 1];
-            for (int i = hit_lo + lane; i < hit_hi; i += kWave) {
-                if (p.by_max_beta && p.assignment[i] != -1) continue;
-                float dsq = 0.f;
-                for (int c = 0; c < C; ++c) {
-                    const float t = centre[c] - p.ccoords[(size_t)i * C + c];
-                    dsq = dsq + t * t;
+        for (int row0 = 0; row0 < n_rows; row0 += kBlock) {
+            // -- every thread resolves one row of the box into a run of hits --
+            int start = 0, len = 0;
+            const int row = row0 + tid;
+            if (row < n_rows) {
+                // per-dimension indices are not range checked (only the flat index
+                // is), like the reference
+                long long base = 0;
+                int rem = row;
+                long long stride = nb[B - 1];
+                bool in_grid = true;
+                float gap_sq = 0.f;
+                for (int d = B - 2; d >= 0; --d) {
+                    const int k = lo_bin[d] + rem % width[d];
+                    rem /= width[d];
+                    base += (long long)k * stride;
+                    stride *= nb[d];
+                    in_grid = in_grid && k >= 0 && k < nb[d];
+                    // distance from the centre to the slab of bin k in this dimension
+                    const float below = (float)k * bw - edge_slack - centre[d];
+                    const float above = centre[d] - ((float)(k + 1) * bw + edge_slack);
+                    const float gap = fmaxf(0.f, fmaxf(below, above));
+                    gap_sq += gap * gap;
                 }
-                const int filt = p.to_filtered[i];
-                const bool inside = (dsq <= radius_sq && !solitary && p.mask[i] == 0) || (solitary && filt == alpha);
-                if (!inside) continue;
-                if (!p.by_max_beta) {
-                    const float lhs = p.best_dsq[i] * radius_sq;
-                    if (!(lhs >= dsq)) continue;
-                    p.best_dsq[i] = dsq;
+                int k_lo = run_lo, k_hi = run_hi;
+                bool keep = true;
+                if (in_grid && !solitary) {
+                    // rows of real bins can be pruned against the sphere: no hit of a
+                    // skipped bin can pass d^2 <= radius^2 (slack covers fp rounding)
+                    const float rest = reach_sq - gap_sq;
+                    if (rest < 0.f) {
+                        keep = false;
+                    } else {
+                        const float half = sqrtf(rest) + edge_slack;
+                        k_lo = max(k_lo, (int)floorf((centre[B - 1] - half) / bw) - 1);
+                        k_hi = min(k_hi, (int)floorf((centre[B - 1] + half) / bw) + 1);
+                    }
                 }
-                p.assignment[i] = shower;
-                p.association[i] = shower_orig;
-                if (filt != -1) p.taken_h[filt] = 1;
+                long long a = base + k_lo, z = base + k_hi;
+                if (a < 0) a = 0;
+                if (z > cells - 1) z = cells - 1;
+                if (keep && a <= z) {
+                    start = bin_splits[a];
+                    len = bin_splits[z + 1] - start;
+                }
             }
+            // -- exclusive scan of the run lengths over the workgroup --
+            const int incl = wave_inclusive_sum(len);
+            if (lane == kWave - 1) s_wave_tot[wave] = incl;
+            __syncthreads();
+            int wave_off = 0, total = 0;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) {
+                const int t = s_wave_tot[w];
+                if (w < wave) wave_off += t;
+                total += t;
+            }
+            s_row_off[tid] = wave_off + incl - len;
+            s_row_start[tid] = start;
+            if (tid == 0) s_row_off[kBlock] = total;
+            __syncthreads();
+
+            // -- all hits of all runs, kHitsPerThread per thread with their loads batched --
+            for (int h0 = 0; h0 < total; h0 += kBlock * kHitsPerThread) {
+                int hit[kHitsPerThread];
+                bool live[kHitsPerThread];
+#pragma unroll
+                for (int k = 0; k < kHitsPerThread; ++k) {
+                    const int h = h0 + k * kBlock + tid;
+                    live[k] = h < total;
+                    // last row whose offset is <= h (empty rows share their successor's offset)
+                    int lo_r = 0;
+#pragma unroll
+                    for (int step = kBlock / 2; step > 0; step >>= 1) {
+                        const int probe = lo_r + step;
+                        if (s_row_off[probe] <= h) lo_r = probe;
+                    }
+                    hit[k] = live[k] ? s_row_start[lo_r] + (h - s_row_off[lo_r]) : first;
+                }
+                int asg[kHitsPerThread], filt[kHitsPerThread], msk[kHitsPerThread];
+                float dsq[kHitsPerThread];
+#pragma unroll
+                for (int k = 0; k < kHitsPerThread; ++k) {
+                    const int i = hit[k];
+                    asg[k] = p.assignment[i];
+                    filt[k] = p.to_filtered[i];
+                    msk[k] = p.mask[i];
+                    float acc = 0.f;
+                    for (int c = 0; c < C; ++c) {
+                        const float t = centre[c] - p.ccoords[(size_t)i * C + c];
+                        acc = acc + t * t;
+                    }
+                    dsq[k] = acc;
+                }
+#pragma unroll
+                for (int k = 0; k < kHitsPerThread; ++k) {
+                    if (!live[k]) continue;
+                    const int i = hit[k];
+                    if (p.by_max_beta && asg[k] != -1) continue;
+                    const bool inside = (dsq[k] <= radius_sq && !solitary && msk[k] == 0) || (solitary && filt[k] == alpha);
+                    if (!inside) continue;
+                    if (!p.by_max_beta) {
+                        const float lhs = p.best_dsq[i] * radius_sq;
+                        if (!(lhs >= dsq[k])) continue;
+                        p.best_dsq[i] = dsq[k];
+                    }
+                    p.assignment[i] = shower;
+                    p.association[i] = shower_orig;
+                    if (filt[k] != -1) taken.set(filt[k] - first_h);
+                }
+            }
+            __syncthreads();  // LDS row tables are reused by the next tile / condensate
         }
         if (tid == 0) {
             p.is_alpha_h[alpha] = 1;
-            p.taken_h[alpha] = 1;
+            taken.set(alpha - first_h);
             p.alpha_indices[first_h + shower] = shower_orig;
         }
         ++shower;
@@ -355,7 +467,13 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int
         p.n_vert_h = n_vert_h;
         p.order_h = order;
         p.event_count = event_count;
-        condensate_event_kernel<<<num_rows, kBlock, 0, s>>>(p);
+        // one claimed-flag bit per high-beta hit of an event lives in LDS when it fits
+        // (n_vert_h bounds every event); 48 KB = 393k hits
+        const int flag_words = ceil_div(std::max(n_vert_h, 1), 32);
+        if ((size_t)flag_words * 4 <= 48 * 1024)
+            condensate_event_kernel<true><<<num_rows, kBlock, (size_t)flag_words * 4, s>>>(p, flag_words);
+        else
+            condensate_event_kernel<false><<<num_rows, kBlock, 0, s>>>(p, 0);
         int rc = check_launch("condensate_event_kernel");
         if (rc) return rc;
     }

@@ -78,19 +78,68 @@ __device__ __forceinline__ float dist_sq(const float (&q)[C > 0 ? C : 1], const 
     return acc;
 }
 
-// insert key c (known to be smaller than the current last key of the list)
+extern "C" __device__ int __llvm_amdgcn_writelane(int, int, int) __asm("llvm.amdgcn.writelane");
+
+// `into` with lane `lane` (wave-uniform) replaced by the wave-uniform `value`
+__device__ __forceinline__ uint64_t writelane_u64(uint64_t value, int lane, uint64_t into) {
+    const uint32_t lo = (uint32_t)__llvm_amdgcn_writelane((int)(uint32_t)value, lane, (int)(uint32_t)into);
+    const uint32_t hi = (uint32_t)__llvm_amdgcn_writelane((int)(uint32_t)(value >> 32), lane, (int)(uint32_t)(into >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// lane i receives v from lane i-1; lane 0 (and lanes whose source is masked off) read 0
+__device__ __forceinline__ uint64_t wave_shift_up1_zero(uint64_t v) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)v, 0x138, 0xf, 0xf, true);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)(v >> 32), 0x138, 0xf, 0xf, true);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// Sorted insert of the wave-uniform key c into the ascending list held across
+// the lanes (and register levels); the largest key falls off the end. Lanes
+// holding a larger key take their left neighbour's key (DPP wave shift under the
+// execution mask of exactly those lanes), then c is written into the first of
+// them. A key that is larger than everything in the list changes nothing.
 template <int S>
 __device__ __forceinline__ void sorted_insert(uint64_t (&key)[S], uint64_t c) {
-    uint64_t carry = 0;  // what enters lane 0 of the next register level
-#pragma unroll
-    for (int s = 0; s < S; ++s) {
-        const uint64_t old = key[s];
-        const uint64_t last = readlane_u64(old, kWave - 1);
-        if (c < last) {  // wave-uniform: the insertion point is in or before this level
-            const uint64_t prev = wave_shift_up1_u64(old, carry);
-            key[s] = (c < prev) ? prev : ((c < old) ? c : old);
+    if constexpr (S == 1) {
+        const uint64_t old = key[0];
+        const bool larger = old > c;
+        const uint64_t run = __ballot(larger);  // contiguous upper lanes, the list is sorted
+        if (run) {
+            if (larger) key[0] = wave_shift_up1_zero(old);
+            key[0] = writelane_u64(c, __ffsll((long long)run) - 1, key[0]);
         }
-        carry = last;
+    } else {
+        uint64_t carry = 0;   // what enters lane 0 of the next register level
+        bool placed = false;  // wave-uniform
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            const uint64_t old = key[s];
+            const uint64_t last = readlane_u64(old, kWave - 1);
+            const bool larger = placed || old > c;
+            const uint64_t run = __ballot(larger);
+            if (run) {
+                if (larger) key[s] = wave_shift_up1_u64(old, carry);
+                if (!placed) {
+                    key[s] = writelane_u64(c, __ffsll((long long)run) - 1, key[s]);
+                    placed = true;
+                }
+            }
+            carry = last;
+        }
+    }
+}
+
+// q = x / w, r = x % w for 0 <= x < 2^23 and small w, without an integer divide
+__device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, int &r) {
+    q = (int)((float)x * inv_w);
+    r = x - q * w;
+    if (r < 0) {
+        r += w;
+        --q;
+    } else if (r >= w) {
+        r -= w;
+        ++q;
     }
 }
 
@@ -145,15 +194,18 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
         const int nb_last = nb[B - 1], qb_last = qb[B - 1];
         const float bw = p.bin_width[0];
 
-        // keys at or above `limit` can never enter: the radius cut, if any
         const bool has_radius = p.radius_sq >= 0.f;
-        const uint64_t limit = has_radius ? ((uint64_t)(__float_as_uint(p.radius_sq) + 1u) << 32) : kEmptyKey;
         const int kth_lane = (Kn - 1) & (kWave - 1);
         const int kth_level = (Kn - 1) >> 6;
-        uint64_t thr = limit;  // min(limit, current K-th key)
+        // With a spare rank behind the K-th one (S*64 > K-1) a candidate that no
+        // longer beats the K-th key may be inserted anyway: it lands in the spare
+        // ranks. Then the K-th key is re-read once per batch instead of per insert.
+        const bool spare_rank = S * kWave > Kn;
+        uint64_t thr = kEmptyKey;  // current K-th key: candidates at or above it cannot enter
 
         for (int d = 0; d <= reach_max; ++d) {
             const int W = 2 * d + 1;
+            const float inv_W = 1.f / (float)W;
             int n_rows = 1;
             for (int i = 0; i < B - 1; ++i) n_rows *= W;
             const int n_slots = d == 0 ? 1 : 2 * n_rows;
@@ -162,6 +214,12 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                 // ---- each lane resolves one segment of the shell ----
                 int seg_start = 0, seg_len = 0;
                 const int slot = slot0 + lane;
+                // Nothing farther than `reach2` can still enter the list (K-th distance
+                // once the list is full, the radius cut otherwise). A bin at offset o
+                // from the query's bin is at least (|o|-1) bin widths away in that
+                // dimension, whatever the query's position inside its own bin.
+                float reach2 = thr == kEmptyKey ? 3.0e38f : __uint_as_float((uint32_t)(thr >> 32));
+                if (has_radius) reach2 = fminf(reach2, p.radius_sq);
                 if (slot < n_slots) {
                     int row = slot >> 1;
                     const int second = slot & 1;
@@ -171,12 +229,13 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                     for (int i = kMaxBinDims - 2; i >= 0; --i) {
                         off[i] = 0;
                         if (i < B - 1) {
-                            const int digit = row % W;
-                            row /= W;
+                            int digit;
+                            divmod_small(row, W, inv_W, row, digit);
                             off[i] = digit - d;
                         }
                     }
                     int cell = 0;
+                    float gap2 = 0.f;  // squared lower bound of the distance to this row of bins
 #pragma unroll
                     for (int i = 0; i < kMaxBinDims - 1; ++i) {
                         if (i < B - 1) {
@@ -184,16 +243,30 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                             inside = inside && k >= 0 && k < nb[i];
                             on_face = on_face || off[i] == d || off[i] == -d;
                             cell = cell * nb[i] + k;
+                            const float g = (float)max(abs(off[i]) - 1, 0) * bw;
+                            gap2 += g * g;
                         }
                     }
                     int lo, hi;
                     if (on_face || d == 0) {  // the whole run of the last dimension
                         lo = qb_last - d;
                         hi = second ? lo - 1 : qb_last + d;
+                        // bins of the run that are provably too far are cut off: keep
+                        // |offset| <= sqrt(rest)/bw + 1 (one extra bin of slack)
+                        const float rest = reach2 - 0.999f * gap2;
+                        if (rest < 0.f) {
+                            hi = lo - 1;
+                        } else if (rest < 1.0e37f) {
+                            const int span = (int)(sqrtf(rest) / bw) + 2;
+                            lo = max(lo, qb_last - span);
+                            hi = min(hi, qb_last + span);
+                        }
                     } else {  // interior row: only the two end caps
                         lo = second ? qb_last + d : qb_last - d;
                         hi = lo;
                         if (lo < 0 || lo >= nb_last) hi = lo - 1;
+                        const float g = (float)(d - 1) * bw;
+                        if (0.999f * (gap2 + g * g) > reach2) hi = lo - 1;
                     }
                     lo = max(lo, 0);
                     hi = min(hi, nb_last - 1);
@@ -230,21 +303,28 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                         if (dj == 1 || dj == 2) valid = false;  // may not be a neighbour
                     }
                     const float dsq = dist_sq<C>(qc, p.coord, jj, p.n_coords, qrow);
+                    if (has_radius) valid = valid && dsq <= p.radius_sq;
                     const uint32_t id = MAPPED ? (uint32_t)p.sorting[jj] : (uint32_t)jj;
                     const uint64_t ck = ((uint64_t)__float_as_uint(dsq) << 32) | id;
                     uint64_t beats = __ballot(valid && ck < thr);
-                    while (beats) {
-                        const int src = __ffsll((long long)beats) - 1;
-                        beats &= beats - 1;
-                        const uint64_t cand = readlane_u64(ck, src);
-                        if (cand < thr) {
-                            sorted_insert<S>(key, cand);
-                            uint64_t kth = kEmptyKey;
+                    if (beats) {
+                        while (beats) {
+                            const int src = __ffsll((long long)beats) - 1;
+                            beats &= beats - 1;
+                            const uint64_t cand = readlane_u64(ck, src);
+                            if (!spare_rank) {  // no spare rank: re-check against the current K-th key
+                                uint64_t kth = kEmptyKey;
 #pragma unroll
-                            for (int s = 0; s < S; ++s)
-                                if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
-                            thr = kth < limit ? kth : limit;
+                                for (int s = 0; s < S; ++s)
+                                    if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
+                                const uint32_t ch = (uint32_t)(cand >> 32), kh = (uint32_t)(kth >> 32);
+                                if (ch > kh || (ch == kh && (uint32_t)cand >= (uint32_t)kth)) continue;
+                            }
+                            sorted_insert<S>(key, cand);
                         }
+#pragma unroll
+                        for (int s = 0; s < S; ++s)
+                            if (s == kth_level) thr = readlane_u64(key[s], kth_lane);
                     }
                 }
             }
