@@ -64,23 +64,11 @@ def BinnedSelectKnn(K, coords, row_splits, direction=None, n_bins=None, max_bin_
         return (torch.empty((0, K), dtype=torch.int32, device=dev),
                 torch.empty((0, K), dtype=torch.float32, device=dev))
 
-    shift, bin_width, nb = ops.bin_setup(coords, max_bin_dims, False, n_bins=n_bins)
-    # per-dimension bin counts are at most n_bins + 1, which bounds the table
-    # sizes without reading anything back from the device
-    total_bound = (n_bins + 1) ** max_bin_dims * n_events
-    dbinning, binning, _ = ops.bin_points(coords, max_bin_dims, shift, rs_dev, bin_width, nb, total_bound, False)
-    sorting, bin_boundaries = ops.sort_by_bin(binning, total_bound)
-
-    scoords = ops.gather_rows(coords, sorting)
-    sbinning = ops.gather_rows(binning, sorting)
-    sdbinning = ops.gather_rows(dbinning, sorting)
-    sdirection = None
-    if direction is not None:
-        sdirection = ops.gather_rows(direction.to(device=dev, dtype=torch.int32).contiguous(), sorting)
-
-    idx, dist = ops.binned_select_knn_fused(scoords, sbinning, sdbinning, bin_boundaries, nb, bin_width, sdirection,
-                                            sorting, max_radius if max_radius is not None else -1.0, int(K),
-                                            bool(tf_compatible), direction is not None)
+    if max_bin_dims < 2:
+        raise ValueError("BinnedSelectKnnOp expects at least 2 binning dimensions.")
+    dir_dev = None if direction is None else direction.to(device=dev, dtype=torch.int32).contiguous()
+    idx, dist = ops.binned_select_knn_pipeline(coords, rs_dev, dir_dev, int(K), n_bins, max_bin_dims,
+                                               bool(tf_compatible), max_radius)
     if not gl.knn_ops_use_tf_gradients:
         return idx, dist
 

@@ -40,6 +40,7 @@ struct KnnParams {
     const int *n_bins;
     const float *bin_width;
     const int *sorting;  // may be null
+    const float *shift;  // may be null: what the binning subtracted from the binned coordinates
     int *out_idx;
     float *out_dist;
     float radius_sq;  // < 0: no radius
@@ -194,6 +195,25 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
         const int nb_last = nb[B - 1], qb_last = qb[B - 1];
         const float bw = p.bin_width[0];
 
+        // Position of the query inside its own bin, in bin widths: to_lower[i] is a
+        // lower bound of its distance to the bin's lower edge, to_upper[i] to the
+        // upper edge (both 0 when the binning shift is unknown). They tighten the
+        // lower bound of the distance to neighbouring bins used for pruning.
+        float to_lower[kMaxBinDims], to_upper[kMaxBinDims];
+#pragma unroll
+        for (int i = 0; i < kMaxBinDims; ++i) {
+            to_lower[i] = 0.f;
+            to_upper[i] = 0.f;
+            if (i < B && p.shift) {
+                const float frac = (qrow[i] - p.shift[i]) / bw - (float)qb[i];
+                if (frac >= 0.f && frac <= 1.f) {
+                    to_lower[i] = fmaxf(frac - 1e-3f, 0.f);
+                    to_upper[i] = fmaxf(1.f - frac - 1e-3f, 0.f);
+                }
+            }
+        }
+        const float tl_last = to_lower[B - 1], tu_last = to_upper[B - 1];
+
         const bool has_radius = p.radius_sq >= 0.f;
         const int kth_lane = (Kn - 1) & (kWave - 1);
         const int kth_level = (Kn - 1) >> 6;
@@ -216,8 +236,8 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                 const int slot = slot0 + lane;
                 // Nothing farther than `reach2` can still enter the list (K-th distance
                 // once the list is full, the radius cut otherwise). A bin at offset o
-                // from the query's bin is at least (|o|-1) bin widths away in that
-                // dimension, whatever the query's position inside its own bin.
+                // from the query's bin is at least (|o|-1) bin widths, plus the
+                // distance to the facing edge of the own bin, away in that dimension.
                 float reach2 = thr == kEmptyKey ? 3.0e38f : __uint_as_float((uint32_t)(thr >> 32));
                 if (has_radius) reach2 = fminf(reach2, p.radius_sq);
                 if (slot < n_slots) {
@@ -243,7 +263,9 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                             inside = inside && k >= 0 && k < nb[i];
                             on_face = on_face || off[i] == d || off[i] == -d;
                             cell = cell * nb[i] + k;
-                            const float g = (float)max(abs(off[i]) - 1, 0) * bw;
+                            const int o = off[i];
+                            const float g = o > 0 ? ((float)(o - 1) + to_upper[i]) * bw
+                                                  : (o < 0 ? ((float)(-o - 1) + to_lower[i]) * bw : 0.f);
                             gap2 += g * g;
                         }
                     }
@@ -251,21 +273,21 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                     if (on_face || d == 0) {  // the whole run of the last dimension
                         lo = qb_last - d;
                         hi = second ? lo - 1 : qb_last + d;
-                        // bins of the run that are provably too far are cut off: keep
-                        // |offset| <= sqrt(rest)/bw + 1 (one extra bin of slack)
+                        // bins of the run that are provably too far are cut off
+                        // (bound generous by 0.1 % and a thousandth of a bin)
                         const float rest = reach2 - 0.999f * gap2;
                         if (rest < 0.f) {
                             hi = lo - 1;
                         } else if (rest < 1.0e37f) {
-                            const int span = (int)(sqrtf(rest) / bw) + 2;
-                            lo = max(lo, qb_last - span);
-                            hi = min(hi, qb_last + span);
+                            const float span = sqrtf(rest) / bw * 1.001f + 1.001f;
+                            lo = max(lo, qb_last - (int)(span - tl_last));
+                            hi = min(hi, qb_last + (int)(span - tu_last));
                         }
                     } else {  // interior row: only the two end caps
                         lo = second ? qb_last + d : qb_last - d;
                         hi = lo;
                         if (lo < 0 || lo >= nb_last) hi = lo - 1;
-                        const float g = (float)(d - 1) * bw;
+                        const float g = ((float)(d - 1) + (second ? tu_last : tl_last)) * bw;
                         if (0.999f * (gap2 + g * g) > reach2) hi = lo - 1;
                     }
                     lo = max(lo, 0);
@@ -392,7 +414,7 @@ extern "C" {
 int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, const int *d_direction,
                                 const int *d_dim_bin_idx, const int *d_bin_boundaries,
                                 const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
-                                float max_radius, int *d_indices, float *d_dist, int n_vert, int n_neigh,
+                                const float *d_shift, float max_radius, int *d_indices, float *d_dist, int n_vert, int n_neigh,
                                 int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
                                 int use_direction, hgc_stream_t stream) {
     // same conditions as the reference op (binned_select_knn_kernel.cc:336-352)
@@ -422,6 +444,7 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
     p.n_bins = d_n_bins;
     p.bin_width = d_bin_width;
     p.sorting = d_sorting;
+    p.shift = d_shift;
     p.out_idx = d_indices;
     p.out_dist = d_dist;
     p.radius_sq = max_radius > 0.f ? max_radius * max_radius : -1.f;
@@ -442,7 +465,7 @@ int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int 
                           int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat, int use_direction,
                           hgc_stream_t stream) {
     return hgc_binned_select_knn_fused(d_coord, d_bin_idx, d_direction, d_dim_bin_idx, d_bin_boundaries,
-                                       d_n_bins, d_bin_width, nullptr, -1.f, d_indices, d_dist, n_vert,
+                                       d_n_bins, d_bin_width, nullptr, nullptr, -1.f, d_indices, d_dist, n_vert,
                                        n_neigh, n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction,
                                        stream);
 }

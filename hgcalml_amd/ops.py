@@ -127,10 +127,27 @@ def binned_select_knn_fused(coords, bin_idx, dim_bin_idx, bin_boundaries, n_bins
     idx = torch.empty((n, n_neighbours), dtype=torch.int32, device=dev)
     dist = torch.empty((n, n_neighbours), dtype=torch.float32, device=dev)
     check(lib.hgc_binned_select_knn_fused(p(coords), p(bin_idx), p(direction), p(dim_bin_idx), p(bin_boundaries),
-                                          p(n_bins), p(bin_width), p(sorting),
+                                          p(n_bins), p(bin_width), p(sorting), None,
                                           float(max_radius) if max_radius is not None else -1.0, p(idx), p(dist), n,
                                           int(n_neighbours), c, n_bins.numel(), bin_boundaries.numel(),
                                           int(tf_compatible), int(use_direction), stream()))
+    return idx, dist
+
+
+def binned_select_knn_pipeline(coords, row_splits, direction, n_neighbours, n_bins, max_bin_dims, tf_compatible,
+                               max_radius):
+    """the whole BinnedSelectKnn wrapper in one C call (inputs/outputs in the caller's order)"""
+    dev = require_device(coords, row_splits, direction)
+    n, c = coords.shape
+    idx = torch.empty((n, n_neighbours), dtype=torch.int32, device=dev)
+    dist = torch.empty((n, n_neighbours), dtype=torch.float32, device=dev)
+    nbytes = lib.hgc_binned_select_knn_pipeline_workspace_bytes(n, c, row_splits.numel(), int(n_bins), int(max_bin_dims),
+                                                                int(direction is not None))
+    ws = workspace(nbytes, dev)
+    check(lib.hgc_binned_select_knn_pipeline(p(coords), p(row_splits), p(direction), n, c, row_splits.numel(),
+                                             int(n_neighbours), int(n_bins), int(max_bin_dims), int(tf_compatible),
+                                             float(max_radius) if max_radius is not None else -1.0, p(idx), p(dist),
+                                             p(ws), ws.numel(), stream()))
     return idx, dist
 
 

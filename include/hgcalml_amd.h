@@ -145,15 +145,33 @@ int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int 
  *   d_sorting (may be NULL) [n_vert]: original index of each sorted point; when
  *     given, neighbour indices are reported in original index space, rows are
  *     written at their original position and ties are broken by original index;
+ *   d_shift (may be NULL) [n_bin_dim]: what the binning subtracted from the
+ *     binned coordinates (hgc_bin_setup); only sharpens the pruning of far bins;
  *   max_radius > 0: neighbours with distance^2 > max_radius^2 are dropped. */
 int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, const int *d_direction,
                                 const int *d_dim_bin_idx, const int *d_bin_boundaries,
                                 const int *d_n_bins, const float *d_bin_width,
-                                const int *d_sorting, float max_radius,
+                                const int *d_sorting, const float *d_shift, float max_radius,
                                 int *d_indices, float *d_dist,
                                 int n_vert, int n_neigh, int n_coords, int n_bin_dim,
                                 int n_bboundaries, int tf_compat, int use_direction,
                                 hgc_stream_t stream);
+
+/* The whole wrapper modules/binned_select_knn_op.py:33-104 in one call:
+ * bounding box and grid (n_bins_scalar bins along the widest of the first
+ * min(max_bin_dims, n_coords) coordinates), bin assignment, stable sort into bin
+ * order, gather of the sorted inputs, search and un-sort. Inputs and outputs are
+ * in the caller's order and index space: d_coords [n_vert, n_coords],
+ * d_row_splits [n_rs], d_direction [n_vert] or NULL; d_indices, d_dist
+ * [n_vert, n_neigh]. No host synchronisation. */
+size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, int n_rs,
+                                                      int n_bins_scalar, int max_bin_dims,
+                                                      int use_direction);
+int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_splits,
+                                   const int *d_direction, int n_vert, int n_coords, int n_rs,
+                                   int n_neigh, int n_bins_scalar, int max_bin_dims, int tf_compat,
+                                   float max_radius, int *d_indices, float *d_dist,
+                                   void *workspace, size_t workspace_bytes, hgc_stream_t stream);
 
 /* out[i] = v < 0 ? v : replacements[v]; entries with v >= n_replacements are
  * left untouched. Replaces IndexReplacerOpFunctor
