@@ -47,7 +47,7 @@ def _compile(src):
 def build(verbose=True, sources=None):
     """Compile `sources` (default: all) and link every object into the library."""
     sources = sources or SOURCES
-    with ThreadPoolExecutor(max_workers=min(4, len(sources))) as pool:
+    with ThreadPoolExecutor(max_workers=min(6, len(sources))) as pool:
         list(pool.map(_compile, sources))
     objs = [os.path.join(CSRC, os.path.splitext(src)[0] + ".o") for src in SOURCES]
     missing = [o for o in objs if not os.path.exists(o)]

@@ -16,7 +16,7 @@
 // reference CPU order (slot order, resp. ascending (vertex, slot) per target
 // through the inverse neighbour index), which makes them bit-identical to it;
 // no float atomics anywhere.
-#include "hgc_common.hpp"
+#include "accumulate_rows.hpp"
 
 #include <cstdlib>
 #include <cstring>
@@ -30,66 +30,10 @@ int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
 
 namespace {
 
+using namespace acc;
+
 // ------------------------------------------------------------------ forward
 
-template <int VEC>
-struct FeatVec;
-template <>
-struct FeatVec<4> {
-    using type = float4;
-};
-template <>
-struct FeatVec<1> {
-    using type = float;
-};
-
-template <int VEC>
-__device__ __forceinline__ void load_vec(const float *p, float (&x)[VEC]) {
-    if constexpr (VEC == 4) {
-        const float4 v = *reinterpret_cast<const float4 *>(p);
-        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
-    } else if constexpr (VEC == 2) {
-        const float2 v = *reinterpret_cast<const float2 *>(p);
-        x[0] = v.x; x[1] = v.y;
-    } else {
-        x[0] = *p;
-    }
-}
-
-template <int VEC>
-__device__ __forceinline__ void load_vec_i(const int *p, int (&x)[VEC]) {
-    if constexpr (VEC == 4) {
-        const int4 v = *reinterpret_cast<const int4 *>(p);
-        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
-    } else if constexpr (VEC == 2) {
-        const int2 v = *reinterpret_cast<const int2 *>(p);
-        x[0] = v.x; x[1] = v.y;
-    } else {
-        x[0] = *p;
-    }
-}
-
-template <int VEC>
-__device__ __forceinline__ void store_vec(float *p, const float (&x)[VEC]) {
-    if constexpr (VEC == 4) {
-        *reinterpret_cast<float4 *>(p) = make_float4(x[0], x[1], x[2], x[3]);
-    } else if constexpr (VEC == 2) {
-        *reinterpret_cast<float2 *>(p) = make_float2(x[0], x[1]);
-    } else {
-        *p = x[0];
-    }
-}
-
-template <int VEC>
-__device__ __forceinline__ void store_vec_i(int *p, const int (&x)[VEC]) {
-    if constexpr (VEC == 4) {
-        *reinterpret_cast<int4 *>(p) = make_int4(x[0], x[1], x[2], x[3]);
-    } else if constexpr (VEC == 2) {
-        *reinterpret_cast<int2 *>(p) = make_int2(x[0], x[1]);
-    } else {
-        *p = x[0];
-    }
-}
 
 constexpr int kUnroll = 8;
 
@@ -190,53 +134,6 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
 // access against the size of the matrix. Chunks of U neighbour slots without
 // padding take a branch-free path with all U row loads in flight.
 
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ int wave_vertex() {
-    const int tile = xcd_contiguous_block(blockIdx.x, gridDim.x);
-    return __builtin_amdgcn_readfirstlane(tile * 4 + (int)(threadIdx.x >> 6));
-}
-
-// A dense [rows, cols] matrix of 4-byte elements seen through a raw buffer
-// descriptor (stride 0, num_records = size in bytes, gfx9 data format word).
-struct RowMatrix {
-    __amdgpu_buffer_rsrc_t rsrc;
-    uint32_t row_bytes;
-    __device__ __forceinline__ RowMatrix(const void *base, size_t rows, size_t cols)
-        : rsrc(__builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)(uint32_t)(rows * cols * 4u),
-                                                 0x00020000)),
-          row_bytes((uint32_t)cols * 4u) {}
-
-    // x[0..VEC) = M[row, col .. col+VEC) with col = lane_bytes/4 (+ col_bytes/4)
-    template <int VEC>
-    __device__ __forceinline__ void load(int row, uint32_t lane_bytes, uint32_t (&x)[VEC]) const {
-        const int soff = (int)((uint32_t)row * row_bytes);
-        if constexpr (VEC == 4) {
-            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_bytes, soff, 0);
-            x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
-        } else if constexpr (VEC == 2) {
-            const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_bytes, soff, 0);
-            x[0] = v.x; x[1] = v.y;
-        } else {
-            x[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_bytes, soff, 0);
-        }
-    }
-    template <int VEC>
-    __device__ __forceinline__ void load(int row, uint32_t lane_bytes, float (&x)[VEC]) const {
-        uint32_t r[VEC];
-        load<VEC>(row, lane_bytes, r);
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) x[e] = __uint_as_float(r[e]);
-    }
-    template <int VEC>
-    __device__ __forceinline__ void load(int row, uint32_t lane_bytes, int (&x)[VEC]) const {
-        uint32_t r[VEC];
-        load<VEC>(row, lane_bytes, r);
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) x[e] = (int)r[e];
-    }
-};
 
 // one slot of the forward recurrence for the VEC features of this lane
 template <int VEC, bool MAX, bool SEED>
@@ -368,15 +265,6 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
     }
 }
 
-// x / K for 0 <= x < 2^31 without an integer divide
-struct FastDiv {
-    uint32_t magic;  // 0: K is a power of two
-    int shift;
-};
-
-__device__ __forceinline__ int fast_div(int x, const FastDiv d) {
-    return d.magic == 0 ? (int)((uint32_t)x >> d.shift) : (int)(__umulhi((uint32_t)x, d.magic) >> d.shift);
-}
 
 // one inverse-list entry of the feature gradient for the VEC features of this lane;
 // `mi` holds arg-max indices compared with `key` = target vertex, or (SLOTS)
@@ -399,18 +287,6 @@ __device__ __forceinline__ void fgrad_entry(const float (&gm)[VEC], const float 
     }
 }
 
-// VEC arg-max slot bytes of row `row`, columns lane_col .. lane_col+VEC
-template <int VEC>
-__device__ __forceinline__ void load_slots(__amdgpu_buffer_rsrc_t rsrc, int row, uint32_t row_bytes, uint32_t lane_col,
-                                           int (&x)[VEC]) {
-    const int soff = (int)((uint32_t)row * row_bytes);
-    uint32_t packed;
-    if constexpr (VEC == 4) packed = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_col, soff, 0);
-    else if constexpr (VEC == 2) packed = __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int)lane_col, soff, 0);
-    else packed = __builtin_amdgcn_raw_buffer_load_b8(rsrc, (int)lane_col, soff, 0);
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) x[e] = (int)((packed >> (8 * e)) & 255u);
-}
 
 // Feature slicing across XCDs: the rows this kernel gathers (gradient row +
 // arg-max row of every vertex that names the target) span a window of the
@@ -534,23 +410,6 @@ __global__ __launch_bounds__(256) void feature_grad_wave_kernel(const float *__r
     }
 }
 
-// 32 partial sums per lane in, after the call lane L holds the sum over all 64
-// lanes of value index (L & 31). Fixed butterfly: deterministic summation order.
-__device__ __forceinline__ float transpose_reduce_32(float (&val)[32]) {
-    const int lane = lane_id();
-#pragma unroll
-    for (int h = 16; h >= 1; h >>= 1) {
-        const bool upper = (lane & h) != 0;
-#pragma unroll
-        for (int i = 0; i < h; ++i) {
-            const float a = val[i], b = val[i + h];
-            const float send = upper ? a : b;
-            const float keep = upper ? b : a;
-            val[i] = keep + __shfl_xor(send, h, kWave);
-        }
-    }
-    return val[0] + __shfl_xor(val[0], 32, kWave);
-}
 
 template <int VEC, bool MAX>
 __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__restrict__ g, const float *__restrict__ feat,
@@ -816,30 +675,6 @@ int inverse_key_bits(int n_vert) {
     return bits;
 }
 
-bool is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
-
-// features per lane of the wave-per-vertex kernels: all 64 lanes busy and
-// every access naturally aligned
-int wave_vec(int n_feat, uintptr_t align_or) {
-    if (n_feat % 256 == 0 && (align_or & 15u) == 0) return 4;
-    if (n_feat % 128 == 0 && (align_or & 7u) == 0) return 2;
-    return 1;
-}
-
-FastDiv make_fast_div(int k) {
-    FastDiv d;
-    if (is_pow2(k)) {
-        d.magic = 0;
-        d.shift = 0;
-        while ((1 << d.shift) < k) ++d.shift;
-        return d;
-    }
-    int s = 0;
-    while ((1ll << s) < k) ++s;  // ceil(log2 k) >= 2
-    d.magic = (uint32_t)((1ull << (31 + s)) / (uint32_t)k + 1);
-    d.shift = s - 1;
-    return d;
-}
 
 }  // namespace
 }  // namespace hgc
