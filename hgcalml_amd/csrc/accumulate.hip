@@ -27,6 +27,11 @@
 namespace hgc {
 
 int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
+// accumulate_grad_fused.hip; returns 1 when the shape is not covered
+int launch_accumulate_grad_fused(const float *g, const float *w, const float *feat, const int *maxidx,
+                                 const unsigned char *maxslot, const int *inv_off, const int *inv_slots, float *gw,
+                                 float *gfeat, int n_vert, int K, int F, int g_cols, bool mean_and_max, const int *idx,
+                                 hipStream_t s);
 
 namespace {
 
@@ -802,10 +807,18 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
 
     const bool fits_32bit = (unsigned long long)n_vert * (unsigned long long)(2 * n_feat) * 4ull < (1ull << 32);
     if (n_feat >= kWave && fits_32bit) {  // one wave per vertex, rows addressed through 32-bit buffer offsets
+        const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
+        // both gradients from one gather pass where that kernel covers the shape
+        if (!mean_and_max || use_slots) {
+            const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
+                                                        d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
+                                                        d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat,
+                                                        mean_and_max != 0, d_neigh_indices, s);
+            if (rc <= 0) return rc;  // 1: shape not covered, use the two-kernel path
+        }
         const int vec = wave_vec(n_feat, align_or);
         const dim3 grid(ceil_div(n_vert, 4)), block(256);
         const FastDiv div_k = make_fast_div(n_neigh);
-        const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
 #define HGC_FGW(VEC, MAX, P2, SL)                                                                                      \
     feature_grad_wave_kernel<VEC, MAX, P2, SL><<<fg_grid, block, 0, s>>>(                                              \
         d_grad_from_out_features, d_distances, d_max_feat_indices, d_max_slots, d_inv_offsets, d_inv_slots,            \

@@ -313,8 +313,11 @@ def test_accumulate_slot_table_path(oracle, K, F):
     gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(g), t(w), t(x), t(idx), arg, slots, *inv)
     gw0, gx0 = torch.ops.hgcalml.accumulate_knn_grad(t(g), t(w), t(x), t(idx), arg, *inv)
     assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
-    assert torch.equal(gx, gx0) and torch.equal(gw, gw0)
-    assert (np.abs(gw.cpu().numpy() - rgw) <= grad_tolerance(g, x, idx, w, K)).all()
+    assert torch.equal(gx, gx0)
+    # the two paths reduce the weight gradient's dot products in different orders
+    tol = grad_tolerance(g, x, idx, w, K)
+    assert (np.abs(gw.cpu().numpy() - rgw) <= tol).all() and (np.abs(gw0.cpu().numpy() - rgw) <= tol).all()
+    assert (gw.cpu().numpy()[idx < 0] == 0).all()
 
 
 def test_inverse_neighbour_index_is_ordered():
