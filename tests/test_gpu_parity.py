@@ -353,6 +353,53 @@ def test_accumulate_autograd_chain(oracle):
     assert np.allclose(tx.grad.cpu().numpy() / 3, rgx, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("K,F,half_width", [(64, 128, 2000), (32, 64, 300), (16, 192, 1000), (12, 256, 50)])
+def test_accumulate_local_neighbour_tables(oracle, K, F, half_width):
+    """several thousand vertices whose neighbours lie within +-half_width rows (the
+    shape of the large accumulate workload), with padding, a far neighbour, repeated
+    self references and exact ties mixed in: forward, slot table and gradient"""
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(40 + K + F)
+    n = 512 * 9 + 77          # ragged last block
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    idx = np.empty((n, K), np.int32)
+    for v in range(n):
+        lo, hi = max(0, v - half_width), min(n, v + half_width + 1)
+        cand = np.delete(np.arange(lo, hi), v - lo)
+        idx[v] = np.concatenate([[v], rng.choice(cand, K - 1, replace=False)])
+    idx[600, K // 2:] = -1                 # padding
+    if half_width < 1500:
+        idx[512 * 3 + 5, 3] = n - 1        # a far neighbour
+    idx[512 * 5 + 9, K // 2:] = 512 * 5 + 9   # repeated self references
+    x[512 * 5 + 9] = 40.0
+    idx[512 * 6 + 1, 1:4] = 512 * 6 + 1
+    x[512 * 6 + 1] = -40.0
+    w = np.exp(-rng.random((n, K), dtype=np.float32)).astype(np.float32)
+    # exact ties between slots of one vertex: the later slot has to win
+    w[100, 5] = w[100, 9]
+    x[idx[100, 5]] = x[idx[100, 9]]
+    for mm in (True, False):
+        ref, rarg = oracle.AccumulateLinKnn(w, x, idx, mm)
+        out, arg, slots = torch.ops.hgcalml.accumulate_knn_slots(t(w), t(x), t(idx), 0, mm)
+        assert (bits(out.cpu().numpy()) == bits(ref)).all()
+        if mm:
+            assert (arg.cpu().numpy() == rarg).all()
+            sl = slots.cpu().numpy().astype(np.int64)
+            rows = np.arange(n)[:, None]
+            taken = sl != 255
+            # the slot names the arg-max index, and it is that index's first occurrence in the row
+            assert (idx[rows, np.where(taken, sl, 0)][taken] == rarg[taken]).all()
+            first = (idx[:, :, None] == rarg[:, None, :]).argmax(1)
+            assert (sl[taken] == first[taken]).all()
+            assert taken[np.setdiff1d(np.arange(n), [600])].all()
+    g = rng.standard_normal((n, 2 * F)).astype(np.float32)
+    rgw, rgx = oracle.accumulate_knn_grad_kernel(g, w, x, idx, rarg)
+    inv = ops.inverse_neighbour_index(t(idx))
+    gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(g), t(w), t(x), t(idx), arg, slots, *inv)
+    assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
+    assert (np.abs(gw.cpu().numpy() - rgw) <= grad_tolerance(g, x, idx, w, K)).all()
+
+
 def test_accumulate_cfg4_scaled(oracle):
     c = workloads.cfg4(scale=0.03)
     w = np.exp(-c["distsq"]).astype(np.float32)
