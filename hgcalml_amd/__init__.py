@@ -2,11 +2,12 @@
 
 Public API (same names and signatures as the reference's Python wrappers):
 BinByCoordinates, BinnedSelectKnn, IndexReplacer, AccumulateKnn,
-AccumulateLinKnn, BuildAndAssignCondensatesBinned. All of them need tensors on
+AccumulateLinKnn, AccumulateKnnSumw, AccumulateLinKnnSumw, PushKnn,
+BuildAndAssignCondensatesBinned. All of them need tensors on
 a HIP device and the in-tree libhgcalml_amd.so; there is no CPU path.
 """
 __all__ = ["BinByCoordinates", "BinnedSelectKnn", "IndexReplacer", "AccumulateKnn", "AccumulateLinKnn",
-           "BuildAndAssignCondensatesBinned"]
+           "AccumulateKnnSumw", "AccumulateLinKnnSumw", "PushKnn", "BuildAndAssignCondensatesBinned"]
 
 
 def __getattr__(name):
@@ -20,6 +21,9 @@ def __getattr__(name):
             "IndexReplacer": "index_replacer_op",
             "AccumulateKnn": "accknn_op",
             "AccumulateLinKnn": "accknn_op",
+            "AccumulateKnnSumw": "accknn_op",
+            "AccumulateLinKnnSumw": "accknn_op",
+            "PushKnn": "push_knn_op",
             "BuildAndAssignCondensatesBinned": "assign_condensate_op",
         }[name]
         return getattr(importlib.import_module("." + mod, __name__), name)

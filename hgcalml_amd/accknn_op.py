@@ -61,3 +61,25 @@ def AccumulateKnn(distances, features, indices, mean_and_max=True, force_tf=Fals
     if (not gl.acc_ops_use_tf_gradients) and (not force_tf):
         return _AccumulateFn.apply(weights, features, indices, bool(mean_and_max))
     return _torch_composition(weights, features, indices, mean_and_max)
+
+
+def _sumw(acc, x, features, indices, mean_and_max):
+    # modules/GravNetLayersRagged.py:35-62: a column of ones rides along and
+    # collects the accumulated weight; divide_no_nan
+    origshape = features.shape[1]
+    features = torch.cat([features, torch.ones_like(features[:, 0:1])], dim=1)
+    f, midx = acc(x, features, indices, mean_and_max=mean_and_max)
+    fmean = f[:, :origshape]
+    fnorm = f[:, origshape:origshape + 1]
+    fmean = torch.where(fnorm == 0, torch.zeros_like(fmean), fmean / fnorm)
+    if mean_and_max:
+        fmean = torch.cat([fmean, f[:, origshape + 1:-1]], dim=1)
+    return fmean, midx
+
+
+def AccumulateKnnSumw(distances, features, indices, mean_and_max=False):
+    return _sumw(AccumulateKnn, distances, features, indices, mean_and_max)
+
+
+def AccumulateLinKnnSumw(weights, features, indices, mean_and_max=False):
+    return _sumw(AccumulateLinKnn, weights, features, indices, mean_and_max)

@@ -20,6 +20,26 @@ def _BinnedSelectKnn(K, coords, bin_idx, dim_bin_idx, bin_boundaries, n_bins, bi
                                                direction, int(K), bool(tf_compatible), use_direction)
 
 
+class _BinnedSelectKnnFn(torch.autograd.Function):
+    """the op with its registered gradient SelectKnnGrad
+    (modules/binned_select_knn_op.py:107-118): distances are differentiable
+    w.r.t. the coordinates, indices are not"""
+
+    @staticmethod
+    def forward(ctx, coords, rs_dev, dir_dev, K, n_bins, max_bin_dims, tf_compatible, max_radius):
+        idx, dist = ops.binned_select_knn_pipeline(coords, rs_dev, dir_dev, K, n_bins, max_bin_dims, tf_compatible,
+                                                   max_radius)
+        ctx.save_for_backward(coords, idx, dist)
+        ctx.mark_non_differentiable(idx)
+        return idx, dist
+
+    @staticmethod
+    def backward(ctx, _grad_idx, grad_dist):
+        coords, idx, dist = ctx.saved_tensors
+        grad_coords = torch.ops.hgcalml.select_knn_grad(grad_dist.contiguous(), idx, dist, coords)
+        return grad_coords, None, None, None, None, None, None, None
+
+
 def default_n_bins(first_event_size, K, max_bin_dims):
     # float32 pow, truncation, clamp to [5, 30] (modules/binned_select_knn_op.py:59-63)
     v = torch.pow(torch.tensor(float(first_event_size), dtype=torch.float32) / torch.tensor(K / 32, dtype=torch.float32),
@@ -67,10 +87,11 @@ def BinnedSelectKnn(K, coords, row_splits, direction=None, n_bins=None, max_bin_
     if max_bin_dims < 2:
         raise ValueError("BinnedSelectKnnOp expects at least 2 binning dimensions.")
     dir_dev = None if direction is None else direction.to(device=dev, dtype=torch.int32).contiguous()
+    if not gl.knn_ops_use_tf_gradients:
+        return _BinnedSelectKnnFn.apply(coords, rs_dev, dir_dev, int(K), n_bins, max_bin_dims, bool(tf_compatible),
+                                        max_radius)
     idx, dist = ops.binned_select_knn_pipeline(coords, rs_dev, dir_dev, int(K), n_bins, max_bin_dims,
                                                bool(tf_compatible), max_radius)
-    if not gl.knn_ops_use_tf_gradients:
-        return idx, dist
 
     # differentiable re-computation of the distances (modules/binned_select_knn_op.py:97-104)
     safe = idx.clamp(min=0).to(torch.int64)

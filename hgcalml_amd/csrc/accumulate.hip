@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
                                                              const int *__restrict__ idx, float *__restrict__ out,
                                                              int *__restrict__ out_maxidx,
                                                              unsigned char *__restrict__ out_maxslot, int n_vert, int K,
-                                                             int F, int out_cols) {
+                                                             int F, int out_cols, float kf) {
     const int tpv = F / VEC;  // threads per vertex
     const long long t = (long long)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
     const int v = (int)(t / tpv);
@@ -102,7 +102,6 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
         }
     }
 
-    const float kf = (float)K;
     float mean[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) mean[e] = sum[e] / kf;
@@ -167,13 +166,12 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                                                                   const int *__restrict__ idx, float *__restrict__ out,
                                                                   int *__restrict__ out_maxidx,
                                                                   unsigned char *__restrict__ out_maxslot, int n_vert,
-                                                                  int K, int F, int out_cols) {
+                                                                  int K, int F, int out_cols, float kf) {
     constexpr int U = VEC == 4 ? 8 : 16;
     const int v = wave_vertex();
     if (v >= n_vert) return;
     const int *irow = idx + (size_t)v * K;
     const float *wrow = w + (size_t)v * K;
-    const float kf = (float)K;
     const RowMatrix X(feat, n_vert, F);
     int first_self = -1;  // first slot that names the vertex itself (wave-uniform, scalar ALU)
 
@@ -307,7 +305,7 @@ __global__ __launch_bounds__(256) void feature_grad_wave_kernel(const float *__r
                                                                 const int *__restrict__ inv_off,
                                                                 const int *__restrict__ inv_slots,
                                                                 float *__restrict__ gfeat, int n_vert, int K, int F,
-                                                                int g_cols, const FastDiv div_k, int n_slices) {
+                                                                int g_cols, const FastDiv div_k, int n_slices, float kf) {
     constexpr int U = VEC == 4 ? 4 : 8;
     int m, first_block = 0;
     if (n_slices == 1) {
@@ -320,8 +318,7 @@ __global__ __launch_bounds__(256) void feature_grad_wave_kernel(const float *__r
         m = __builtin_amdgcn_readfirstlane(tile * 4 + (int)(threadIdx.x >> 6));
     }
     if (m >= n_vert) return;
-    const float kf = (float)K;
-    const float inv_k = 1.f / kf;  // exact when K is a power of two
+    const float inv_k = 1.f / kf;  // exact when the divisor is a power of two
     const int begin = inv_off[m], end = inv_off[m + 1];
     const RowMatrix G(g, n_vert, g_cols);
     const RowMatrix MI(maxidx, (MAX && !SLOTS) ? n_vert : 0, F);
@@ -420,14 +417,14 @@ template <int VEC, bool MAX>
 __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__restrict__ g, const float *__restrict__ feat,
                                                                const int *__restrict__ maxidx, const int *__restrict__ idx,
                                                                float *__restrict__ gw, int n_vert, int K, int F,
-                                                               int g_cols) {
+                                                               int g_cols, float kf) {
     constexpr int U = 8;
     constexpr int G = 16;  // slots per reduction group: 16 mean sums + 16 max sums = 32 values
     const int m = wave_vertex();
     if (m >= n_vert) return;
     const int lane = lane_id();
     const int *irow = idx + (size_t)m * K;
-    const double inv_k = 1.0 / (double)(float)K;
+    const double inv_k = 1.0 / (double)kf;
     const RowMatrix X(feat, n_vert, F);
 
     for (int l0 = 0; l0 < K; l0 += G) {
@@ -517,15 +514,14 @@ __global__ __launch_bounds__(256) void feature_grad_kernel(const float *__restri
                                                            const int *__restrict__ inv_off,
                                                            const int *__restrict__ inv_slots,
                                                            float *__restrict__ gfeat, int n_vert, int K, int F,
-                                                           int g_cols) {
+                                                           int g_cols, float kf) {
     const int tpv = F / VEC;
     const long long t = (long long)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
     const int m = (int)(t / tpv);
     if (m >= n_vert) return;
     const int f0 = (int)(t - (long long)m * tpv) * VEC;
 
-    const float kf = (float)K;
-    const float inv_k = 1.f / kf;  // exact when K is a power of two
+    const float inv_k = 1.f / kf;  // exact when the divisor is a power of two
     float acc[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
@@ -601,7 +597,7 @@ template <int VEC, bool MAX>
 __global__ __launch_bounds__(256) void weight_grad_kernel(const float *__restrict__ g, const float *__restrict__ feat,
                                                           const int *__restrict__ maxidx, const int *__restrict__ idx,
                                                           float *__restrict__ gw, int n_vert, int K, int F, int g_cols,
-                                                          int tpv) {
+                                                          int tpv, float kf) {
     const long long t = (long long)xcd_contiguous_block(blockIdx.x, gridDim.x) * blockDim.x + threadIdx.x;
     const int m = (int)(t / tpv);
     const int sub = (int)(t - (long long)m * tpv);
@@ -611,7 +607,7 @@ __global__ __launch_bounds__(256) void weight_grad_kernel(const float *__restric
     // features owned by this thread: f = sub*VEC + e + i*tpv*VEC
     const int stride = tpv * VEC;
     const int *irow = idx + (size_t)mm * K;
-    const double inv_k = 1.0 / (double)(float)K;
+    const double inv_k = 1.0 / (double)kf;
 
     for (int l0 = 0; l0 < K; l0 += kUnroll) {
         float pm[kUnroll], px[kUnroll];
@@ -684,14 +680,13 @@ int inverse_key_bits(int n_vert) {
 }  // namespace
 }  // namespace hgc
 
-using namespace hgc;
+namespace hgc {
 
-extern "C" {
-
-int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
-                             int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat, int n_out_feat, int n_moments,
-                       int mean_and_max, hgc_stream_t stream) {
-    (void)n_moments;  // carried by the reference op, never used by its kernels
+// Forward pass shared by accumulate_knn (divisor = K) and the feature gradient of
+// push_knn (divisor = 1): out = (sum over the slots of w * feat[idx]) / divisor.
+int accumulate_forward(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
+                       int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat,
+                       int n_out_feat, int mean_and_max, float divisor, hgc_stream_t stream) {
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_out_feat == n_feat * (mean_and_max ? 2 : 1), "n_out_feat must be n_feat * (mean_and_max ? 2 : 1)");
     HGC_REQUIRE((long long)n_vert * std::max(n_neigh, 2 * n_feat) < (1ll << 31), "tensor too large for int32 indexing");
@@ -709,7 +704,7 @@ int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, cons
         const dim3 grid(ceil_div(n_vert, 4)), block(256);
 #define HGC_FWD(VEC, MAX)                                                                                         \
     accumulate_fwd_wave_kernel<VEC, MAX><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, \
-                                                               d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat)
+                                                               d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor)
         if (mean_and_max) {
             if (vec == 4) HGC_FWD(4, true); else if (vec == 2) HGC_FWD(2, true); else HGC_FWD(1, true);
         } else {
@@ -724,19 +719,33 @@ int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, cons
     if (vec4) {
         if (mean_and_max)
             accumulate_fwd_kernel<4, true><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                  d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
+                                                                  d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor);
         else
             accumulate_fwd_kernel<4, false><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                   d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
+                                                                   d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor);
     } else {
         if (mean_and_max)
             accumulate_fwd_kernel<1, true><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                  d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
+                                                                  d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor);
         else
             accumulate_fwd_kernel<1, false><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs,
-                                                                   d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat);
+                                                                   d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor);
     }
     return check_launch("accumulate_fwd_kernel");
+}
+
+}  // namespace hgc
+
+using namespace hgc;
+
+extern "C" {
+
+int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
+                             int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat,
+                             int n_out_feat, int n_moments, int mean_and_max, hgc_stream_t stream) {
+    (void)n_moments;  // carried by the reference op, never used by its kernels
+    return accumulate_forward(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, d_out_maxslots, n_vert, n_neigh,
+                              n_feat, n_out_feat, mean_and_max, (float)n_neigh, stream);
 }
 
 int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
@@ -783,33 +792,40 @@ int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh, int 
     return check_launch("inverse_offsets");
 }
 
-int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
-                                  const int *d_max_feat_indices, const unsigned char *d_max_slots,
-                                  const int *d_neigh_indices, const int *d_inv_offsets, const int *d_inv_slots,
-                                  float *d_out_grad_distances, float *d_out_grad_features, int n_vert, int n_neigh,
-                                  int n_feat, int n_grad_from_out_feat, int n_moments, int mean_and_max,
-                                  hgc_stream_t stream) {
-    (void)n_moments;
+}  // extern "C"
+
+namespace hgc {
+
+// Gradient shared by accumulate_knn_grad (divisor = K) and push_knn (divisor = 1).
+// Either output may be null: the weight gradient needs neither the inverse index
+// nor the weights, the feature gradient needs neither the features nor the
+// neighbour table.
+int accumulate_gradient(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
+                        const int *d_max_feat_indices, const unsigned char *d_max_slots, const int *d_neigh_indices,
+                        const int *d_inv_offsets, const int *d_inv_slots, float *d_out_grad_distances,
+                        float *d_out_grad_features, int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
+                        int mean_and_max, float divisor, hgc_stream_t stream) {
+    const bool want_w = d_out_grad_distances != nullptr, want_f = d_out_grad_features != nullptr;
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_grad_from_out_feat == n_feat * (mean_and_max ? 2 : 1),
                 "gradient width must be n_feat * (mean_and_max ? 2 : 1)");
     HGC_REQUIRE((long long)n_vert * std::max(n_neigh, 2 * n_feat) < (1ll << 31), "tensor too large for int32 indexing");
     if (n_vert == 0) return HGC_OK;
-    HGC_REQUIRE(d_grad_from_out_features && d_distances && d_feat && d_neigh_indices && d_inv_offsets &&
-                    d_inv_slots && d_out_grad_distances && d_out_grad_features,
-                "null pointer");
+    HGC_REQUIRE(d_grad_from_out_features && (want_w || want_f), "null pointer");
+    HGC_REQUIRE(!want_w || (d_feat && d_neigh_indices), "null pointer");
+    HGC_REQUIRE(!want_f || (d_distances && d_inv_offsets && d_inv_slots), "null pointer");
     HGC_REQUIRE(!mean_and_max || d_max_feat_indices, "mean_and_max needs d_max_feat_indices");
     hipStream_t s = as_stream(stream);
     const uintptr_t align_or = reinterpret_cast<uintptr_t>(d_grad_from_out_features) | reinterpret_cast<uintptr_t>(d_feat) |
                                reinterpret_cast<uintptr_t>(d_max_feat_indices) |
                                reinterpret_cast<uintptr_t>(d_out_grad_features);
-    const bool pow2k = is_pow2(n_neigh);
+    const bool pow2k = divisor == (float)(int)divisor && is_pow2((int)divisor);
 
     const bool fits_32bit = (unsigned long long)n_vert * (unsigned long long)(2 * n_feat) * 4ull < (1ull << 32);
     if (n_feat >= kWave && fits_32bit) {  // one wave per vertex, rows addressed through 32-bit buffer offsets
         const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
         // both gradients from one gather pass where that kernel covers the shape
-        if (!mean_and_max || use_slots) {
+        if (want_w && want_f && divisor == (float)n_neigh && (!mean_and_max || use_slots)) {
             const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
                                                         d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
                                                         d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat,
@@ -822,7 +838,7 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
 #define HGC_FGW(VEC, MAX, P2, SL)                                                                                      \
     feature_grad_wave_kernel<VEC, MAX, P2, SL><<<fg_grid, block, 0, s>>>(                                              \
         d_grad_from_out_features, d_distances, d_max_feat_indices, d_max_slots, d_inv_offsets, d_inv_slots,            \
-        d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat, div_k, n_slices)
+        d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat, div_k, n_slices, divisor)
 #define HGC_FGW_V(VEC)                                                                                   \
     do {                                                                                                 \
         if (mean_and_max && use_slots) { if (pow2k) HGC_FGW(VEC, true, true, true); else HGC_FGW(VEC, true, false, true); } \
@@ -839,15 +855,17 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
         const int fg_vec = n_slices == 1 ? vec : wave_vec(n_feat / 2, align_or);
         const int tiles = ceil_div(n_vert, 4);
         const dim3 fg_grid(n_slices == 1 ? tiles : kNumXcd * ceil_div(tiles, kNumXcd / n_slices));
-        if (fg_vec == 4) HGC_FGW_V(4); else if (fg_vec == 2) HGC_FGW_V(2); else HGC_FGW_V(1);
+        if (want_f) {
+            if (fg_vec == 4) HGC_FGW_V(4); else if (fg_vec == 2) HGC_FGW_V(2); else HGC_FGW_V(1);
+        }
 #undef HGC_FGW_V
 #undef HGC_FGW
         int rc = check_launch("feature_grad_wave_kernel");
-        if (rc) return rc;
+        if (rc || !want_w) return rc;
 #define HGC_WGW(VEC, MAX)                                                                                       \
     weight_grad_wave_kernel<VEC, MAX><<<grid, block, 0, s>>>(d_grad_from_out_features, d_feat, d_max_feat_indices, \
                                                             d_neigh_indices, d_out_grad_distances, n_vert, n_neigh, \
-                                                            n_feat, n_grad_from_out_feat)
+                                                            n_feat, n_grad_from_out_feat, divisor)
         if (mean_and_max) {
             if (vec == 4) HGC_WGW(4, true); else if (vec == 2) HGC_WGW(2, true); else HGC_WGW(1, true);
         } else {
@@ -860,13 +878,13 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
     const bool vec4 = (n_feat % 4 == 0) && (align_or & 15u) == 0;
 
     // ---- feature gradient ----
-    {
+    if (want_f) {
         const long long threads = (long long)n_vert * (vec4 ? n_feat / 4 : n_feat);
         const dim3 grid(ceil_div(threads, 256)), block(256);
 #define HGC_FG(VEC, MAX, P2)                                                                                      \
     feature_grad_kernel<VEC, MAX, P2><<<grid, block, 0, s>>>(d_grad_from_out_features, d_distances, d_max_feat_indices, \
                                                             d_inv_offsets, d_inv_slots, d_out_grad_features, n_vert, \
-                                                            n_neigh, n_feat, n_grad_from_out_feat)
+                                                            n_neigh, n_feat, n_grad_from_out_feat, divisor)
         if (vec4) {
             if (mean_and_max) { if (pow2k) HGC_FG(4, true, true); else HGC_FG(4, true, false); }
             else              { if (pow2k) HGC_FG(4, false, true); else HGC_FG(4, false, false); }
@@ -880,7 +898,7 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
     }
 
     // ---- weight gradient ----
-    {
+    if (want_w) {
         // threads per vertex: largest power of two <= min(64, F/VEC)
         const int vec = vec4 ? 4 : 1;
         int tpv = 1;
@@ -891,23 +909,41 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
             if (mean_and_max)
                 weight_grad_kernel<4, true><<<grid, block, 0, s>>>(d_grad_from_out_features, d_feat, d_max_feat_indices,
                                                                    d_neigh_indices, d_out_grad_distances, n_vert, n_neigh,
-                                                                   n_feat, n_grad_from_out_feat, tpv);
+                                                                   n_feat, n_grad_from_out_feat, tpv, divisor);
             else
                 weight_grad_kernel<4, false><<<grid, block, 0, s>>>(d_grad_from_out_features, d_feat, d_max_feat_indices,
                                                                     d_neigh_indices, d_out_grad_distances, n_vert, n_neigh,
-                                                                    n_feat, n_grad_from_out_feat, tpv);
+                                                                    n_feat, n_grad_from_out_feat, tpv, divisor);
         } else {
             if (mean_and_max)
                 weight_grad_kernel<1, true><<<grid, block, 0, s>>>(d_grad_from_out_features, d_feat, d_max_feat_indices,
                                                                    d_neigh_indices, d_out_grad_distances, n_vert, n_neigh,
-                                                                   n_feat, n_grad_from_out_feat, tpv);
+                                                                   n_feat, n_grad_from_out_feat, tpv, divisor);
             else
                 weight_grad_kernel<1, false><<<grid, block, 0, s>>>(d_grad_from_out_features, d_feat, d_max_feat_indices,
                                                                     d_neigh_indices, d_out_grad_distances, n_vert, n_neigh,
-                                                                    n_feat, n_grad_from_out_feat, tpv);
+                                                                    n_feat, n_grad_from_out_feat, tpv, divisor);
         }
         return check_launch("weight_grad_kernel");
     }
+    return HGC_OK;
+}
+
+}  // namespace hgc
+
+extern "C" {
+
+int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
+                                  const int *d_max_feat_indices, const unsigned char *d_max_slots,
+                                  const int *d_neigh_indices, const int *d_inv_offsets, const int *d_inv_slots,
+                                  float *d_out_grad_distances, float *d_out_grad_features, int n_vert, int n_neigh,
+                                  int n_feat, int n_grad_from_out_feat, int n_moments, int mean_and_max,
+                                  hgc_stream_t stream) {
+    (void)n_moments;
+    HGC_REQUIRE(n_vert <= 0 || (d_out_grad_distances && d_out_grad_features), "null pointer");
+    return accumulate_gradient(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices, d_max_slots,
+                               d_neigh_indices, d_inv_offsets, d_inv_slots, d_out_grad_distances, d_out_grad_features,
+                               n_vert, n_neigh, n_feat, n_grad_from_out_feat, mean_and_max, (float)n_neigh, stream);
 }
 
 int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,

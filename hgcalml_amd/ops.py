@@ -277,6 +277,63 @@ def accumulate_knn_grad_slots(grad_from_out_features: torch.Tensor, distances: t
                                 max_slots, inv_offsets, inv_slots)
 
 
+# --------------------------------------------------------------------------- ops next to the accumulation
+
+@torch.library.custom_op("hgcalml::select_knn_grad", mutates_args=())
+def select_knn_grad(grad_distances: torch.Tensor, indices: torch.Tensor, distances: torch.Tensor,
+                    coordinates: torch.Tensor) -> torch.Tensor:
+    """modules/compiled/select_knn_grad_module.cc:7-12: gradient of the kNN squared
+    distances w.r.t. the coordinates (the registered gradient of BinnedSelectKnn)"""
+    dev = require_device(grad_distances, indices, distances, coordinates)
+    g, idx, d, x = f32(grad_distances), i32(indices), f32(distances), f32(coordinates)
+    # modules/compiled/select_knn_grad_kernel.cc:66-74
+    if g.dim() != 2 or idx.shape != g.shape or x.dim() != 2 or x.shape[0] != idx.shape[0]:
+        raise ValueError("SelectKnnGradOp expects gradients and indices [N,K] and coordinates [N,C]")
+    n, k = idx.shape
+    inv_offsets, inv_slots = cached_inverse_neighbour_index(indices if indices is idx else idx)
+    out = torch.empty_like(x)
+    check(lib.hgc_select_knn_grad(p(g), p(idx), p(d), p(x), p(inv_offsets), p(inv_slots), p(out), n, k, x.shape[1],
+                                  stream()))
+    return out
+
+
+def _push_checks(weights, features, indices):
+    # modules/compiled/push_knn_kernel.cc:86-91
+    if weights.dim() != 2 or features.dim() != 2 or indices.dim() != 2:
+        raise ValueError("PushKnnOp expects rank 2 tensors")
+    if not (weights.shape[0] == indices.shape[0] == features.shape[0]):
+        raise ValueError("PushKnnOp expects first dimensions of all inputs to match.")
+    if indices.shape[1] != weights.shape[1]:
+        raise ValueError("PushKnnOp expects second dimension of distance and neighbour index tensor to match")
+
+
+@torch.library.custom_op("hgcalml::push_knn", mutates_args=())
+def push_knn(weights: torch.Tensor, features: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    """modules/compiled/push_knn_module.cc:7-11: sums w[v,n] * features[v] into row indices[v,n]"""
+    dev = require_device(weights, features, indices)
+    w, x, idx = f32(weights), f32(features), i32(indices)
+    _push_checks(w, x, idx)
+    n, k = idx.shape
+    inv_offsets, inv_slots = cached_inverse_neighbour_index(indices if indices is idx else idx)
+    out = torch.empty_like(x)
+    check(lib.hgc_push_knn(p(w), p(x), p(idx), p(inv_offsets), p(inv_slots), p(out), n, k, x.shape[1], stream()))
+    return out
+
+
+@torch.library.custom_op("hgcalml::push_knn_grad", mutates_args=())
+def push_knn_grad(grad: torch.Tensor, weights: torch.Tensor, features: torch.Tensor,
+                  indices: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """modules/compiled/push_knn_grad_module.cc:7-13: (weight_grad, feature_grad)"""
+    dev = require_device(grad, weights, features, indices)
+    g, w, x, idx = f32(grad), f32(weights), f32(features), i32(indices)
+    _push_checks(w, x, idx)
+    n, k = idx.shape
+    wgrad = torch.empty_like(w)
+    fgrad = torch.empty_like(x)
+    check(lib.hgc_push_knn_grad(p(g), p(w), p(x), p(idx), p(fgrad), p(wgrad), n, k, x.shape[1], stream()))
+    return wgrad, fgrad
+
+
 # --------------------------------------------------------------------------- condensates
 
 @torch.library.custom_op("hgcalml::binned_assign_to_condensates", mutates_args=())

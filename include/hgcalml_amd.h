@@ -251,6 +251,44 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
                                   int n_moments, int mean_and_max, hgc_stream_t stream);
 
 /* ------------------------------------------------------------------ */
+/* Ops over the same neighbour table, either side of the accumulation  */
+/* ------------------------------------------------------------------ */
+
+/* Gradient of the kNN squared distances w.r.t. the coordinates: the
+ * registered gradient of BinnedSelectKnn (modules/binned_select_knn_op.py:107-118).
+ * Replaces SelectKnnGradOpFunctor (modules/compiled/select_knn_grad_kernel.h;
+ * its CPU body is empty, the arithmetic is that of _kernel.cu.cc:81-164):
+ *   grad_coord[i,c] = - sum_n 2 g[i,n] (x[idx[i,n],c] - x[i,c])
+ *                     + sum over (v,n) with idx[v,n] == i of 2 g[v,n] (x[i,c] - x[v,c]).
+ * The second sum runs over the inverse neighbour index in ascending (v,n)
+ * order instead of the reference's atomicAdd. Indices < 0 or >= n_vert are
+ * skipped. d_dist is accepted for signature parity and not read.
+ *   d_grad_dist, d_dist [n_vert, n_neigh], d_indices [n_vert, n_neigh],
+ *   d_coord, d_grad_coord [n_vert, n_coords]. */
+int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const float *d_dist,
+                        const float *d_coord, const int *d_inv_offsets, const int *d_inv_slots,
+                        float *d_grad_coord, int n_vert, int n_neigh, int n_coords,
+                        hgc_stream_t stream);
+
+/* out[m,f] = sum over (v,n) with idx[v,n] == m of feat[v,f] * w[v,n]
+ * (idx < 0: no neighbour). Replaces PushKnnOpFunctor
+ * (modules/compiled/push_knn_kernel.h, _kernel.cc:40-62); the additions of
+ * one target happen in ascending (v,n) order, which is the CPU kernel's, so
+ * the result is bit-identical to it. */
+int hgc_push_knn(const float *d_weights, const float *d_feat, const int *d_idxs,
+                 const int *d_inv_offsets, const int *d_inv_slots, float *d_out_feat,
+                 int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
+
+/* Gradients of hgc_push_knn. Replaces PushKnnGradOpFunctor
+ * (modules/compiled/push_knn_grad_kernel.h, _kernel.cc:23-71):
+ *   feat_grad[v,f] = sum_n grad[idx[v,n],f] * w[v,n]   (slot order, bit-identical),
+ *   w_grad[v,n]    = sum_f grad[idx[v,n],f] * feat[v,f] (tree reduction over f),
+ *   0 where idx[v,n] < 0. */
+int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *d_feat,
+                      const int *d_idxs, float *d_feat_grad, float *d_w_grad,
+                      int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
+
+/* ------------------------------------------------------------------ */
 /* Condensate assignment                                               */
 /* ------------------------------------------------------------------ */
 

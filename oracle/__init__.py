@@ -9,6 +9,8 @@ reference's Python wrappers so that whole-op results can be compared:
   IndexReplacer                     modules/index_replacer_op.py:7-16
   AccumulateKnn / AccumulateLinKnn  modules/accknn_op.py:18-89
   BuildAndAssignCondensatesBinned   modules/assign_condensate_op.py:210-373
+  select_knn_grad_kernel            modules/binned_select_knn_op.py:107-118 (the op it registers)
+  PushKnn / push_knn_grad_kernel    modules/push_knn_op.py:10-36
 
 Only tests/, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
 ``bench.py`` may import this package. Nothing in ``hgcalml_amd`` does.
@@ -152,6 +154,37 @@ def accumulate_knn_grad_kernel(grad_out, weights, features, indices, maxidx, opt
     return gw, gx
 
 
+def select_knn_grad_kernel(grad_dist, indices, coords):
+    g, pg = _f(grad_dist)
+    idx, pidx = _i(indices)
+    x, px = _f(coords)
+    out = np.zeros_like(x)
+    lib().hgo_select_knn_grad(pg, pidx, px, out.ctypes.data_as(_f32p), idx.shape[0], idx.shape[1], x.shape[1])
+    return out
+
+
+def push_knn_kernel(weights, features, indices):
+    w, pw = _f(weights)
+    x, px = _f(features)
+    idx, pidx = _i(indices)
+    out = np.zeros_like(x)
+    lib().hgo_push_knn(pw, px, pidx, out.ctypes.data_as(_f32p), idx.shape[0], idx.shape[1], x.shape[1])
+    return out
+
+
+def push_knn_grad_kernel(grad, weights, features, indices):
+    """(weight_grad, feature_grad), the output order of modules/compiled/push_knn_grad_module.cc:12-13"""
+    g, pg = _f(grad)
+    w, pw = _f(weights)
+    x, px = _f(features)
+    idx, pidx = _i(indices)
+    fgrad = np.zeros_like(x)
+    wgrad = np.zeros_like(w)
+    lib().hgo_push_knn_grad(pg, pw, px, pidx, fgrad.ctypes.data_as(_f32p), wgrad.ctypes.data_as(_f32p),
+                            idx.shape[0], idx.shape[1], x.shape[1])
+    return wgrad, fgrad
+
+
 def assign_to_condensates_kernel(ccoords, dist, beta, mask, bin_splits, to_filtered, orig_h,
                                  row_splits, n_bins, bin_width, ccoords_h, dist_h, beta_h, mask_h,
                                  row_splits_h, assign_by_max_beta, opt_level_0=False):
@@ -293,6 +326,24 @@ def AccumulateLinKnn(weights, features, indices, mean_and_max=True):
 def AccumulateKnn(distances, features, indices, mean_and_max=True):
     w = np.exp(-np.asarray(distances, np.float32)).astype(np.float32)
     return accumulate_knn_kernel(w, features, indices, mean_and_max)
+
+
+def AccumulateKnnSumw(distances, features, indices, mean_and_max=False, linear=False):
+    """modules/GravNetLayersRagged.py:35-62: weighted mean normalised by the
+    accumulated weight (a column of ones rides along), divide_no_nan"""
+    F = features.shape[1]
+    x = np.concatenate([features, np.ones_like(features[:, :1])], axis=1).astype(np.float32)
+    f, midx = (AccumulateLinKnn if linear else AccumulateKnn)(distances, x, indices, mean_and_max)
+    norm = f[:, F:F + 1]
+    with np.errstate(divide="ignore", invalid="ignore"):
+        fmean = np.where(norm == 0, np.float32(0), f[:, :F] / norm).astype(np.float32)
+    if mean_and_max:
+        fmean = np.concatenate([fmean, f[:, F + 1:-1]], axis=1)
+    return fmean, midx
+
+
+def PushKnn(w, f, nidx):
+    return push_knn_kernel(w, f, nidx)
 
 
 def AccumulateKnnGrad(grad_out, distances, features, indices, maxidx, linear=False):

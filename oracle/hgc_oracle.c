@@ -14,6 +14,9 @@
  *   hgo_index_replacer            modules/compiled/index_replacer_kernel.cc:29-40
  *   hgo_accumulate_knn            modules/compiled/accumulate_knn_kernel.cc:48-81
  *   hgo_accumulate_knn_grad       modules/compiled/accumulate_knn_grad_kernel.cc:24-165
+ *   hgo_select_knn_grad           modules/compiled/select_knn_grad_kernel.cu.cc:81-164
+ *   hgo_push_knn                  modules/compiled/push_knn_kernel.cc:40-62
+ *   hgo_push_knn_grad             modules/compiled/push_knn_grad_kernel.cc:23-71
  *   hgo_box_* / hgo_assign_to_condensates
  *                                 modules/compiled/binstepper.h:100-165,
  *                                 modules/compiled/binned_assign_to_condensates_kernel.cc:23-241
@@ -30,6 +33,9 @@
  *   hgo_index_replacer       pinned: closed form.
  *   hgo_accumulate_knn       pinned: gather/multiply/mean/max composition.
  *   hgo_accumulate_knn_grad  pinned: autograd of that composition.
+ *   hgo_select_knn_grad      pinned: float64 autograd of sum((x_i - x_k)^2).
+ *   hgo_push_knn             pinned: ordered unbuffered scatter-add (bitwise).
+ *   hgo_push_knn_grad        pinned: float64 autograd of that scatter-add.
  *   hgo_assign_to_condensates pinned for an all-zero no_condensation_mask by a
  *                            bin-free sequential greedy; behaviour with a
  *                            non-zero mask is "parity unpinned".
@@ -646,4 +652,112 @@ int hgo_assign_to_condensates(int C, int B,
         n_condensates[r + 1] = running;
     }
     return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* select_knn_grad: gradient of the kNN squared distances              */
+/* ------------------------------------------------------------------ */
+
+/* modules/compiled/select_knn_grad_kernel.cu.cc:81-164 (the reference's CPU
+ * functor has an empty body, select_knn_grad_kernel.cc:23-41, so its device
+ * kernels define the op). First every vertex collects -2 g (x_k - x_i) over
+ * its own neighbours (accumulated in a float, each step evaluated in double as
+ * the literal `2.` makes it), then every (vertex, slot) adds 2 g (x_m - x_i)
+ * rounded to float into its neighbour m. The reference does the latter with
+ * atomicAdd in no particular order; the order here is ascending (vertex,
+ * slot), one of its possible outcomes. */
+void hgo_select_knn_grad(const float *grad_dist, const int *indices,
+                         const float *coords, float *grad_coords,
+                         int n_vert, int K, int C)
+{
+    for (int i = 0; i < n_vert; ++i) {
+        for (int c = 0; c < C; ++c) {
+            const float xi = coords[(size_t)i * C + c];
+            float self = 0.f;
+            for (int n = 0; n < K; ++n) {
+                int k = indices[(size_t)i * K + n];
+                if (k < 0 || k >= n_vert)
+                    continue;
+                const float g = grad_dist[(size_t)i * K + n];
+                const float xk = coords[(size_t)k * C + c];
+                self -= 2. * g * (xk - xi);
+            }
+            grad_coords[(size_t)i * C + c] = self;
+        }
+    }
+    for (int i = 0; i < n_vert; ++i) {
+        for (int n = 0; n < K; ++n) {
+            int m = indices[(size_t)i * K + n];
+            if (m < 0 || m >= n_vert)
+                continue;
+            const float g = grad_dist[(size_t)i * K + n];
+            for (int c = 0; c < C; ++c) {
+                const float xi = coords[(size_t)i * C + c];
+                const float xm = coords[(size_t)m * C + c];
+                float add = 2. * g * (xm - xi);
+                grad_coords[(size_t)m * C + c] += add;
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* push_knn forward and gradient                                       */
+/* ------------------------------------------------------------------ */
+
+/* modules/compiled/push_knn_kernel.cc:40-62 */
+void hgo_push_knn(const float *weights, const float *features,
+                  const int *indices, float *out,
+                  int n_vert, int K, int F)
+{
+    memset(out, 0, sizeof(float) * (size_t)n_vert * F);
+    for (int v = 0; v < n_vert; ++v) {
+        for (int f = 0; f < F; ++f) {
+            const float x = features[(size_t)v * F + f];
+            for (int n = 0; n < K; ++n) {
+                int m = indices[(size_t)v * K + n];
+                if (m < 0)
+                    continue;
+                const float w = weights[(size_t)v * K + n];
+                float term = x * w;
+                out[(size_t)m * F + f] += term;
+            }
+        }
+    }
+}
+
+/* modules/compiled/push_knn_grad_kernel.cc:23-71 */
+void hgo_push_knn_grad(const float *grad, const float *weights,
+                       const float *features, const int *indices,
+                       float *feat_grad, float *w_grad,
+                       int n_vert, int K, int F)
+{
+    for (int v = 0; v < n_vert; ++v) {
+        for (int f = 0; f < F; ++f) {
+            float acc = 0.f;
+            for (int n = 0; n < K; ++n) {
+                int m = indices[(size_t)v * K + n];
+                if (m < 0)
+                    continue;
+                float term = grad[(size_t)m * F + f] * weights[(size_t)v * K + n];
+                acc += term;
+            }
+            feat_grad[(size_t)v * F + f] = acc;
+        }
+    }
+    for (int v = 0; v < n_vert; ++v) {
+        for (int n = 0; n < K; ++n) {
+            int m = indices[(size_t)v * K + n];
+            if (m < 0) {
+                w_grad[(size_t)v * K + n] = 0.f;
+                continue;
+            }
+            float acc = 0.f;
+            for (int f = 0; f < F; ++f) {
+                float term = grad[(size_t)m * F + f] * features[(size_t)v * F + f];
+                acc += term;
+            }
+            w_grad[(size_t)v * K + n] = acc;
+        }
+    }
 }

@@ -445,6 +445,85 @@ def test_accumulate_cfg4_full_size_properties(oracle):
     assert torch.allclose(total, mean_total + max_total, rtol=1e-6, atol=1e-3)
 
 
+# ------------------------------------------------------------------ ops next to the accumulation
+
+@pytest.mark.parametrize("K,C", [(16, 3), (64, 4), (5, 8)])
+def test_select_knn_grad(oracle, K, C):
+    rng = np.random.default_rng(50 + K)
+    n = 3000
+    x = rng.standard_normal((n, C)).astype(np.float32)
+    idx = np.stack([np.concatenate([[v], rng.choice(np.delete(np.arange(n), v), K - 1, replace=False)])
+                    for v in range(n)]).astype(np.int32)
+    idx[100:200, K // 2:] = -1
+    idx[300, :] = -1
+    g = rng.standard_normal((n, K)).astype(np.float32)
+    ref = oracle.select_knn_grad_kernel(g, idx, x)
+    got = torch.ops.hgcalml.select_knn_grad(t(g), t(idx), t(np.zeros_like(g)), t(x))
+    # same terms in the same order as the oracle: identical bits
+    assert (bits(got.cpu().numpy()) == bits(ref)).all()
+
+
+def test_knn_distance_gradient_through_wrapper(oracle):
+    """BinnedSelectKnn's distances are differentiable w.r.t. the coordinates
+    (registered gradient SelectKnnGrad); compared with float64 autograd of the
+    re-computed distances"""
+    from hgcalml_amd import BinnedSelectKnn
+    cfg = workloads.cfg2(scale=0.02)
+    coords = cfg["coords"]
+    rs = np.array([0, 1000, len(coords)], np.int32)
+    K = 12
+    tc = t(coords).requires_grad_(True)
+    idx, dist = BinnedSelectKnn(K, tc, t(rs), n_bins=8)
+    g = np.random.default_rng(3).standard_normal(dist.shape).astype(np.float32)
+    (dist * t(g)).sum().backward()
+    x64 = torch.tensor(coords, dtype=torch.float64, requires_grad=True)
+    i64 = idx.cpu().to(torch.int64)
+    d2 = ((x64[:, None, :] - x64[i64.clamp(min=0)]) ** 2).sum(2)
+    d2 = torch.where(i64 >= 0, d2, torch.zeros_like(d2))
+    (d2 * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    want = x64.grad.numpy()
+    assert np.abs(tc.grad.cpu().numpy() - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.allclose(dist.detach().cpu().numpy(), d2.detach().numpy(), rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("K,F", [(8, 5), (16, 32), (64, 64), (12, 128), (20, 192)])
+def test_push_knn_and_gradient(oracle, K, F):
+    from hgcalml_amd import PushKnn
+    rng = np.random.default_rng(60 + K + F)
+    n = 700
+    d, x, idx = make_acc_case(rng, n, K, F)
+    w = np.exp(-d).astype(np.float32)
+    ref = oracle.PushKnn(w, x, idx)
+    tw, tx = t(w).requires_grad_(True), t(x).requires_grad_(True)
+    out = PushKnn(tw, tx, t(idx))
+    assert (bits(out.detach().cpu().numpy()) == bits(ref)).all()
+    g = rng.standard_normal((n, F)).astype(np.float32)
+    out.backward(t(g))
+    rwg, rfg = oracle.push_knn_grad_kernel(g, w, x, idx)
+    assert (bits(tx.grad.cpu().numpy()) == bits(rfg)).all()
+    # weight gradient: tree reduction over the features, 1e-5 relative to the sum of |terms|
+    scale = (np.abs(g[np.maximum(idx, 0)]) * np.abs(x)[:, None, :]).sum(-1)
+    assert (np.abs(tw.grad.cpu().numpy() - rwg) <= 1e-5 * scale + 1e-30).all()
+    assert (tw.grad.cpu().numpy()[idx < 0] == 0).all()
+
+
+@pytest.mark.parametrize("linear", [True, False])
+def test_accumulate_sumw_wrappers(oracle, linear):
+    from hgcalml_amd import AccumulateKnnSumw, AccumulateLinKnnSumw
+    rng = np.random.default_rng(70)
+    d, x, idx = make_acc_case(rng, 500, 16, 32)
+    w = d + np.float32(0.1)
+    for mm in (False, True):
+        ref, rarg = oracle.AccumulateKnnSumw(w, x, idx, mean_and_max=mm, linear=linear)
+        fn = AccumulateLinKnnSumw if linear else AccumulateKnnSumw
+        out, arg = fn(t(w), t(x), t(idx), mean_and_max=mm)
+        assert out.shape == ref.shape
+        if linear:
+            assert (bits(out.cpu().numpy()) == bits(ref)).all()
+        else:
+            assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-6)
+
+
 # ------------------------------------------------------------------ condensates
 
 def run_condensates(oracle, cfg, by_max_beta, mask=None):

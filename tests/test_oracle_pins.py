@@ -355,6 +355,98 @@ def bin_free_greedy(oracle, cfg, by_max_beta):
     return assignment, asso, np.array(alphas, np.int32), np.array(ncond, np.int32)
 
 
+# ------------------------------------------------------------------ ops next to the accumulation
+
+def neighbour_case(rng, n, K, with_holes=True):
+    idx = np.stack([np.concatenate([[v], rng.permutation(np.delete(np.arange(n), v))[:K - 1]])
+                    for v in range(n)]).astype(np.int32)
+    if with_holes:
+        idx[3:9, K // 2:] = -1
+        idx[11, :] = -1
+    return idx
+
+
+def test_select_knn_grad_vs_autograd(oracle):
+    """d(sum g_ik |x_i - x_k|^2)/dx by float64 autograd; a wrong sign, a dropped
+    self or neighbour term, or a swapped index each change the result by O(1)"""
+    import torch
+    rng = np.random.default_rng(31)
+    n, K, C = 200, 7, 4
+    x = rng.standard_normal((n, C)).astype(np.float32)
+    idx = neighbour_case(rng, n, K)
+    g = rng.standard_normal((n, K)).astype(np.float32)
+    got = oracle.select_knn_grad_kernel(g, idx, x)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tidx = torch.tensor(idx, dtype=torch.int64)
+    d2 = ((tx[:, None, :] - tx[tidx.clamp(min=0)]) ** 2).sum(2)
+    d2 = torch.where(tidx >= 0, d2, torch.zeros_like(d2))
+    (d2 * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    scale = np.abs(tx.grad.numpy()).max()
+    assert np.abs(got - tx.grad.numpy()).max() <= 1e-5 * scale
+    # a vertex nobody names and without neighbours gets exactly zero
+    lonely = np.setdiff1d(np.arange(n), idx[idx >= 0])
+    for v in lonely:
+        if (idx[v] < 0).all():
+            assert (got[v] == 0).all()
+    # out-of-range indices are skipped like -1
+    idx2 = idx.copy()
+    idx2[20, 2] = n + 5
+    idx3 = idx.copy()
+    idx3[20, 2] = -1
+    assert (oracle.select_knn_grad_kernel(g, idx2, x) == oracle.select_knn_grad_kernel(g, idx3, x)).all()
+
+
+def test_push_knn_vs_ordered_scatter_and_autograd(oracle):
+    import torch
+    rng = np.random.default_rng(32)
+    n, K, F = 150, 6, 5
+    idx = neighbour_case(rng, n, K)
+    w = (rng.random((n, K)) + 0.1).astype(np.float32)
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    out = oracle.PushKnn(w, x, idx)
+    # unbuffered scatter-add in ascending (vertex, slot) order: same bits
+    ref = np.zeros((n, F), np.float32)
+    valid = idx >= 0
+    terms = (x[:, None, :] * w[:, :, None]).astype(np.float32)
+    np.add.at(ref, idx[valid], terms[valid])
+    assert (ref.view(np.int32) == out.view(np.int32)).all()
+    # the reference's own slow composition (modules/push_knn_op.py:38-66) in float64
+    tw = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tidx = torch.tensor(idx, dtype=torch.int64)
+    contrib = tx[:, None, :] * tw[:, :, None]
+    contrib = torch.where((tidx >= 0)[:, :, None], contrib, torch.zeros_like(contrib))
+    tout = torch.zeros((n, F), dtype=torch.float64).index_add(0, tidx.clamp(min=0).reshape(-1), contrib.reshape(-1, F))
+    assert np.allclose(out, tout.detach().numpy(), rtol=1e-5, atol=1e-6)
+    g = rng.standard_normal((n, F)).astype(np.float32)
+    (tout * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    wgrad, fgrad = oracle.push_knn_grad_kernel(g, w, x, idx)
+    assert np.allclose(wgrad, tw.grad.numpy(), rtol=1e-5, atol=1e-5)
+    assert np.allclose(fgrad, tx.grad.numpy(), rtol=1e-5, atol=1e-5)
+    assert (wgrad[idx < 0] == 0).all()
+
+
+def test_accumulate_sumw_composition(oracle):
+    """weighted mean over the accumulated weight: equals sum(w x)/sum(w) per vertex"""
+    rng = np.random.default_rng(33)
+    n, K, F = 80, 5, 3
+    idx = neighbour_case(rng, n, K)
+    w = (rng.random((n, K)) + 0.1).astype(np.float32)
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    for mm in (False, True):
+        out, _ = oracle.AccumulateKnnSumw(w, x, idx, mean_and_max=mm, linear=True)
+        valid = (idx >= 0)[:, :, None]
+        wx = np.where(valid, x[np.maximum(idx, 0)].astype(np.float64) * w[:, :, None], 0.)
+        sw = np.where(idx >= 0, w, 0.).astype(np.float64).sum(1, keepdims=True)
+        want = np.divide(wx.sum(1), sw, out=np.zeros((n, F)), where=sw != 0)
+        assert out.shape == (n, 2 * F if mm else F)
+        assert np.allclose(out[:, :F], want, rtol=1e-5, atol=1e-6)
+        assert (out[11] == 0).all()   # no neighbours at all: divide_no_nan
+        if mm:
+            full, _ = oracle.AccumulateLinKnn(w, x, idx)
+            assert (out[:, F:] == full[:, F:]).all()
+
+
 @pytest.mark.parametrize("by_max_beta", [True, False])
 @pytest.mark.parametrize("t_d", [0.5, 0.15])
 def test_condensates_vs_bin_free_greedy(oracle, by_max_beta, t_d):
