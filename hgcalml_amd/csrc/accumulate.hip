@@ -134,8 +134,9 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
 // indices and weights of its row come in through scalar loads, and gathered
 // rows are fetched with buffer loads whose address is
 //   descriptor base + scalar row offset + per-lane column offset,
-// i.e. no vector ALU is spent on addressing and the hardware range-checks every
-// access against the size of the matrix. Chunks of U neighbour slots without
+// i.e. no vector ALU is spent on addressing. The scalar row offset is not part
+// of the hardware's range check, so every row index is validated on the scalar
+// side before it is used. Chunks of U neighbour slots without
 // padding take a branch-free path with all U row loads in flight.
 
 
@@ -190,13 +191,14 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
             int j[U];
             float wn[U];
             float x[U][VEC];
-            bool all_valid = true;
+            uint32_t j_max = 0;  // unsigned: a negative index is the largest
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 j[u] = irow[n0 + u];
                 wn[u] = wrow[n0 + u];
-                all_valid = all_valid && (unsigned)j[u] < (unsigned)n_vert;
+                j_max = max(j_max, (uint32_t)j[u]);
             }
+            const bool all_valid = j_max < (uint32_t)n_vert;
             if (MAX) {
                 int fs = -1;
 #pragma unroll
@@ -449,11 +451,12 @@ __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__re
                     const int l = l0 + u0 + u;
                     j[u] = l < K ? irow[l] : -1;
                 }
-                // rows outside [0, n_vert) read as arbitrary in-range data or zeros
-                // (hardware range check) and can never equal an arg-max index of a
-                // valid row; their result is overwritten with 0 below
+                // slots without a neighbour read row 0; an index outside [0, n_vert)
+                // can never equal an arg-max index of a valid row, and the slot's
+                // result is overwritten with 0 below
 #pragma unroll
-                for (int u = 0; u < U; ++u) X.load<VEC>(j[u], lane_bytes, x[u]);
+                for (int u = 0; u < U; ++u)
+                    X.load<VEC>((uint32_t)j[u] < (uint32_t)n_vert ? j[u] : 0, lane_bytes, x[u]);
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
 #pragma unroll

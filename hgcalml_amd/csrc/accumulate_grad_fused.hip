@@ -37,11 +37,34 @@ constexpr int kGroup = 16;  // entries per cross-lane reduction
 template <int VEC, bool SLOTS>
 struct ArgInfo {
     uint32_t v[SLOTS ? 1 : VEC];
-    __device__ __forceinline__ bool hit(int e, int key) const {
-        if constexpr (SLOTS) return ((v[0] >> (8 * e)) & 255u) == (uint32_t)key;
-        else return (int)v[e] == key;
-    }
 };
+
+// Does byte E of `packed` equal the wave-uniform `key`? One SDWA compare that
+// leaves the lane mask in scalar registers, where the selects below consume it.
+template <int E>
+__device__ __forceinline__ bool slot_byte_is(uint32_t packed, uint32_t key) {
+    uint64_t mask;
+    if constexpr (E == 0) asm("v_cmp_eq_u32_sdwa %0, %1, %2 src0_sel:BYTE_0 src1_sel:DWORD" : "=s"(mask) : "v"(packed), "s"(key));
+    else if constexpr (E == 1) asm("v_cmp_eq_u32_sdwa %0, %1, %2 src0_sel:BYTE_1 src1_sel:DWORD" : "=s"(mask) : "v"(packed), "s"(key));
+    else if constexpr (E == 2) asm("v_cmp_eq_u32_sdwa %0, %1, %2 src0_sel:BYTE_2 src1_sel:DWORD" : "=s"(mask) : "v"(packed), "s"(key));
+    else asm("v_cmp_eq_u32_sdwa %0, %1, %2 src0_sel:BYTE_3 src1_sel:DWORD" : "=s"(mask) : "v"(packed), "s"(key));
+    return __builtin_amdgcn_inverse_ballot_w64(mask);
+}
+
+template <int VEC, bool SLOTS>
+__device__ __forceinline__ void arg_hits(const ArgInfo<VEC, SLOTS> &ai, uint32_t key, bool (&hit)[VEC]) {
+    if constexpr (SLOTS) {
+        hit[0] = slot_byte_is<0>(ai.v[0], key);
+        if constexpr (VEC >= 2) hit[1] = slot_byte_is<1>(ai.v[0], key);
+        if constexpr (VEC >= 4) {
+            hit[2] = slot_byte_is<2>(ai.v[0], key);
+            hit[3] = slot_byte_is<3>(ai.v[0], key);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) hit[e] = ai.v[e] == key;
+    }
+}
 
 template <int VEC>
 __device__ __forceinline__ uint32_t load_slot_bytes(__amdgpu_buffer_rsrc_t rsrc, uint32_t row_byte_offset,
@@ -72,38 +95,54 @@ __device__ __forceinline__ float transpose_reduce_16(float (&val)[kGroup]) {
     return r;
 }
 
+// With arg-max slots a row's byte offset (a multiple of 512) and the entry's
+// slot share one word, so that one cross-lane read brings both.
+constexpr uint32_t kKeyMask = 511u;
+// a per-lane buffer offset no matrix reaches: the hardware range check turns
+// the load into "return 0" without a memory access
+constexpr uint32_t kOutOfRange = 0xfffffff0u;
+
 // Entries [c, c+16) of the current 64-entry batch. FAST: all 16 exist and none
 // is a repeated self reference.
+//
+// Feature gradient addend of one entry, per feature: ((g/K)*w) + (hit ? g_max*w : 0),
+// added in list order -- the reference's terms in its order. Two rewrites keep
+// the bits and save vector instructions: for a power-of-two K the exact
+// scaling 1/K moves onto the weight (wk = w/K, identical unless g/K is
+// subnormal), and the max part is formed as (hit ? g_max : 0) * w, whose zero
+// may carry the weight's sign, which cannot change a sum that started at +0
+// (it would differ for an infinite weight only).
 template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool FAST>
 __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix &MI, __amdgpu_buffer_rsrc_t MS,
                                            const uint32_t (&lane_bytes)[NB], uint32_t max_col_bytes, int c, int cnt,
-                                           uint64_t repmask, int self_key, int m, uint32_t off_v, float w_v, int key_v,
-                                           const float (&xo)[NB][VEC], const float (&xk)[NB][VEC], float (&acc)[NB][VEC], float kf,
-                                           float inv_kf,
-                                           float (&val)[kGroup]) {
+                                           uint64_t repmask, int self_key, int m, uint32_t offkey_v, float w_v,
+                                           float wk_v, const float (&xo)[NB][VEC], const float (&xk)[NB][VEC],
+                                           float (&acc)[NB][VEC], float kf, float (&val)[kGroup]) {
 #pragma unroll
     for (int h = 0; h < kGroup; h += kRows) {
-        uint32_t soff[kRows];
-        float sw[kRows];
-        int skey[kRows];
+        uint32_t soff[kRows], skey[kRows];
+        float sw[kRows], swk[kRows];
         bool rep[kRows], live[kRows];
 #pragma unroll
         for (int u = 0; u < kRows; ++u) {
             const int li = c + h + u;  // lanes past the end of the list hold a copy of its last entry
-            soff[u] = (uint32_t)__builtin_amdgcn_readlane((int)off_v, li);
+            const uint32_t ok = (uint32_t)__builtin_amdgcn_readlane((int)offkey_v, li);
+            soff[u] = (MAX && SLOTS) ? (ok & ~kKeyMask) : ok;
+            skey[u] = (MAX && SLOTS) ? (ok & kKeyMask) : (uint32_t)m;
             sw[u] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(w_v), li));
-            skey[u] = (MAX && SLOTS) ? __builtin_amdgcn_readlane(key_v, li) : m;
+            swk[u] = POW2K ? __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(wk_v), li)) : 0.f;
             rep[u] = false;
             live[u] = true;
             if (!FAST) {
                 live[u] = li < cnt;
                 rep[u] = ((repmask >> li) & 1ull) != 0;
-                if (MAX && SLOTS && rep[u]) skey[u] = self_key;
+                if (MAX && SLOTS && rep[u]) skey[u] = (uint32_t)self_key;
             }
         }
         // arg-max tables first (they gate the loads of the max half), then the mean half
         ArgInfo<VEC, SLOTS> ai[kRows][NB];
         float gm[kRows][NB][VEC], gx[kRows][NB][VEC];
+        bool hit[kRows][NB][VEC];
         if (MAX) {
 #pragma unroll
             for (int u = 0; u < kRows; ++u)
@@ -119,18 +158,17 @@ __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix 
             for (int b = 0; b < NB; ++b) Gm.load_at<VEC>(soff[u], lane_bytes[b], gm[u][b]);
         if (MAX) {
             // the max half of a gradient row is fetched only by the lanes whose
-            // feature has its maximum at this entry (about F/K lanes per row)
+            // feature has its maximum at this entry (about F/K lanes per row); the
+            // other lanes aim out of range and receive 0
 #pragma unroll
             for (int u = 0; u < kRows; ++u)
 #pragma unroll
                 for (int b = 0; b < NB; ++b) {
+                    arg_hits<VEC, SLOTS>(ai[u][b], skey[u], hit[u][b]);
                     bool any = false;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) {
-                        any = any || ai[u][b].hit(e, skey[u]);
-                        gx[u][b][e] = 0.f;
-                    }
-                    if (any) Gm.load_at<VEC>(soff[u], lane_bytes[b] + max_col_bytes, gx[u][b]);
+                    for (int e = 0; e < VEC; ++e) any = any || hit[u][b][e];
+                    Gm.load_at<VEC>(soff[u], any ? lane_bytes[b] + max_col_bytes : kOutOfRange, gx[u][b]);
                 }
         }
 #pragma unroll
@@ -140,23 +178,20 @@ __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix 
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    // feature gradient: the reference's addend ((g/K)*w) + max part, in list order
-                    float part = POW2K ? gm[u][b][e] * inv_kf : gm[u][b][e] / kf;
-                    part = part * sw[u];
-                    float part_max = 0.f;
-                    bool hit = false;
-                    if (MAX) {
-                        hit = ai[u][b].hit(e, skey[u]);
-                        const float pmx = gx[u][b][e] * sw[u];
-                        part_max = (hit && !rep[u]) ? pmx : 0.f;  // repeated self references carry the max part once
-                    }
-                    const float add = part + part_max;
-                    acc[b][e] = acc[b][e] + add;
+                    const float g = gm[u][b][e];
+                    const float part = POW2K ? g * swk[u] : (g / kf) * sw[u];
                     // weight gradient of slot (v, n): partial dot products with the wave's own row
-                    val[h + u] = __builtin_fmaf(gm[u][b][e], xk[b][e], val[h + u]);
+                    val[h + u] = __builtin_fmaf(g, xk[b][e], val[h + u]);
                     if (MAX) {
-                        const float t = __builtin_fmaf(gx[u][b][e], xo[b][e], val[h + u]);
-                        val[h + u] = hit ? t : val[h + u];
+                        // a lane with one hit among its VEC features has loaded all of them
+                        const float gsel = (VEC == 1 || hit[u][b][e]) ? gx[u][b][e] : 0.f;
+                        val[h + u] = __builtin_fmaf(gsel, xo[b][e], val[h + u]);
+                        // repeated self references carry the max part once, at the first self slot
+                        const float part_max = (!FAST && rep[u]) ? 0.f : gsel * sw[u];
+                        const float add = part + part_max;
+                        acc[b][e] = acc[b][e] + add;
+                    } else {
+                        acc[b][e] = acc[b][e] + part;  // the reference's "+ 0" cannot change the sum
                     }
                 }
         }
@@ -214,7 +249,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
         const float w_v = w[slot_v];
         const int v = fast_div(slot_v, div_k);
         const int key_v = slot_v - v * K;
-        const uint32_t off_v = (uint32_t)v * g_row_bytes;
+        // row offset of the entry's vertex, with the entry's slot in its low bits
+        const uint32_t offkey_v = (uint32_t)v * g_row_bytes | ((MAX && SLOTS) ? (uint32_t)key_v : 0u);
+        const float wk_v = w_v * inv_kf;
         const uint64_t repmask = __ballot(v == m && key_v != self_key && lane < cnt);
         for (int c = 0; c < cnt; c += kGroup) {
             float val[kGroup];
@@ -223,10 +260,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
             const bool fast = (c + kGroup <= cnt) && ((repmask >> c) & ((1ull << kGroup) - 1)) == 0;
             if (fast)
                 grad_group<VEC, NB, MAX, POW2K, SLOTS, true>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
-                                                             self_key, m, off_v, w_v, key_v, xo, xk, acc, kf, inv_kf, val);
+                                                             self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
             else
                 grad_group<VEC, NB, MAX, POW2K, SLOTS, false>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
-                                                              self_key, m, off_v, w_v, key_v, xo, xk, acc, kf, inv_kf, val);
+                                                              self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
             const float r = transpose_reduce_16(val);  // lane L: entry c + (L & 15)
             const int dst = __shfl(slot_v, c + (lane & (kGroup - 1)), kWave);
             if (lane < kGroup && c + lane < cnt) {
@@ -235,7 +272,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
         }
     }
 #pragma unroll
-    for (int b = 0; b < NB; ++b) store_vec<VEC>(gfeat + (size_t)m * F + (b * kWave + lane) * VEC, acc[b]);
+    for (int b = 0; b < NB; ++b) store_vec<VEC>(gfeat + (size_t)m * F + (lane_bytes[b] >> 2), acc[b]);
 }
 
 // weight gradient of padded slots (index < 0 or out of range): they sort to the
@@ -277,12 +314,13 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
     if (F % kWave != 0) return 1;
     const uintptr_t align_or = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(feat) |
                                reinterpret_cast<uintptr_t>(maxidx) | reinterpret_cast<uintptr_t>(gfeat);
-    const int vec = wave_vec(F, align_or);
-    const int nb = F / (kWave * vec);
-    if (nb < 1 || nb > 3) return 1;
     // rows are addressed through 32-bit buffer offsets
     if ((unsigned long long)n_vert * (unsigned long long)g_cols * 4ull >= (1ull << 32)) return 1;
     if (maxslot && K > 254) maxslot = nullptr;
+    const int vec = wave_vec(F, align_or);
+    const int nb = F / (kWave * vec);
+    // wider rows would not fit the register budget that keeps 5+ waves per SIMD resident
+    if (nb < 1 || vec * nb > 4) return 1;
 
     const long long total = (long long)n_vert * K;
     zero_padded_weight_grad_kernel<<<256, 256, 0, s>>>(inv_off, inv_slots, gw, n_vert, total);
@@ -296,10 +334,7 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
         case 13: return launch_fused<1, 3>(HGC_ARGS);
         case 21: return launch_fused<2, 1>(HGC_ARGS);
         case 22: return launch_fused<2, 2>(HGC_ARGS);
-        case 23: return launch_fused<2, 3>(HGC_ARGS);
         case 41: return launch_fused<4, 1>(HGC_ARGS);
-        case 42: return launch_fused<4, 2>(HGC_ARGS);
-        case 43: return launch_fused<4, 3>(HGC_ARGS);
     }
 #undef HGC_ARGS
     return 1;
