@@ -828,7 +828,7 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
     if (n_feat >= kWave && fits_32bit) {  // one wave per vertex, rows addressed through 32-bit buffer offsets
         const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
         // both gradients from one gather pass where that kernel covers the shape
-        if (want_w && want_f && divisor == (float)n_neigh && (!mean_and_max || use_slots)) {
+        if (want_w && want_f && divisor == (float)n_neigh) {
             const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
                                                         d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
                                                         d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat,
