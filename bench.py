@@ -40,7 +40,7 @@ HBM_PEAK_GBS = 8000.0
 # both scaled by what the counters read for the 512 MB calibration copy below);
 # summary in profiles/accumulate_knn_cfg4_hbm_counters.txt. Counters cannot be
 # read from inside the timed run, so this is the last profiled value.
-CFG4_MEASURED_HBM_BYTES = 18.9e9
+CFG4_MEASURED_HBM_BYTES = 22.6e9
 
 
 def log(*a):
@@ -65,8 +65,8 @@ def event_ms(fn, steps, warmup):
     return float(np.mean(times)), float(np.median(times)), float(np.min(times))
 
 
-def cpu_baseline_knn(cfg):
-    """the oracle's binned kNN kernel over all queries of cfg2, one thread"""
+def cpu_baseline_knn(cfg, reps=5):
+    """the oracle's binned kNN kernel over all queries of cfg2, `reps` passes, one thread"""
     import oracle
     coords, rs, K = cfg["coords"], cfg["row_splits"], cfg["K"]
     dbin, flat, nb, bw, nper = oracle.BinByCoordinates(coords[:, :3], rs, n_bins=cfg["n_bins"])
@@ -74,9 +74,10 @@ def cpu_baseline_knn(cfg):
     bb = np.concatenate([[0], np.cumsum(nper)]).astype(np.int32)
     sc, sf, sd = coords[order], flat[order], dbin[order]
     t0 = time.perf_counter()
-    oracle.binned_select_knn_kernel(K, sc, sf, sd, bb, nb, bw)
+    for _ in range(reps):
+        oracle.binned_select_knn_kernel(K, sc, sf, sd, bb, nb, bw)
     dt = time.perf_counter() - t0
-    return len(coords) / dt, dt
+    return reps * len(coords) / dt, dt
 
 
 def cpu_baseline_accumulate(cfg4_small):
@@ -194,12 +195,12 @@ def main():
     if not args.skip_cpu_baseline:
         log("bench: CPU baseline (oracle, 1 thread): binned kNN kernel over cfg2 ...")
         qps, secs = cpu_baseline_knn(c2)
-        small = workloads.cfg4(scale=0.02)
+        small = workloads.cfg4(scale=0.1)
         f_s, b_s = cpu_baseline_accumulate(small)
         ns = len(small["indices"])
         cpu = {"value": round(qps, 1), "unit": "queries/s", "cores": 1, "kind": "port",
-               "sample": "all %d queries of cfg2 through the oracle's binned_select_knn kernel (gcc -O2, one run, "
-                         "%.1f s); binning/sort glue not included" % (n2, secs),
+               "sample": "5 passes over all %d queries of cfg2 through the oracle's binned_select_knn kernel "
+                         "(gcc -O2, %.1f s); binning/sort glue not included" % (n2, secs),
                "accumulate_fwd_grad_GBps": round((4.0 * ns * (2 * K4 + 4 * F4) + 4.0 * ns * (3 * K4 + 5 * F4)) /
                                                  (f_s + b_s) / 1e9, 4),
                "accumulate_sample": "cfg4 at N=%d (fwd %.2f s, grad %.2f s)" % (ns, f_s, b_s),
