@@ -853,8 +853,7 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
         // indices) and the neighbour window overflows one XCD's L2: slice. With it
         // the row shrinks to 640 B plus a few lanes of the max half and the wider
         // unsliced loads win.
-        int n_slices = (n_feat >= 2 * kWave && !(mean_and_max && use_slots)) ? 2 : 1;
-        if (const char *env = getenv("HGC_FGRAD_SLICES")) n_slices = atoi(env) == 2 && n_feat >= 2 * kWave ? 2 : 1;  // tuning aid
+        const int n_slices = (n_feat >= 2 * kWave && mean_and_max && !use_slots) ? 2 : 1;
         const int fg_vec = n_slices == 1 ? vec : wave_vec(n_feat / 2, align_or);
         const int tiles = ceil_div(n_vert, 4);
         const dim3 fg_grid(n_slices == 1 ? tiles : kNumXcd * ceil_div(tiles, kNumXcd / n_slices));
