@@ -187,6 +187,19 @@ def main():
         for mode in (True, False):
             m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode), 5, 2)
             extra["cfg5_condensates_ms_max_beta" if mode else "cfg5_condensates_ms_min_dist"] = round(m5[0], 3)
+        # one GravNet block (learned 4-D coordinates -> kNN K=64+self -> accumulate F=64 -> dense), forward + backward
+        from hgcalml_amd import RaggedGravNet
+        torch.manual_seed(0)
+        layer = RaggedGravNet(64, 64, 4, 128, 64, n_knn_bins=30).to(dev)
+        xg = torch.from_numpy(c2["features"]).to(dev).requires_grad_(True)
+        rs2 = torch.from_numpy(c2["row_splits"]).to(dev)
+
+        def gravnet_step():
+            out, _, _, dist = layer(xg, rs2)
+            (out.sum() + dist.sum()).backward()
+            xg.grad = None
+        mg = event_ms(gravnet_step, 5, 2)
+        extra["gravnet_block_fwd_bwd_ms_N150k_K64_F64"] = round(mg[0], 3)
     except Exception as e:  # information only; never hide the headline numbers
         extra["info_error"] = repr(e)
 

@@ -3,11 +3,11 @@
 Public API (same names and signatures as the reference's Python wrappers):
 BinByCoordinates, BinnedSelectKnn, IndexReplacer, AccumulateKnn,
 AccumulateLinKnn, AccumulateKnnSumw, AccumulateLinKnnSumw, PushKnn,
-BuildAndAssignCondensatesBinned. All of them need tensors on
+BuildAndAssignCondensatesBinned, and the RaggedGravNet layer on top of them. All of them need tensors on
 a HIP device and the in-tree libhgcalml_amd.so; there is no CPU path.
 """
 __all__ = ["BinByCoordinates", "BinnedSelectKnn", "IndexReplacer", "AccumulateKnn", "AccumulateLinKnn",
-           "AccumulateKnnSumw", "AccumulateLinKnnSumw", "PushKnn", "BuildAndAssignCondensatesBinned"]
+           "AccumulateKnnSumw", "AccumulateLinKnnSumw", "PushKnn", "BuildAndAssignCondensatesBinned", "RaggedGravNet"]
 
 
 def __getattr__(name):
@@ -24,6 +24,7 @@ def __getattr__(name):
             "AccumulateKnnSumw": "accknn_op",
             "AccumulateLinKnnSumw": "accknn_op",
             "PushKnn": "push_knn_op",
+            "RaggedGravNet": "GravNetLayersRagged",
             "BuildAndAssignCondensatesBinned": "assign_condensate_op",
         }[name]
         return getattr(importlib.import_module("." + mod, __name__), name)

@@ -524,6 +524,59 @@ def test_accumulate_sumw_wrappers(oracle, linear):
             assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("n_propagate,n_neighbours,sumwnorm", [(64, 16, False), (8, 15, False), (64, 16, True)])
+def test_gravnet_block_forward_and_all_gradients(n_propagate, n_neighbours, sumwnorm):
+    """one GravNet block end to end: outputs and the gradients w.r.t. the input and
+    every weight (through the accumulation, through the distances into the learned
+    coordinates, through the dense layers) against a float64 torch composition over
+    the same neighbour table"""
+    from hgcalml_amd import RaggedGravNet
+    torch.manual_seed(5)
+    n, f_in, n_dims, n_filters = 3000, 16, 3, 24
+    rs = np.array([0, 1300, n], np.int32)
+    layer = RaggedGravNet(f_in, n_neighbours, n_dims, n_filters, n_propagate, sumwnorm=sumwnorm,
+                          coord_initialiser_noise=0.3, n_knn_bins=6).to(DEV)
+    x = torch.randn(n, f_in, device=DEV, requires_grad=True)
+    out, coords, idx, dist = layer(x, t(rs))
+    assert out.shape == (n, n_filters) and coords.shape == (n, n_dims)
+    assert idx.shape == (n, n_neighbours + 1) and dist.shape == idx.shape
+    assert (idx[:, 0].cpu().numpy() == np.arange(n)).all()
+    g_out = torch.randn_like(out)
+    g_dist = torch.randn_like(dist) * 0.1
+    ((out * g_out).sum() + (dist * g_dist).sum()).backward()
+
+    # float64 composition on the CPU over the same neighbour table
+    p64 = {k: v.detach().cpu().double().requires_grad_(True) for k, v in layer.named_parameters()}
+    x64 = x.detach().cpu().double().requires_grad_(True)
+    i64 = idx.cpu().to(torch.int64)
+    c64 = x64 @ p64["input_spatial_transform.weight"].t()
+    d2 = ((c64[:, None, :] - c64[i64.clamp(min=0)]) ** 2).sum(2)
+    d2 = torch.where(i64 >= 0, d2, torch.zeros_like(d2))
+    feat = torch.relu(x64 @ p64["input_feature_transform.weight"].t() + p64["input_feature_transform.bias"])
+    nidx, nd2 = i64[:, 1:], d2[:, 1:]
+    w = torch.exp(-10.0 * nd2)
+    valid = (nidx >= 0)[:, :, None]
+    wf = feat[nidx.clamp(min=0)] * w[:, :, None]
+    mean = torch.where(valid, wf, torch.zeros_like(wf)).sum(1) / n_neighbours
+    mx = torch.where(valid, wf, torch.full_like(wf, -1e300)).max(1).values
+    if sumwnorm:
+        norm = torch.where(nidx >= 0, w, torch.zeros_like(w)).sum(1, keepdim=True) / n_neighbours
+        mean = torch.where(norm == 0, torch.zeros_like(mean), mean / norm)
+    acc = torch.cat([mean, mx], 1) - feat.repeat(1, 2)
+    ref = torch.relu(torch.cat([acc, x64], 1) @ p64["output_feature_transform.weight"].t()
+                     + p64["output_feature_transform.bias"])
+    assert torch.allclose(out.detach().cpu().double(), ref, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(dist.detach().cpu().double(), d2, rtol=1e-5, atol=1e-7)
+    ((ref * g_out.cpu().double()).sum() + (d2 * g_dist.cpu().double()).sum()).backward()
+
+    def close(a, b):
+        scale = b.abs().max().item()
+        return (a.detach().cpu().double() - b).abs().max().item() <= 2e-4 * scale + 1e-7
+    assert close(x.grad, x64.grad)
+    for k, v in layer.named_parameters():
+        assert close(v.grad, p64[k].grad), k
+
+
 # ------------------------------------------------------------------ condensates
 
 def run_condensates(oracle, cfg, by_max_beta, mask=None):
