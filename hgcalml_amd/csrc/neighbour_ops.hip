@@ -10,7 +10,7 @@
 // The reference's device kernels scatter with atomicAdd; here every scatter is
 // an ordered gather through the inverse neighbour index (ascending (vertex,
 // slot) per target), so results do not depend on scheduling.
-#include "hgc_common.hpp"
+#include "accumulate_rows.hpp"
 
 #include <algorithm>
 
@@ -37,31 +37,59 @@ __global__ __launch_bounds__(256) void select_knn_grad_kernel(const float *__res
                                                               const float *__restrict__ coord,
                                                               const int *__restrict__ inv_off,
                                                               const int *__restrict__ inv_slots,
-                                                              float *__restrict__ grad_coord, int n_vert, int K, int C) {
+                                                              float *__restrict__ grad_coord, int n_vert, int K, int C,
+                                                              const acc::FastDiv div_k) {
     const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const int i = (int)(t / C);
     if (i >= n_vert) return;
     const int c = (int)(t - (long long)i * C);
     const float xi = coord[(size_t)i * C + c];
 
-    float acc = 0.f;
-    for (int n = 0; n < K; ++n) {
-        const int k = idx[(size_t)i * K + n];
-        if (k < 0 || k >= n_vert) continue;
-        const float g = grad_dist[(size_t)i * K + n];
-        const float diff = coord[(size_t)k * C + c] - xi;
-        acc = (float)((double)acc - 2. * (double)g * (double)diff);
+    // loads of U slots are issued together; the additions stay in slot / list order
+    constexpr int U = 8;
+    float sum = 0.f;
+    for (int n0 = 0; n0 < K; n0 += U) {
+        int k[U];
+        float g[U], xk[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int n = min(n0 + u, K - 1);
+            k[u] = idx[(size_t)i * K + n];
+            g[u] = grad_dist[(size_t)i * K + n];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const bool ok = n0 + u < K && k[u] >= 0 && k[u] < n_vert;
+            k[u] = ok ? k[u] : -1;
+            xk[u] = coord[(size_t)(ok ? k[u] : i) * C + c];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (k[u] < 0) continue;
+            const float diff = xk[u] - xi;
+            sum = (float)((double)sum - 2. * (double)g[u] * (double)diff);
+        }
     }
     const int begin = inv_off[i], end = inv_off[i + 1];
-    for (int e = begin; e < end; ++e) {
-        const int slot = inv_slots[e];
-        const int v = slot / K;
-        const float g = grad_dist[slot];
-        const float diff = xi - coord[(size_t)v * C + c];
-        const float add = (float)(2. * (double)g * (double)diff);
-        acc = acc + add;
+    for (int e0 = begin; e0 < end; e0 += U) {
+        int slot[U];
+        float g[U], xv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) slot[u] = inv_slots[min(e0 + u, end - 1)];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            g[u] = grad_dist[slot[u]];
+            xv[u] = coord[(size_t)acc::fast_div(slot[u], div_k) * C + c];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (e0 + u >= end) break;
+            const float diff = xi - xv[u];
+            const float add = (float)(2. * (double)g[u] * (double)diff);
+            sum = sum + add;
+        }
     }
-    grad_coord[(size_t)i * C + c] = acc;
+    grad_coord[(size_t)i * C + c] = sum;
 }
 
 }  // namespace
@@ -81,7 +109,8 @@ int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const fl
     HGC_REQUIRE(d_grad_dist && d_indices && d_coord && d_inv_offsets && d_inv_slots && d_grad_coord, "null pointer");
     const long long threads = (long long)n_vert * n_coords;
     select_knn_grad_kernel<<<ceil_div(threads, 256), 256, 0, as_stream(stream)>>>(
-        d_grad_dist, d_indices, d_coord, d_inv_offsets, d_inv_slots, d_grad_coord, n_vert, n_neigh, n_coords);
+        d_grad_dist, d_indices, d_coord, d_inv_offsets, d_inv_slots, d_grad_coord, n_vert, n_neigh, n_coords,
+        acc::make_fast_div(n_neigh));
     return check_launch("select_knn_grad_kernel");
 }
 
