@@ -166,11 +166,14 @@ def main():
     inv = ops.inverse_neighbour_index(i4)
     grad_ms = event_ms(lambda: torch.ops.hgcalml.accumulate_knn_grad_slots(g4, w4, x4, i4, arg4, slots4, *inv),
                        args.steps, args.warmup)
+    # the bare K-fold row gather of the same neighbour table: what the memory system delivers
+    probe_ms = event_ms(lambda: ops.probe_row_gather(x4, i4), args.steps, 2)
+    gathered_bytes = 4.0 * n4 * K4 * F4
     bytes_fwd = 4.0 * n4 * (2 * K4 + 4 * F4)
     bytes_bwd = 4.0 * n4 * (3 * K4 + 5 * F4)
     achieved = (bytes_fwd + bytes_bwd) / ((fwd_ms[0] + grad_ms[0]) * 1e-3) / 1e9
-    log("bench: cfg4 fwd %.3f ms, grad %.3f ms, inverse index (one-off) %.3f ms -> %.1f GB/s" %
-        (fwd_ms[0], grad_ms[0], inv_ms[0], achieved))
+    log("bench: cfg4 fwd %.3f ms, grad %.3f ms, inverse index (one-off) %.3f ms -> %.1f GB/s; bare row gather %.3f ms" %
+        (fwd_ms[0], grad_ms[0], inv_ms[0], achieved, probe_ms[0]))
 
     if args.section == "roofline":
         return
@@ -187,6 +190,11 @@ def main():
         for mode in (True, False):
             m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode), 5, 2)
             extra["cfg5_condensates_ms_max_beta" if mode else "cfg5_condensates_ms_min_dist"] = round(m5[0], 3)
+        # PushKnn forward / gradient over the cfg4 neighbour table (F=128)
+        from hgcalml_amd import PushKnn
+        pf = event_ms(lambda: torch.ops.hgcalml.push_knn(w4, x4, i4), 5, 2)
+        pg = event_ms(lambda: torch.ops.hgcalml.push_knn_grad(g4[:, :F4].contiguous(), w4, x4, i4), 5, 2)
+        extra["cfg4_push_knn_fwd_ms"], extra["cfg4_push_knn_grad_ms"] = round(pf[0], 3), round(pg[0], 3)
         # one GravNet block (learned 4-D coordinates -> kNN K=64+self -> accumulate F=64 -> dense), forward + backward
         from hgcalml_amd import RaggedGravNet
         torch.manual_seed(0)
@@ -245,7 +253,11 @@ def main():
                      "fwd_ms": round(fwd_ms[0], 4), "grad_ms": round(grad_ms[0], 4),
                      "fwd_GBps": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9, 1),
                      "grad_GBps": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9, 1),
-                     "inverse_index_build_ms": round(inv_ms[0], 3)},
+                     "inverse_index_build_ms": round(inv_ms[0], 3),
+                     "row_gather_probe": {"ms": round(probe_ms[0], 4),
+                                          "gathered_TBps": round(gathered_bytes / (probe_ms[0] * 1e-3) / 1e12, 2),
+                                          "forward_over_probe": round(fwd_ms[0] / probe_ms[0], 3),
+                                          "note": "K rows of 4F bytes per vertex through L2, no arithmetic"}},
         "cpu_baseline": cpu,
         "extra": extra,
     }

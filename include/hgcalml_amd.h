@@ -288,6 +288,14 @@ int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *
                       const int *d_idxs, float *d_feat_grad, float *d_w_grad,
                       int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
 
+/* Measurement aid without a counterpart in the reference: out[v,:] = sum over
+ * the K rows d_feat[d_idxs[v,n],:] with the forward kernel's access pattern and
+ * no other arithmetic. Its run time is the rate at which the memory system
+ * delivers the K-fold re-read rows; bench.py reports the accumulation kernels
+ * against it. n_feat must be a multiple of 64. */
+int hgc_probe_row_gather(const float *d_feat, const int *d_idxs, float *d_out,
+                         int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
+
 /* ------------------------------------------------------------------ */
 /* Condensate assignment                                               */
 /* ------------------------------------------------------------------ */

@@ -577,6 +577,19 @@ def test_gravnet_block_forward_and_all_gradients(n_propagate, n_neighbours, sumw
         assert close(v.grad, p64[k].grad), k
 
 
+def test_row_gather_probe():
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(80)
+    n, K, F = 1000, 20, 128
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    idx = rng.integers(0, n, size=(n, K)).astype(np.int32)
+    got = ops.probe_row_gather(t(x), t(idx)).cpu().numpy()
+    want = np.zeros((n, F), np.float32)
+    for k in range(K):
+        want = (want + x[idx[:, k]]).astype(np.float32)
+    assert (bits(got) == bits(want)).all()
+
+
 # ------------------------------------------------------------------ condensates
 
 def run_condensates(oracle, cfg, by_max_beta, mask=None):
