@@ -11,10 +11,12 @@ returned squared distances. Inputs are resident in HBM before the timed region.
 `value` is kNN queries per second of the whole step.
 
 The `roofline` object is measured in a second timed loop of the same run (also
-K iterations, HIP events on the stream the kernels are launched on):
-accumulate_knn forward + gradient at cfg4 (N=1,000,000, K=64, F=128, banded
-neighbour table), algorithmic bytes 4*N*(2K+4F) forward and 4*N*(3K+5F)
-gradient against the 8 TB/s HBM peak.
+K iterations, HIP events on the stream the kernels are launched on) at cfg4
+(N=1,000,000, K=64, F=128, banded neighbour table): the dominant kernel, one
+launch of the accumulate_knn gradient (algorithmic bytes 4*N*(3K+5F)), with
+the forward launch (4*N*(2K+4F)) and the forward+gradient pair next to it,
+against the 8 TB/s HBM peak; plus the bare K-fold row gather of the same
+table, the rate the memory system delivers those rows at.
 
 `cpu_baseline` times the CPU oracle (a single-threaded C restatement of the
 reference CPU kernels) on this box's host: the binned kNN kernel over the full
@@ -35,12 +37,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per forward+gradient pass at full cfg4, from two hardware-counter
-# runs of this file's roofline section (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB,
-# both scaled by what the counters read for the 512 MB calibration copy below);
-# summary in profiles/accumulate_knn_cfg4_hbm_counters.txt. Counters cannot be
-# read from inside the timed run, so this is the last profiled value.
-CFG4_MEASURED_HBM_BYTES = 22.6e9
+# HBM bytes per launch at full cfg4, from two hardware-counter runs of this
+# file's roofline section (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, both scaled
+# by what the counters read for the 512 MB calibration copy below); summary in
+# profiles/accumulate_knn_cfg4_hbm_counters.txt. Counters cannot be read from
+# inside the timed run, so these are the last profiled values.
+CFG4_FWD_MEASURED_HBM_BYTES = 3.22e9
+CFG4_GRAD_MEASURED_HBM_BYTES = 19.4e9
 
 
 def log(*a):
@@ -245,14 +248,23 @@ def main():
                                "(3 binned dims, n_bins=30) + AccumulateKnn forward F=64",
                    "knn_op_ms": round(knn_ms[0], 4), "accumulate_fwd_ms": round(acc2_ms[0], 4)},
         "accumulate_fwd_grad_GBps": round(achieved, 1),
-        "roofline": {"bound": "hbm", "kernel": "accumulate_knn forward + gradient, cfg4 (N=%d, K=%d, F=%d)" % (n4, K4, F4),
-                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": CFG4_MEASURED_HBM_BYTES if args.roofline_scale == 1.0 else None,
-                     "algorithmic_bytes": bytes_fwd + bytes_bwd,
-                     "fwd_ms": round(fwd_ms[0], 4), "grad_ms": round(grad_ms[0], 4),
-                     "fwd_GBps": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9, 1),
-                     "grad_GBps": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9, 1),
+        # the dominant kernel of the graded path: one launch of the one-pass gradient kernel
+        "roofline": {"bound": "hbm",
+                     "kernel": "accumulate_grad_fused_kernel: accumulate_knn gradient (weights + features), cfg4 "
+                               "(N=%d, K=%d, F=%d), one launch" % (n4, K4, F4),
+                     "achieved": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": CFG4_GRAD_MEASURED_HBM_BYTES if args.roofline_scale == 1.0 else None,
+                     "algorithmic_bytes": bytes_bwd, "launch_ms": round(grad_ms[0], 4),
+                     "forward": {"kernel": "accumulate_fwd_wave_kernel, same workload, one launch",
+                                 "achieved": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9, 1),
+                                 "frac": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                 "traffic": CFG4_FWD_MEASURED_HBM_BYTES if args.roofline_scale == 1.0 else None,
+                                 "algorithmic_bytes": bytes_fwd, "launch_ms": round(fwd_ms[0], 4)},
+                     "forward_plus_gradient": {"achieved": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBS, 4),
+                                               "algorithmic_bytes": bytes_fwd + bytes_bwd,
+                                               "traffic": (CFG4_FWD_MEASURED_HBM_BYTES + CFG4_GRAD_MEASURED_HBM_BYTES)
+                                               if args.roofline_scale == 1.0 else None},
                      "inverse_index_build_ms": round(inv_ms[0], 3),
                      "row_gather_probe": {"ms": round(probe_ms[0], 4),
                                           "gathered_TBps": round(gathered_bytes / (probe_ms[0] * 1e-3) / 1e12, 2),

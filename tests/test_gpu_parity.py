@@ -590,6 +590,63 @@ def test_row_gather_probe():
     assert (bits(got) == bits(want)).all()
 
 
+# ------------------------------------------------------------------ empty inputs and refused arguments
+
+def test_empty_inputs_and_empty_events(oracle):
+    from hgcalml_amd import AccumulateLinKnn, BinnedSelectKnn, PushKnn, ops
+    e_f = torch.empty((0, 8), device=DEV)
+    e_i = torch.empty((0, 4), dtype=torch.int32, device=DEV)
+    e_w = torch.empty((0, 4), device=DEV)
+    out, arg = AccumulateLinKnn(e_w, e_f, e_i)
+    assert out.shape == (0, 16) and arg.shape == (0, 8)
+    assert PushKnn(e_w, e_f, e_i).shape == (0, 8)
+    off, slots = ops.inverse_neighbour_index(e_i)
+    assert off.cpu().tolist() == [0]
+    idx, dist = BinnedSelectKnn(4, torch.empty((0, 3), device=DEV), t(np.array([0, 0], np.int32)), n_bins=5)
+    assert idx.shape == (0, 4) and dist.shape == (0, 4)
+    # events without points between events with points
+    rng = np.random.default_rng(90)
+    coords = rng.random((120, 3), dtype=np.float32)
+    rs = np.array([0, 0, 50, 50, 120, 120], np.int32)
+    idx, dist = BinnedSelectKnn(6, t(coords), t(rs), n_bins=5)
+    ref_i, ref_d = oracle.canonical_knn(*oracle.BinnedSelectKnn(6, coords, rs, n_bins=5))
+    assert (idx.cpu().numpy() == ref_i).all() and (bits(dist.cpu().numpy()) == bits(ref_d)).all()
+    # a single neighbour slot
+    x = rng.standard_normal((40, 64)).astype(np.float32)
+    i1 = np.arange(40, dtype=np.int32)[:, None]
+    w1 = rng.random((40, 1), dtype=np.float32)
+    out, arg = AccumulateLinKnn(t(w1), t(x), t(i1))
+    ref, rarg = oracle.AccumulateLinKnn(w1, x, i1)
+    assert (bits(out.cpu().numpy()) == bits(ref)).all() and (arg.cpu().numpy() == rarg).all()
+
+
+def test_refused_arguments():
+    """shape errors are reported before anything is launched, with the reference op's conditions"""
+    from hgcalml_amd import AccumulateLinKnn, BinnedSelectKnn, PushKnn
+    from hgcalml_amd._lib import lib, p, stream
+    w = torch.ones((10, 4), device=DEV)
+    x = torch.ones((10, 8), device=DEV)
+    i = torch.zeros((10, 4), dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError):
+        AccumulateLinKnn(w[:, :3], x, i)                # weights and indices differ in shape
+    with pytest.raises(ValueError):
+        AccumulateLinKnn(w, x[:5], i)                   # first dimensions differ
+    with pytest.raises(ValueError):
+        PushKnn(w, x[:5], i)
+    with pytest.raises(ValueError):
+        BinnedSelectKnn(4, torch.rand((10, 3), device=DEV), torch.tensor([0, 7], dtype=torch.int32), n_bins=5)
+    with pytest.raises(ValueError):
+        BinnedSelectKnn(4, torch.rand((10, 1), device=DEV), torch.tensor([0, 10], dtype=torch.int32), n_bins=5)
+    with pytest.raises(RuntimeError):
+        AccumulateLinKnn(w.cpu(), x.cpu(), i.cpu())     # no CPU path
+    # C ABI: status code and message, nothing launched
+    out = torch.empty((10, 16), device=DEV)
+    rc = lib.hgc_accumulate_knn(p(w), p(x), p(i), p(out), None, 10, 4, 8, 16, 0, 1, stream())
+    assert rc == -1 and b"d_out_maxidxs" in lib.hgc_last_error()
+    rc = lib.hgc_accumulate_knn(p(w), p(x), p(i), p(out), None, 10, 4, 8, 99, 0, 0, stream())
+    assert rc == -1 and b"n_out_feat" in lib.hgc_last_error()
+
+
 # ------------------------------------------------------------------ condensates
 
 def run_condensates(oracle, cfg, by_max_beta, mask=None):
