@@ -3,11 +3,12 @@
 Public API (same names and signatures as the reference's Python wrappers):
 BinByCoordinates, BinnedSelectKnn, IndexReplacer, AccumulateKnn,
 AccumulateLinKnn, AccumulateKnnSumw, AccumulateLinKnnSumw, PushKnn,
-BuildAndAssignCondensatesBinned, and the RaggedGravNet layer on top of them. All of them need tensors on
+BuildAndAssignCondensatesBinned, LocalDistance, NeighbourCovariance and the RaggedGravNet layer on top of them. All of them need tensors on
 a HIP device and the in-tree libhgcalml_amd.so; there is no CPU path.
 """
 __all__ = ["BinByCoordinates", "BinnedSelectKnn", "IndexReplacer", "AccumulateKnn", "AccumulateLinKnn",
-           "AccumulateKnnSumw", "AccumulateLinKnnSumw", "PushKnn", "BuildAndAssignCondensatesBinned", "RaggedGravNet"]
+           "AccumulateKnnSumw", "AccumulateLinKnnSumw", "PushKnn", "BuildAndAssignCondensatesBinned", "RaggedGravNet",
+           "LocalDistance", "NeighbourCovariance"]
 
 
 def __getattr__(name):
@@ -25,6 +26,8 @@ def __getattr__(name):
             "AccumulateLinKnnSumw": "accknn_op",
             "PushKnn": "push_knn_op",
             "RaggedGravNet": "GravNetLayersRagged",
+            "LocalDistance": "local_distance_op",
+            "NeighbourCovariance": "neighbour_covariance_op",
             "BuildAndAssignCondensatesBinned": "assign_condensate_op",
         }[name]
         return getattr(importlib.import_module("." + mod, __name__), name)

@@ -40,6 +40,7 @@ _SIGNATURES = {
     "hgc_accumulate_knn_grad": (_c_int, [_ptr] * 9 + [_c_int] * 6 + [_ptr]),
     "hgc_accumulate_knn_grad_slots": (_c_int, [_ptr] * 10 + [_c_int] * 6 + [_ptr]),
     "hgc_select_knn_grad": (_c_int, [_ptr] * 7 + [_c_int] * 3 + [_ptr]),
+    "hgc_local_distance": (_c_int, [_ptr] * 3 + [_c_int] * 4 + [_ptr]),
     "hgc_push_knn": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),
     "hgc_push_knn_grad": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),
     "hgc_probe_row_gather": (_c_int, [_ptr] * 3 + [_c_int] * 3 + [_ptr]),

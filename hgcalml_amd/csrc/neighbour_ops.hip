@@ -6,6 +6,7 @@
 //   modules/compiled/select_knn_grad_kernel.cu.cc:81-164
 //   modules/compiled/push_knn_kernel.cc:40-62
 //   modules/compiled/push_knn_grad_kernel.cc:23-71
+//   modules/compiled/local_distance_kernel.cc:18-70
 //
 // The reference's device kernels scatter with atomicAdd; here every scatter is
 // an ordered gather through the inverse neighbour index (ascending (vertex,
@@ -92,6 +93,26 @@ __global__ __launch_bounds__(256) void select_knn_grad_kernel(const float *__res
     grad_coord[(size_t)i * C + c] = sum;
 }
 
+// one thread per (vertex, slot): serial fp32 sum over the coordinates, 0 for a
+// missing neighbour and for the vertex itself
+__global__ __launch_bounds__(256) void local_distance_kernel(const int *__restrict__ idx,
+                                                             const float *__restrict__ coord,
+                                                             float *__restrict__ dist, int C, int n_in_vert,
+                                                             long long total, int K) {
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= total) return;
+    const int i = (int)(t / K);
+    const int j = idx[t];
+    float dsq = 0.f;
+    if (j >= 0 && j < n_in_vert && j != i) {
+        for (int c = 0; c < C; ++c) {
+            const float d = coord[(size_t)i * C + c] - coord[(size_t)j * C + c];
+            dsq = dsq + d * d;
+        }
+    }
+    dist[t] = dsq;
+}
+
 }  // namespace
 }  // namespace hgc
 
@@ -112,6 +133,19 @@ int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const fl
         d_grad_dist, d_indices, d_coord, d_inv_offsets, d_inv_slots, d_grad_coord, n_vert, n_neigh, n_coords,
         acc::make_fast_div(n_neigh));
     return check_launch("select_knn_grad_kernel");
+}
+
+int hgc_local_distance(const int *d_neigh_idxs, const float *d_coords, float *d_distances, int n_coords, int n_in_vert,
+                       int n_out_vert, int n_neigh, hgc_stream_t stream) {
+    HGC_REQUIRE(n_in_vert >= 0 && n_out_vert >= 0 && n_out_vert <= n_in_vert && n_neigh >= 1 && n_coords >= 1,
+                "bad sizes");
+    HGC_REQUIRE((long long)n_out_vert * n_neigh < (1ll << 31), "tensor too large for int32 indexing");
+    if (n_out_vert == 0) return HGC_OK;
+    HGC_REQUIRE(d_neigh_idxs && d_coords && d_distances, "null pointer");
+    const long long total = (long long)n_out_vert * n_neigh;
+    local_distance_kernel<<<ceil_div(total, 256), 256, 0, as_stream(stream)>>>(d_neigh_idxs, d_coords, d_distances,
+                                                                              n_coords, n_in_vert, total, n_neigh);
+    return check_launch("local_distance_kernel");
 }
 
 int hgc_push_knn(const float *d_weights, const float *d_feat, const int *d_idxs, const int *d_inv_offsets,

@@ -297,6 +297,18 @@ def select_knn_grad(grad_distances: torch.Tensor, indices: torch.Tensor, distanc
     return out
 
 
+@torch.library.custom_op("hgcalml::local_distance", mutates_args=())
+def local_distance(coordinates: torch.Tensor, neighbour_idxs: torch.Tensor) -> torch.Tensor:
+    """modules/compiled/local_distance_module.cc: squared distances to the listed neighbours"""
+    dev = require_device(coordinates, neighbour_idxs)
+    x, idx = f32(coordinates), i32(neighbour_idxs)
+    if x.dim() != 2 or idx.dim() != 2 or idx.shape[0] > x.shape[0]:
+        raise ValueError("LocalDistanceOp expects coordinates [N,C] and neighbour indices [M<=N,K]")
+    out = torch.empty(idx.shape, dtype=torch.float32, device=dev)
+    check(lib.hgc_local_distance(p(idx), p(x), p(out), x.shape[1], x.shape[0], idx.shape[0], idx.shape[1], stream()))
+    return out
+
+
 def _push_checks(weights, features, indices):
     # modules/compiled/push_knn_kernel.cc:86-91
     if weights.dim() != 2 or features.dim() != 2 or indices.dim() != 2:

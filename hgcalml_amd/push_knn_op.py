@@ -6,6 +6,8 @@ self index is a neighbour like any other.
 """
 import torch
 
+from . import ops  # noqa: F401  (registers torch.ops.hgcalml.*)
+
 
 class _PushKnnFn(torch.autograd.Function):
     """op + registered gradient (modules/push_knn_op.py:21-36)"""

@@ -270,6 +270,16 @@ int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const fl
                         float *d_grad_coord, int n_vert, int n_neigh, int n_coords,
                         hgc_stream_t stream);
 
+/* distances[i,n] = |x_i - x_idx[i,n]|^2 (serial fp32 sum over the coordinates),
+ * 0 where idx[i,n] < 0 or idx[i,n] == i. Replaces LocalDistanceOpFunctor
+ * (modules/compiled/local_distance_kernel.h, _kernel.cc:18-70), same argument
+ * order. Its registered gradient is hgc_select_knn_grad
+ * (modules/local_distance_op.py:24-40).
+ *   d_neigh_idxs, d_distances [n_out_vert, n_neigh], d_coords [n_in_vert, n_coords]. */
+int hgc_local_distance(const int *d_neigh_idxs, const float *d_coords, float *d_distances,
+                       int n_coords, int n_in_vert, int n_out_vert, int n_neigh,
+                       hgc_stream_t stream);
+
 /* out[m,f] = sum over (v,n) with idx[v,n] == m of feat[v,f] * w[v,n]
  * (idx < 0: no neighbour). Replaces PushKnnOpFunctor
  * (modules/compiled/push_knn_kernel.h, _kernel.cc:40-62); the additions of

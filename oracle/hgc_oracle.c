@@ -17,6 +17,7 @@
  *   hgo_select_knn_grad           modules/compiled/select_knn_grad_kernel.cu.cc:81-164
  *   hgo_push_knn                  modules/compiled/push_knn_kernel.cc:40-62
  *   hgo_push_knn_grad             modules/compiled/push_knn_grad_kernel.cc:23-71
+ *   hgo_local_distance            modules/compiled/local_distance_kernel.cc:18-70
  *   hgo_box_* / hgo_assign_to_condensates
  *                                 modules/compiled/binstepper.h:100-165,
  *                                 modules/compiled/binned_assign_to_condensates_kernel.cc:23-241
@@ -36,6 +37,7 @@
  *   hgo_select_knn_grad      pinned: float64 autograd of sum((x_i - x_k)^2).
  *   hgo_push_knn             pinned: ordered unbuffered scatter-add (bitwise).
  *   hgo_push_knn_grad        pinned: float64 autograd of that scatter-add.
+ *   hgo_local_distance       pinned: the brute-force serial fp32 distance.
  *   hgo_assign_to_condensates pinned for an all-zero no_condensation_mask by a
  *                            bin-free sequential greedy; behaviour with a
  *                            non-zero mask is "parity unpinned".
@@ -758,6 +760,33 @@ void hgo_push_knn_grad(const float *grad, const float *weights,
                 acc += term;
             }
             w_grad[(size_t)v * K + n] = acc;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* local_distance: squared distances to the listed neighbours          */
+/* ------------------------------------------------------------------ */
+
+/* modules/compiled/local_distance_kernel.cc:18-70: 0 for a missing neighbour
+ * (index < 0) and for the vertex itself, else the serial fp32 sum of squared
+ * coordinate differences */
+void hgo_local_distance(const int *neigh_idxs, const float *coords,
+                        float *distances, int n_coords, int n_out_vert,
+                        int n_neigh)
+{
+    for (int i = 0; i < n_out_vert; ++i) {
+        for (int n = 0; n < n_neigh; ++n) {
+            const int j = neigh_idxs[(size_t)i * n_neigh + n];
+            float dsq = 0.f;
+            if (j >= 0 && j != i) {
+                for (int c = 0; c < n_coords; ++c) {
+                    float d = coords[(size_t)i * n_coords + c] - coords[(size_t)j * n_coords + c];
+                    float sq = d * d;
+                    dsq += sq;
+                }
+            }
+            distances[(size_t)i * n_neigh + n] = dsq;
         }
     }
 }

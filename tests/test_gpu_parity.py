@@ -590,6 +590,43 @@ def test_row_gather_probe():
     assert (bits(got) == bits(want)).all()
 
 
+def test_local_distance_and_gradient(oracle):
+    from hgcalml_amd import LocalDistance
+    rng = np.random.default_rng(81)
+    n, K, C = 2500, 12, 4
+    x = rng.standard_normal((n, C)).astype(np.float32)
+    idx = np.stack([np.concatenate([[v], rng.choice(np.delete(np.arange(n), v), K - 1, replace=False)])
+                    for v in range(n)]).astype(np.int32)
+    idx[10:40, K // 2:] = -1
+    tx = t(x).requires_grad_(True)
+    dist = LocalDistance(tx, t(idx))
+    assert (bits(dist.detach().cpu().numpy()) == bits(oracle.LocalDistance(x, idx))).all()
+    g = rng.standard_normal((n, K)).astype(np.float32)
+    (dist * t(g)).sum().backward()
+    assert (bits(tx.grad.cpu().numpy()) == bits(oracle.select_knn_grad_kernel(g, idx, x))).all()
+    # fewer index rows than coordinates (forward only)
+    d_part = torch.ops.hgcalml.local_distance(t(x), t(idx[:700]))
+    assert torch.equal(d_part, dist.detach()[:700])
+
+
+def test_neighbour_covariance(oracle):
+    from hgcalml_amd import NeighbourCovariance
+    rng = np.random.default_rng(82)
+    n, K, C, F = 1500, 10, 3, 6
+    x = rng.standard_normal((n, C)).astype(np.float32)
+    feat = rng.standard_normal((n, F)).astype(np.float32)
+    idx = np.stack([np.concatenate([[v], rng.choice(np.delete(np.arange(n), v), K - 1, replace=False)])
+                    for v in range(n)]).astype(np.int32)
+    idx[5:50, K // 2:] = -1
+    d2 = rng.random((n, K), dtype=np.float32)
+    rcov, rmean = oracle.NeighbourCovariance(x, d2, feat, idx)
+    cov, mean = NeighbourCovariance(t(x), t(d2), t(feat), t(idx))
+    assert cov.shape == (n, F, C * C) and mean.shape == (n, F, C)
+    # exp and sigmoid come from different libraries: 1e-5 relative to the largest entry
+    assert np.abs(mean.cpu().numpy() - rmean).max() <= 1e-5 * np.abs(rmean).max()
+    assert np.abs(cov.cpu().numpy() - rcov).max() <= 1e-5 * np.abs(rcov).max()
+
+
 # ------------------------------------------------------------------ empty inputs and refused arguments
 
 def test_empty_inputs_and_empty_events(oracle):

@@ -447,6 +447,44 @@ def test_accumulate_sumw_composition(oracle):
             assert (out[:, F:] == full[:, F:]).all()
 
 
+def test_local_distance_vs_brute_force(oracle):
+    from helpers import serial_distsq
+    rng = np.random.default_rng(34)
+    n, K, C = 120, 6, 5
+    x = rng.standard_normal((n, C)).astype(np.float32)
+    idx = neighbour_case(rng, n, K)
+    got = oracle.LocalDistance(x, idx)
+    for v in range(n):
+        for k in range(K):
+            j = idx[v, k]
+            want = np.float32(0) if (j < 0 or j == v) else serial_distsq(x[j:j + 1], x[v])[0]
+            assert got[v, k].view(np.int32) == np.float32(want).view(np.int32)
+    # fewer index rows than coordinates
+    assert (oracle.LocalDistance(x, idx[:50]) == got[:50]).all()
+
+
+def test_neighbour_covariance_vs_float64_formula(oracle):
+    rng = np.random.default_rng(35)
+    n, K, C, F = 90, 5, 3, 4
+    x = rng.standard_normal((n, C)).astype(np.float32)
+    feat = rng.standard_normal((n, F)).astype(np.float32)
+    idx = neighbour_case(rng, n, K)
+    d2 = rng.random((n, K), dtype=np.float32)
+    cov, mean_c = oracle.NeighbourCovariance(x, d2, feat, idx)
+    assert cov.shape == (n, F, C * C) and mean_c.shape == (n, F, C)
+    fs = 1.0 / (1.0 + np.exp(-feat.astype(np.float64))) + 1e-3
+    w = np.where(idx >= 0, np.exp(-d2.astype(np.float64)), 0.0)            # [n, K]
+    j = np.maximum(idx, 0)
+    sum_f = (w[:, :, None] * fs[j]).sum(1)                                  # [n, F]
+    sum_fc = (w[:, :, None, None] * fs[j][:, :, :, None] * x.astype(np.float64)[j][:, :, None, :]).sum(1)
+    want_mean = sum_fc / (sum_f[:, :, None] + 1e-3)
+    assert np.allclose(mean_c, want_mean, rtol=1e-4, atol=1e-6)
+    cen = x.astype(np.float64)[:, None, :] - want_mean                     # per vertex, [n, F, C]
+    outer = (cen[:, :, :, None] * cen[:, :, None, :]).reshape(n, F, C * C) * fs[:, :, None]
+    want_cov = (w[:, :, None, None] * outer[j]).sum(1) / (sum_f[:, :, None] + 1e-3)
+    assert np.allclose(cov, want_cov, rtol=1e-4, atol=1e-6)
+
+
 @pytest.mark.parametrize("by_max_beta", [True, False])
 @pytest.mark.parametrize("t_d", [0.5, 0.15])
 def test_condensates_vs_bin_free_greedy(oracle, by_max_beta, t_d):
