@@ -11,6 +11,7 @@ and through the dense layers (torch).
 import torch
 from torch import nn
 
+from . import ops
 from .accknn_op import AccumulateKnn, AccumulateKnnSumw
 from .binned_select_knn_op import BinnedSelectKnn
 
@@ -69,9 +70,13 @@ class RaggedGravNet(nn.Module):
                                     tf_compatible=False, n_bins=self.n_knn_bins)
         dist = torch.where(idx < 0, torch.zeros_like(dist), dist)
         self.update_dynamic_radius(dist.detach())
+        # the table without its self column, as tensors of their own; it lists the
+        # same vertices row by row, so the kNN's processing order applies to it too
+        nidx, ndist = idx[:, 1:].contiguous(), dist[:, 1:].contiguous()
+        ops.share_vertex_order(idx, nidx)
         if self.return_self:
-            return idx[:, 1:], dist[:, 1:], idx, dist
-        return idx[:, 1:], dist[:, 1:], None, None
+            return nidx, ndist, idx, dist
+        return nidx, ndist, None, None
 
     def collect_neighbours(self, features, neighbour_indices, distancesq):
         acc = AccumulateKnnSumw if self.sumwnorm else AccumulateKnn
@@ -90,9 +95,6 @@ class RaggedGravNet(nn.Module):
         assert x.dim() == 2 and row_splits.dim() == 1
         coordinates = self.input_spatial_transform(x)
         neighbour_indices, distancesq, sidx, sdist = self.compute_neighbours_and_distancesq(coordinates, row_splits)
-        # the strided views without the self column become the tensors the accumulation keeps
-        neighbour_indices = neighbour_indices.contiguous()
-        distancesq = distancesq.contiguous()
         outfeats = self.create_output_features(x, neighbour_indices, distancesq)
         if self.return_self:
             neighbour_indices, distancesq = sidx, sdist

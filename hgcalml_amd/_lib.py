@@ -31,14 +31,14 @@ _SIGNATURES = {
     "hgc_binned_select_knn": (_c_int, [_ptr] * 9 + [_c_int] * 7 + [_ptr]),
     "hgc_binned_select_knn_fused": (_c_int, [_ptr] * 9 + [_c_float] + [_ptr] * 2 + [_c_int] * 7 + [_ptr]),
     "hgc_binned_select_knn_pipeline_workspace_bytes": (_c_size, [_c_int] * 6),
-    "hgc_binned_select_knn_pipeline": (_c_int, [_ptr] * 3 + [_c_int] * 7 + [_c_float, _ptr, _ptr, _ptr, _c_size, _ptr]),
+    "hgc_binned_select_knn_pipeline": (_c_int, [_ptr] * 3 + [_c_int] * 7 + [_c_float, _ptr, _ptr, _ptr, _ptr, _c_size, _ptr]),
     "hgc_index_replacer": (_c_int, [_ptr, _ptr, _ptr, _c_int, _c_int, _ptr]),
     "hgc_accumulate_knn": (_c_int, [_ptr] * 5 + [_c_int] * 6 + [_ptr]),
-    "hgc_accumulate_knn_slots": (_c_int, [_ptr] * 6 + [_c_int] * 6 + [_ptr]),
+    "hgc_accumulate_knn_slots": (_c_int, [_ptr] * 7 + [_c_int] * 6 + [_ptr]),
     "hgc_inverse_neighbour_index_workspace_bytes": (_c_size, [_c_int, _c_int]),
     "hgc_inverse_neighbour_index": (_c_int, [_ptr, _c_int, _c_int, _ptr, _ptr, _ptr, _c_size, _ptr]),
     "hgc_accumulate_knn_grad": (_c_int, [_ptr] * 9 + [_c_int] * 6 + [_ptr]),
-    "hgc_accumulate_knn_grad_slots": (_c_int, [_ptr] * 10 + [_c_int] * 6 + [_ptr]),
+    "hgc_accumulate_knn_grad_slots": (_c_int, [_ptr] * 11 + [_c_int] * 6 + [_ptr]),
     "hgc_select_knn_grad": (_c_int, [_ptr] * 7 + [_c_int] * 3 + [_ptr]),
     "hgc_local_distance": (_c_int, [_ptr] * 3 + [_c_int] * 4 + [_ptr]),
     "hgc_push_knn": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),

@@ -31,7 +31,7 @@ int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
 int launch_accumulate_grad_fused(const float *g, const float *w, const float *feat, const int *maxidx,
                                  const unsigned char *maxslot, const int *inv_off, const int *inv_slots, float *gw,
                                  float *gfeat, int n_vert, int K, int F, int g_cols, bool mean_and_max, const int *idx,
-                                 hipStream_t s);
+                                 const int *order, hipStream_t s);
 
 namespace {
 
@@ -167,9 +167,10 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                                                                   const int *__restrict__ idx, float *__restrict__ out,
                                                                   int *__restrict__ out_maxidx,
                                                                   unsigned char *__restrict__ out_maxslot, int n_vert,
-                                                                  int K, int F, int out_cols, float kf) {
+                                                                  int K, int F, int out_cols, float kf,
+                                                                  const int *__restrict__ order) {
     constexpr int U = VEC == 4 ? 8 : 16;
-    const int v = wave_vertex();
+    const int v = wave_vertex(order, n_vert);
     if (v >= n_vert) return;
     const int *irow = idx + (size_t)v * K;
     const float *wrow = w + (size_t)v * K;
@@ -307,19 +308,21 @@ __global__ __launch_bounds__(256) void feature_grad_wave_kernel(const float *__r
                                                                 const int *__restrict__ inv_off,
                                                                 const int *__restrict__ inv_slots,
                                                                 float *__restrict__ gfeat, int n_vert, int K, int F,
-                                                                int g_cols, const FastDiv div_k, int n_slices, float kf) {
+                                                                int g_cols, const FastDiv div_k, int n_slices, float kf,
+                                                                const int *__restrict__ order) {
     constexpr int U = VEC == 4 ? 4 : 8;
     int m, first_block = 0;
     if (n_slices == 1) {
-        m = wave_vertex();
+        m = wave_vertex(order, n_vert);
     } else {
         const int xcd = blockIdx.x % kNumXcd, seq = blockIdx.x / kNumXcd;
         const int per_xcd = gridDim.x / kNumXcd;
         first_block = xcd % n_slices;
         const int tile = (xcd / n_slices) * per_xcd + seq;
-        m = __builtin_amdgcn_readfirstlane(tile * 4 + (int)(threadIdx.x >> 6));
+        const int i = __builtin_amdgcn_readfirstlane(tile * 4 + (int)(threadIdx.x >> 6));
+        m = i < n_vert ? (order ? __builtin_amdgcn_readfirstlane(order[i]) : i) : n_vert;
     }
-    if (m >= n_vert) return;
+    if ((uint32_t)m >= (uint32_t)n_vert) return;
     const float inv_k = 1.f / kf;  // exact when the divisor is a power of two
     const int begin = inv_off[m], end = inv_off[m + 1];
     const RowMatrix G(g, n_vert, g_cols);
@@ -419,10 +422,11 @@ template <int VEC, bool MAX>
 __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__restrict__ g, const float *__restrict__ feat,
                                                                const int *__restrict__ maxidx, const int *__restrict__ idx,
                                                                float *__restrict__ gw, int n_vert, int K, int F,
-                                                               int g_cols, float kf) {
+                                                               int g_cols, float kf,
+                                                               const int *__restrict__ order) {
     constexpr int U = 8;
     constexpr int G = 16;  // slots per reduction group: 16 mean sums + 16 max sums = 32 values
-    const int m = wave_vertex();
+    const int m = wave_vertex(order, n_vert);
     if (m >= n_vert) return;
     const int lane = lane_id();
     const int *irow = idx + (size_t)m * K;
@@ -689,7 +693,7 @@ namespace hgc {
 // push_knn (divisor = 1): out = (sum over the slots of w * feat[idx]) / divisor.
 int accumulate_forward(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
                        int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat,
-                       int n_out_feat, int mean_and_max, float divisor, hgc_stream_t stream) {
+                       int n_out_feat, int mean_and_max, float divisor, const int *d_order, hgc_stream_t stream) {
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_out_feat == n_feat * (mean_and_max ? 2 : 1), "n_out_feat must be n_feat * (mean_and_max ? 2 : 1)");
     HGC_REQUIRE((long long)n_vert * std::max(n_neigh, 2 * n_feat) < (1ll << 31), "tensor too large for int32 indexing");
@@ -707,7 +711,8 @@ int accumulate_forward(const float *d_distances, const float *d_feat, const int 
         const dim3 grid(ceil_div(n_vert, 4)), block(256);
 #define HGC_FWD(VEC, MAX)                                                                                         \
     accumulate_fwd_wave_kernel<VEC, MAX><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, \
-                                                               d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor)
+                                                               d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor, \
+                                                               d_order)
         if (mean_and_max) {
             if (vec == 4) HGC_FWD(4, true); else if (vec == 2) HGC_FWD(2, true); else HGC_FWD(1, true);
         } else {
@@ -744,18 +749,19 @@ using namespace hgc;
 extern "C" {
 
 int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
-                             int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat,
-                             int n_out_feat, int n_moments, int mean_and_max, hgc_stream_t stream) {
+                             int *d_out_maxidxs, unsigned char *d_out_maxslots, const int *d_vertex_order, int n_vert,
+                             int n_neigh, int n_feat, int n_out_feat, int n_moments, int mean_and_max,
+                             hgc_stream_t stream) {
     (void)n_moments;  // carried by the reference op, never used by its kernels
     return accumulate_forward(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, d_out_maxslots, n_vert, n_neigh,
-                              n_feat, n_out_feat, mean_and_max, (float)n_neigh, stream);
+                              n_feat, n_out_feat, mean_and_max, (float)n_neigh, d_vertex_order, stream);
 }
 
 int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
                        int *d_out_maxidxs, int n_vert, int n_neigh, int n_feat, int n_out_feat, int n_moments,
                        int mean_and_max, hgc_stream_t stream) {
-    return hgc_accumulate_knn_slots(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, nullptr, n_vert, n_neigh,
-                                    n_feat, n_out_feat, n_moments, mean_and_max, stream);
+    return hgc_accumulate_knn_slots(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, nullptr, nullptr, n_vert,
+                                    n_neigh, n_feat, n_out_feat, n_moments, mean_and_max, stream);
 }
 
 size_t hgc_inverse_neighbour_index_workspace_bytes(int n_vert, int n_neigh) {
@@ -807,7 +813,7 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
                         const int *d_max_feat_indices, const unsigned char *d_max_slots, const int *d_neigh_indices,
                         const int *d_inv_offsets, const int *d_inv_slots, float *d_out_grad_distances,
                         float *d_out_grad_features, int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
-                        int mean_and_max, float divisor, hgc_stream_t stream) {
+                        int mean_and_max, float divisor, const int *d_order, hgc_stream_t stream) {
     const bool want_w = d_out_grad_distances != nullptr, want_f = d_out_grad_features != nullptr;
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_grad_from_out_feat == n_feat * (mean_and_max ? 2 : 1),
@@ -832,7 +838,7 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
             const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
                                                         d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
                                                         d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat,
-                                                        mean_and_max != 0, d_neigh_indices, s);
+                                                        mean_and_max != 0, d_neigh_indices, d_order, s);
             if (rc <= 0) return rc;  // 1: shape not covered, use the two-kernel path
         }
         const int vec = wave_vec(n_feat, align_or);
@@ -841,7 +847,7 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
 #define HGC_FGW(VEC, MAX, P2, SL)                                                                                      \
     feature_grad_wave_kernel<VEC, MAX, P2, SL><<<fg_grid, block, 0, s>>>(                                              \
         d_grad_from_out_features, d_distances, d_max_feat_indices, d_max_slots, d_inv_offsets, d_inv_slots,            \
-        d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat, div_k, n_slices, divisor)
+        d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat, div_k, n_slices, divisor, d_order)
 #define HGC_FGW_V(VEC)                                                                                   \
     do {                                                                                                 \
         if (mean_and_max && use_slots) { if (pow2k) HGC_FGW(VEC, true, true, true); else HGC_FGW(VEC, true, false, true); } \
@@ -867,7 +873,7 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
 #define HGC_WGW(VEC, MAX)                                                                                       \
     weight_grad_wave_kernel<VEC, MAX><<<grid, block, 0, s>>>(d_grad_from_out_features, d_feat, d_max_feat_indices, \
                                                             d_neigh_indices, d_out_grad_distances, n_vert, n_neigh, \
-                                                            n_feat, n_grad_from_out_feat, divisor)
+                                                            n_feat, n_grad_from_out_feat, divisor, d_order)
         if (mean_and_max) {
             if (vec == 4) HGC_WGW(4, true); else if (vec == 2) HGC_WGW(2, true); else HGC_WGW(1, true);
         } else {
@@ -938,14 +944,15 @@ extern "C" {
 int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
                                   const int *d_max_feat_indices, const unsigned char *d_max_slots,
                                   const int *d_neigh_indices, const int *d_inv_offsets, const int *d_inv_slots,
-                                  float *d_out_grad_distances, float *d_out_grad_features, int n_vert, int n_neigh,
-                                  int n_feat, int n_grad_from_out_feat, int n_moments, int mean_and_max,
-                                  hgc_stream_t stream) {
+                                  const int *d_vertex_order, float *d_out_grad_distances, float *d_out_grad_features,
+                                  int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat, int n_moments,
+                                  int mean_and_max, hgc_stream_t stream) {
     (void)n_moments;
     HGC_REQUIRE(n_vert <= 0 || (d_out_grad_distances && d_out_grad_features), "null pointer");
     return accumulate_gradient(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices, d_max_slots,
                                d_neigh_indices, d_inv_offsets, d_inv_slots, d_out_grad_distances, d_out_grad_features,
-                               n_vert, n_neigh, n_feat, n_grad_from_out_feat, mean_and_max, (float)n_neigh, stream);
+                               n_vert, n_neigh, n_feat, n_grad_from_out_feat, mean_and_max, (float)n_neigh,
+                               d_vertex_order, stream);
 }
 
 int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
@@ -954,7 +961,7 @@ int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *
                             int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat, int n_moments,
                             int mean_and_max, hgc_stream_t stream) {
     return hgc_accumulate_knn_grad_slots(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices, nullptr,
-                                         d_neigh_indices, d_inv_offsets, d_inv_slots, d_out_grad_distances,
+                                         d_neigh_indices, d_inv_offsets, d_inv_slots, nullptr, d_out_grad_distances,
                                          d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat, n_moments,
                                          mean_and_max, stream);
 }

@@ -206,8 +206,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
     const float *__restrict__ g, const float *__restrict__ w, const float *__restrict__ feat,
     const int *__restrict__ maxidx, const unsigned char *__restrict__ maxslot, const int *__restrict__ inv_off,
     const int *__restrict__ inv_slots, float *__restrict__ gw, float *__restrict__ gfeat, int n_vert, int K, int F,
-    int g_cols, const FastDiv div_k, const int *__restrict__ idx) {
-    const int m = wave_vertex();
+    int g_cols, const FastDiv div_k, const int *__restrict__ idx, const int *__restrict__ order) {
+    const int m = wave_vertex(order, n_vert);
     if (m >= n_vert) return;
     const int lane = lane_id();
     const float kf = (float)K;
@@ -289,7 +289,7 @@ __global__ __launch_bounds__(256) void zero_padded_weight_grad_kernel(const int 
 template <int VEC, int NB>
 int launch_fused(const float *g, const float *w, const float *feat, const int *maxidx, const unsigned char *maxslot,
                  const int *inv_off, const int *inv_slots, float *gw, float *gfeat, int n_vert, int K, int F, int g_cols,
-                 bool mean_and_max, const int *idx, hipStream_t s) {
+                 bool mean_and_max, const int *idx, const int *order, hipStream_t s) {
     const dim3 grid(ceil_div(n_vert, 4)), block(256);
     const FastDiv div_k = make_fast_div(K);
     const bool pow2k = is_pow2(K);
@@ -297,7 +297,7 @@ int launch_fused(const float *g, const float *w, const float *feat, const int *m
 #define HGC_FUSED(MAX, P2, SL)                                                                                      \
     accumulate_grad_fused_kernel<VEC, NB, MAX, P2, SL><<<grid, block, 0, s>>>(g, w, feat, maxidx, maxslot, inv_off, \
                                                                               inv_slots, gw, gfeat, n_vert, K, F,    \
-                                                                              g_cols, div_k, idx)
+                                                                              g_cols, div_k, idx, order)
     if (mean_and_max && slots) { if (pow2k) HGC_FUSED(true, true, true); else HGC_FUSED(true, false, true); }
     else if (mean_and_max) { if (pow2k) HGC_FUSED(true, true, false); else HGC_FUSED(true, false, false); }
     else { if (pow2k) HGC_FUSED(false, true, false); else HGC_FUSED(false, false, false); }
@@ -310,7 +310,7 @@ int launch_fused(const float *g, const float *w, const float *feat, const int *m
 int launch_accumulate_grad_fused(const float *g, const float *w, const float *feat, const int *maxidx,
                                  const unsigned char *maxslot, const int *inv_off, const int *inv_slots, float *gw,
                                  float *gfeat, int n_vert, int K, int F, int g_cols, bool mean_and_max, const int *idx,
-                                 hipStream_t s) {
+                                 const int *order, hipStream_t s) {
     if (F % kWave != 0) return 1;
     const uintptr_t align_or = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(feat) |
                                reinterpret_cast<uintptr_t>(maxidx) | reinterpret_cast<uintptr_t>(gfeat);
@@ -327,7 +327,7 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
     int rc = check_launch("zero_padded_weight_grad_kernel");
     if (rc) return rc;
 #define HGC_ARGS \
-    g, w, feat, maxidx, maxslot, inv_off, inv_slots, gw, gfeat, n_vert, K, F, g_cols, mean_and_max, idx, s
+    g, w, feat, maxidx, maxslot, inv_off, inv_slots, gw, gfeat, n_vert, K, F, g_cols, mean_and_max, idx, order, s
     switch (vec * 10 + nb) {
         case 11: return launch_fused<1, 1>(HGC_ARGS);
         case 12: return launch_fused<1, 2>(HGC_ARGS);

@@ -77,6 +77,19 @@ __device__ __forceinline__ int wave_vertex() {
     return __builtin_amdgcn_readfirstlane(tile * 4 + (int)(threadIdx.x >> 6));
 }
 
+// The vertex a wave works on when the caller gives a processing order (a
+// permutation of the vertices, e.g. their order along a space-filling sort):
+// waves that run at the same time then work on vertices that share neighbours,
+// and the rows they gather are found in L2. Results do not depend on it.
+// Returns n_vert for waves beyond the last vertex.
+__device__ __forceinline__ int wave_vertex(const int *__restrict__ order, int n_vert) {
+    const int i = wave_vertex();
+    if (i >= n_vert) return n_vert;
+    if (!order) return i;
+    const int v = __builtin_amdgcn_readfirstlane(order[i]);
+    return (uint32_t)v < (uint32_t)n_vert ? v : n_vert;
+}
+
 // A dense [rows, cols] matrix of 4-byte elements seen through a raw buffer
 // descriptor (stride 0, num_records = size in bytes, gfx9 data format word).
 struct RowMatrix {

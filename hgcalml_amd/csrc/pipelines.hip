@@ -63,7 +63,8 @@ size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, 
 int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_splits, const int *d_direction,
                                    int n_vert, int n_coords, int n_rs, int n_neigh, int n_bins_scalar,
                                    int max_bin_dims, int tf_compat, float max_radius, int *d_indices,
-                                   float *d_dist, void *workspace, size_t workspace_bytes, hgc_stream_t stream) {
+                                   float *d_dist, int *d_out_sorting, void *workspace, size_t workspace_bytes,
+                                   hgc_stream_t stream) {
     const int n_bin_dims = std::min(max_bin_dims, n_coords);
     HGC_REQUIRE(n_vert >= 0 && n_rs >= 2, "bad sizes");
     HGC_REQUIRE(n_bins_scalar >= 1, "n_bins must be positive");
@@ -82,7 +83,7 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
     int *n_bins = reinterpret_cast<int *>(ws + L.n_bins);
     int *binass = reinterpret_cast<int *>(ws + L.binass);
     int *flat = reinterpret_cast<int *>(ws + L.flat);
-    int *sorting = reinterpret_cast<int *>(ws + L.sorting);
+    int *sorting = d_out_sorting ? d_out_sorting : reinterpret_cast<int *>(ws + L.sorting);
     int *bounds = reinterpret_cast<int *>(ws + L.bounds);
     float *scoords = reinterpret_cast<float *>(ws + L.scoords);
     int *sflat = reinterpret_cast<int *>(ws + L.sflat);

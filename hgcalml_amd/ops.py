@@ -141,13 +141,16 @@ def binned_select_knn_pipeline(coords, row_splits, direction, n_neighbours, n_bi
     n, c = coords.shape
     idx = torch.empty((n, n_neighbours), dtype=torch.int32, device=dev)
     dist = torch.empty((n, n_neighbours), dtype=torch.float32, device=dev)
+    sorting = torch.empty((n,), dtype=torch.int32, device=dev)
     nbytes = lib.hgc_binned_select_knn_pipeline_workspace_bytes(n, c, row_splits.numel(), int(n_bins), int(max_bin_dims),
                                                                 int(direction is not None))
     ws = workspace(nbytes, dev)
     check(lib.hgc_binned_select_knn_pipeline(p(coords), p(row_splits), p(direction), n, c, row_splits.numel(),
                                              int(n_neighbours), int(n_bins), int(max_bin_dims), int(tf_compatible),
                                              float(max_radius) if max_radius is not None else -1.0, p(idx), p(dist),
-                                             p(ws), ws.numel(), stream()))
+                                             p(sorting), p(ws), ws.numel(), stream()))
+    # the points' bin order is a processing order with locality for everything that runs over this table
+    set_vertex_order(idx, sorting)
     return idx, dist
 
 
@@ -162,6 +165,36 @@ def index_replacer(to_be_replaced: torch.Tensor, replacements: torch.Tensor) -> 
 
 
 # --------------------------------------------------------------------------- accumulate
+
+_VERTEX_ORDER = {}
+
+
+def set_vertex_order(indices, order):
+    """Remembers a processing order (a permutation of the vertices with spatial
+    locality) for the neighbour table `indices`; the accumulation ops look it up
+    by tensor object. Results never depend on it, only how well the gathered
+    rows are found in cache."""
+    if len(_VERTEX_ORDER) > 64:
+        for k in [k for k, v in _VERTEX_ORDER.items() if v[0]() is None]:
+            del _VERTEX_ORDER[k]
+        if len(_VERTEX_ORDER) > 64:
+            _VERTEX_ORDER.clear()
+    _VERTEX_ORDER[id(indices)] = (weakref.ref(indices), order)
+
+
+def vertex_order_of(indices):
+    hit = _VERTEX_ORDER.get(id(indices))
+    if hit is not None and hit[0]() is indices and hit[1].numel() == indices.shape[0]:
+        return hit[1]
+    return None
+
+
+def share_vertex_order(source_indices, derived_indices):
+    """`derived_indices` (e.g. the table without its self column) lists the same vertices row by row"""
+    order = vertex_order_of(source_indices)
+    if order is not None:
+        set_vertex_order(derived_indices, order)
+
 
 def _accumulate_forward(distances, features, indices, n_moments, mean_and_max, with_slots):
     dev = require_device(distances, features, indices)
@@ -180,8 +213,8 @@ def _accumulate_forward(distances, features, indices, n_moments, mean_and_max, w
     slots = None
     if with_slots and mean_and_max and k <= 254:
         slots = torch.empty((n, f), dtype=torch.uint8, device=dev)
-    check(lib.hgc_accumulate_knn_slots(p(w), p(x), p(idx), p(out), p(maxidx), p(slots), n, k, f, out.shape[1],
-                                       int(n_moments), int(mean_and_max), stream()))
+    check(lib.hgc_accumulate_knn_slots(p(w), p(x), p(idx), p(out), p(maxidx), p(slots), p(vertex_order_of(indices)),
+                                       n, k, f, out.shape[1], int(n_moments), int(mean_and_max), stream()))
     return out, maxidx, slots
 
 
@@ -253,8 +286,8 @@ def _accumulate_backward(grad_from_out_features, distances, features, neigh_indi
     gw = torch.empty((n, k), dtype=torch.float32, device=dev)
     gx = torch.empty((n, f), dtype=torch.float32, device=dev)
     check(lib.hgc_accumulate_knn_grad_slots(p(g), p(w), p(x), p(mi), p(max_slots), p(idx), p(inv_offsets),
-                                            p(inv_slots), p(gw), p(gx), n, k, f, g.shape[1], 0, int(mean_and_max),
-                                            stream()))
+                                            p(inv_slots), p(vertex_order_of(neigh_indices)), p(gw), p(gx), n, k, f,
+                                            g.shape[1], 0, int(mean_and_max), stream()))
     return gw, gx
 
 

@@ -627,6 +627,50 @@ def test_neighbour_covariance(oracle):
     assert np.abs(cov.cpu().numpy() - rcov).max() <= 1e-5 * np.abs(rcov).max()
 
 
+def test_vertex_processing_order_changes_nothing(oracle):
+    """the kNN hands its bin order to the accumulation as a processing order:
+    same bits with it, without it and with an arbitrary permutation"""
+    from hgcalml_amd import AccumulateKnn, BinnedSelectKnn, ops
+    from hgcalml_amd._lib import check, lib, p, stream
+    cfg = workloads.cfg2(scale=0.04)
+    coords = t(cfg["coords"])
+    n = coords.shape[0]
+    rs = t(np.array([0, n // 3, n], np.int32))
+    idx, dist = BinnedSelectKnn(16, coords, rs, n_bins=10)
+    order = ops.vertex_order_of(idx)
+    assert order is not None and sorted(order.cpu().tolist()) == list(range(n))
+    F = 128
+    rng = np.random.default_rng(83)
+    x = t(rng.standard_normal((n, F)).astype(np.float32))
+    w = torch.exp(-10 * dist)
+    g = t(rng.standard_normal((n, 2 * F)).astype(np.float32))
+    inv = ops.inverse_neighbour_index(idx)
+
+    def run(order_tensor):
+        out = torch.empty((n, 2 * F), device=DEV)
+        arg = torch.empty((n, F), dtype=torch.int32, device=DEV)
+        slots = torch.empty((n, F), dtype=torch.uint8, device=DEV)
+        check(lib.hgc_accumulate_knn_slots(p(w), p(x), p(idx), p(out), p(arg), p(slots), p(order_tensor), n, 16, F,
+                                           2 * F, 0, 1, stream()))
+        gw, gx = torch.empty((n, 16), device=DEV), torch.empty((n, F), device=DEV)
+        check(lib.hgc_accumulate_knn_grad_slots(p(g), p(w), p(x), p(arg), p(slots), p(idx), p(inv[0]), p(inv[1]),
+                                                p(order_tensor), p(gw), p(gx), n, 16, F, 2 * F, 0, 1, stream()))
+        gw2, gx2 = torch.empty((n, 16), device=DEV), torch.empty((n, F), device=DEV)
+        check(lib.hgc_accumulate_knn_grad_slots(p(g), p(w), p(x), p(arg), None, p(idx), p(inv[0]), p(inv[1]),
+                                                p(order_tensor), p(gw2), p(gx2), n, 16, F, 2 * F, 0, 1, stream()))
+        return out, arg, slots, gw, gx, gx2
+    base = run(None)
+    shuffled = t(rng.permutation(n).astype(np.int32))
+    for o in (order, shuffled):
+        for a, b in zip(base, run(o)):
+            assert torch.equal(a, b)
+    ref, rarg = oracle.AccumulateLinKnn(w.cpu().numpy(), x.cpu().numpy(), idx.cpu().numpy())
+    assert (bits(base[0].cpu().numpy()) == bits(ref)).all() and (base[1].cpu().numpy() == rarg).all()
+    # the wrapper finds the order by itself
+    out, _ = AccumulateKnn(10 * dist, x, idx)
+    assert torch.equal(out, base[0])
+
+
 # ------------------------------------------------------------------ empty inputs and refused arguments
 
 def test_empty_inputs_and_empty_events(oracle):
