@@ -19,7 +19,10 @@
 //   * The K-1 best keys live in registers, sorted across the lanes (rank r in
 //     lane r%64, register r/64). A ballot finds the candidates that beat the
 //     current K-th key; each is inserted with one DPP wave shift and two
-//     compares, and the new K-th key is read back with a readlane.
+//     compares, and the new K-th key is read back with a readlane. When 16 or
+//     more of a step's 64 candidates enter (the first steps of every query), the
+//     step is sorted across the lanes by a bitonic network and merged into the
+//     list in one go instead.
 //   * The shell loop stops exactly as the reference does: list full and
 //     ((bw*d)*bw)*d > K-th distance, or no bin of the shell inside the grid.
 //   * No LDS, no atomics, no barriers; every wave exits on its own.
@@ -130,6 +133,65 @@ __device__ __forceinline__ void sorted_insert(uint64_t (&key)[S], uint64_t c) {
         }
     }
 }
+
+// ---- bulk insert: sort a batch of 64 keys across the lanes and merge it into the list ----
+//
+// A compare-exchange step of the bitonic network between lanes i and i^J. Which
+// of the two lanes keeps the smaller key is a compile-time lane pattern, so it
+// sits in scalar registers as a constant and the swap decision is one 64-bit
+// compare plus a scalar xor; keys are unique apart from the empty key, for which
+// a swap changes nothing.
+constexpr uint64_t keeps_min_mask(int k, int j) {
+    uint64_t m = 0;
+    for (int i = 0; i < 64; ++i)
+        if (((i & j) == 0) == ((i & k) == 0)) m |= 1ull << i;
+    return m;
+}
+
+template <int K, int J>
+__device__ __forceinline__ uint64_t compare_exchange(uint64_t key) {
+    constexpr uint64_t kMin = keeps_min_mask(K, J);
+    const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)key, J, kWave);
+    const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(key >> 32), J, kWave);
+    const uint64_t other = ((uint64_t)hi << 32) | lo;
+    const uint64_t lt = __ballot(other < key);
+    // the lane that keeps the smaller key swaps when the other one is smaller, its partner when not
+    const bool swap = __builtin_amdgcn_inverse_ballot_w64(lt ^ ~kMin);
+    return swap ? other : key;
+}
+
+template <int K>
+__device__ __forceinline__ uint64_t bitonic_merge_steps(uint64_t key) {
+    if constexpr (K >= 64) key = compare_exchange<K, 32>(key);
+    if constexpr (K >= 32) key = compare_exchange<K, 16>(key);
+    if constexpr (K >= 16) key = compare_exchange<K, 8>(key);
+    if constexpr (K >= 8) key = compare_exchange<K, 4>(key);
+    if constexpr (K >= 4) key = compare_exchange<K, 2>(key);
+    return compare_exchange<K, 1>(key);
+}
+
+// ascending sort of one key per lane
+__device__ __forceinline__ uint64_t wave_sort_u64(uint64_t key) {
+    key = bitonic_merge_steps<2>(key);
+    key = bitonic_merge_steps<4>(key);
+    key = bitonic_merge_steps<8>(key);
+    key = bitonic_merge_steps<16>(key);
+    key = bitonic_merge_steps<32>(key);
+    return bitonic_merge_steps<64>(key);
+}
+
+// the 64 smallest of an ascending list and an ascending batch, ascending:
+// min(list[i], batch[63-i]) is a bitonic sequence, six more steps sort it
+__device__ __forceinline__ uint64_t merge_lowest_64(uint64_t list, uint64_t batch) {
+    const int mirror = (kWave - 1) - lane_id();
+    const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)batch, mirror, kWave);
+    const uint32_t hi = (uint32_t)__shfl((int)(uint32_t)(batch >> 32), mirror, kWave);
+    const uint64_t rev = ((uint64_t)hi << 32) | lo;
+    return bitonic_merge_steps<128>(rev < list ? rev : list);
+}
+
+// below this many entering candidates in a step of 64 the one-by-one insert is cheaper
+constexpr int kBulkInsertMin = 16;
 
 // q = x / w, r = x % w for 0 <= x < 2^23 and small w, without an integer divide
 __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, int &r) {
@@ -328,8 +390,13 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                     if (has_radius) valid = valid && dsq <= p.radius_sq;
                     const uint32_t id = MAPPED ? (uint32_t)p.sorting[jj] : (uint32_t)jj;
                     const uint64_t ck = ((uint64_t)__float_as_uint(dsq) << 32) | id;
-                    uint64_t beats = __ballot(valid && ck < thr);
+                    const bool enters = valid && ck < thr;
+                    uint64_t beats = __ballot(enters);
                     if (beats) {
+                        if (S == 1 && __popcll(beats) >= kBulkInsertMin) {
+                            key[0] = merge_lowest_64(key[0], wave_sort_u64(enters ? ck : kEmptyKey));
+                            beats = 0;
+                        }
                         while (beats) {
                             const int src = __ffsll((long long)beats) - 1;
                             beats &= beats - 1;
