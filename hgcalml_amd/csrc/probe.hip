@@ -26,22 +26,28 @@ __global__ __launch_bounds__(256) void row_gather_probe_kernel(const float *__re
         float sum[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) sum[e] = 0.f;
-        for (int n0 = 0; n0 < K; n0 += U) {
+        int n0 = 0;
+        for (; n0 + U <= K; n0 += U) {  // full chunks: all U row loads in flight
             float x[U][VEC];
             int j[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int jj = n0 + u < K ? irow[n0 + u] : v;
+                const int jj = irow[n0 + u];
                 j[u] = (uint32_t)jj < (uint32_t)n_vert ? jj : v;  // slots without a neighbour re-read the own row
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) X.load<VEC>(j[u], lane_bytes, x[u]);
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (n0 + u >= K) break;  // wave-uniform
+            for (int u = 0; u < U; ++u)
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) sum[e] += x[u][e];
-            }
+        }
+        for (; n0 < K; ++n0) {  // K not a multiple of U
+            const int jj = irow[n0];
+            float xs[VEC];
+            X.load<VEC>((uint32_t)jj < (uint32_t)n_vert ? jj : v, lane_bytes, xs);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) sum[e] += xs[e];
         }
         store_vec<VEC>(out + (size_t)v * F + fb, sum);
     }
