@@ -822,3 +822,31 @@ def test_condensates_keep_noise_structure(oracle):
         # gathering the assignment at the alpha indices gives 0..n-1 per event
         assert (a1[al1[n1[e]:n1[e + 1]], 0] == np.arange(n1[e + 1] - n1[e])).all()
     assert c1.sum() == len(al1)
+
+
+@pytest.mark.parametrize("keep_noise", [False, True])
+def test_condensates_ragged_index_helpers_on_device(keep_noise):
+    """the chain of the reference's own test (tests/unit/condensate.py:48-112) on the GPU"""
+    from hgcalml_amd import BuildAndAssignCondensatesBinned
+    from hgcalml_amd.assign_condensate_op import calc_ragged_cond_indices, calc_ragged_shower_indices
+    cfg = workloads.cfg5(scale=0.03, n_events=3)
+    args = [t(cfg[k]) for k in ("ccoords", "betas", "dist", "row_splits")]
+    assignment, asso, alpha, is_cond, ncond = BuildAndAssignCondensatesBinned(*args, 0.4, keep_noise=keep_noise,
+                                                                              assign_by_max_beta=False)
+    sh = calc_ragged_shower_indices(assignment, args[3])
+    rc, rev, flat = calc_ragged_cond_indices(assignment, alpha, ncond, args[3])
+    assert torch.equal(sh.nested_row_splits[0], rc.nested_row_splits[0])
+    a = assignment[:, 0]
+    per_hit = sh.gather(a)
+    per_cond = rc.gather(a).flat_values
+    # every hit of a shower carries the assignment of the shower's condensation point
+    n_showers = per_hit.nested_row_splits[1].numel() - 1
+    owner = torch.searchsorted(per_hit.nested_row_splits[1][1:].contiguous(),
+                               torch.arange(per_hit.flat_values.numel(), device=DEV), right=True)
+    assert n_showers == per_cond.numel() and torch.equal(per_hit.flat_values, per_cond[owner])
+    # both reverse indices bring the condensation point's value back to every hit
+    assert torch.equal(per_cond[flat[:, 0].to(torch.int64)], a)
+    ev_start = rc.nested_row_splits[0][:-1]
+    assert torch.equal(per_cond[ev_start[rev[:, 0].to(torch.int64)] + rev[:, 1].to(torch.int64)], a)
+    if keep_noise:
+        assert (a >= 0).all()
