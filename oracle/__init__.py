@@ -273,7 +273,7 @@ def BinnedSelectKnn(K, coords, row_splits, direction=None, n_bins=None, max_bin_
                     tf_compatible=False, max_radius=None, raw_slot_order=True, opt_level_0=False):
     """Reference wrapper, then (only if ``max_radius`` > 0) the radius mask of
     modules/compiled/select_knn_kernel.cc:158,244-245: neighbours with
-    d^2 > r^2 become (-1, 0.0). The reference wrapper itself ignores
+    d^2 > r^2 become padding ((-1, 0.0), or (self, 0.0) in tf_compatible mode). The reference wrapper itself ignores
     ``max_radius``; pass ``None`` to get exactly what it returns."""
     coords = np.asarray(coords, np.float32)
     row_splits = np.asarray(row_splits, np.int32)
@@ -302,7 +302,10 @@ def BinnedSelectKnn(K, coords, row_splits, direction=None, n_bins=None, max_bin_
         rsq = np.float32(r * r)
         outside = dist > rsq
         outside[:, 0] = False
-        idx = np.where(outside, np.int32(-1), idx)
+        # a neighbour beyond the radius is never filled in, so its slot keeps the
+        # default: -1, or the vertex itself in tf_compatible mode (select_knn_kernel.cc:61-84)
+        pad = np.arange(idx.shape[0], dtype=np.int32)[:, None] if tf_compatible else np.int32(-1)
+        idx = np.where(outside, pad, idx)
         dist = np.where(outside, np.float32(0.), dist)
     return idx, dist
 
