@@ -262,7 +262,7 @@ def grad_tolerance(g, x, idx, w, K):
     return 1e-5 * scale + 1e-30
 
 
-@pytest.mark.parametrize("K,F", [(8, 4), (16, 32), (64, 64), (12, 128), (5, 7), (64, 96), (9, 384)])
+@pytest.mark.parametrize("K,F", [(8, 4), (16, 32), (64, 64), (12, 128), (5, 7), (64, 96), (9, 384), (260, 64), (255, 128)])
 def test_accumulate_gradient(oracle, K, F):
     rng = np.random.default_rng(20 + K + F)
     d, x, idx = make_acc_case(rng, 300, K, F)
