@@ -222,12 +222,21 @@ def main():
         small = workloads.cfg4(scale=0.1)
         f_s, b_s = cpu_baseline_accumulate(small)
         ns = len(small["indices"])
+        import oracle
+        c5_cpu = workloads.cfg5()
+        t_c = time.perf_counter()
+        oracle.BuildAndAssignCondensatesBinned(c5_cpu["ccoords"], c5_cpu["betas"], c5_cpu["dist"], c5_cpu["row_splits"],
+                                               c5_cpu["beta_threshold"], assign_by_max_beta=True)
+        cond_s = time.perf_counter() - t_c
         cpu = {"value": round(qps, 1), "unit": "queries/s", "cores": 1, "kind": "port",
                "sample": "5 passes over all %d queries of cfg2 through the oracle's binned_select_knn kernel "
                          "(gcc -O2, %.1f s); binning/sort glue not included" % (n2, secs),
                "accumulate_fwd_grad_GBps": round((4.0 * ns * (2 * K4 + 4 * F4) + 4.0 * ns * (3 * K4 + 5 * F4)) /
                                                  (f_s + b_s) / 1e9, 4),
                "accumulate_sample": "cfg4 at N=%d (fwd %.2f s, grad %.2f s)" % (ns, f_s, b_s),
+               "condensates_cfg5_ms": round(cond_s * 1e3, 1),
+               "condensates_sample": "all of cfg5 (8 events, 500k hits, max-beta mode) through the oracle's wrapper "
+                                     "(numpy glue + C kernel)",
                "host_cpus": os.cpu_count()}
         log("bench: CPU oracle kNN %.0f queries/s (%.1f s)" % (qps, secs))
 
