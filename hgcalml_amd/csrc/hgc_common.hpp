@@ -104,13 +104,38 @@ __device__ __forceinline__ uint64_t wave_shift_up1_u64(uint64_t v, uint64_t into
     return ((uint64_t)hi << 32) | lo;
 }
 
-// inclusive prefix sum over the 64 lanes
-__device__ __forceinline__ int wave_inclusive_sum(int v) {
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        int t = __shfl_up(v, off, kWave);
-        if (lane_id() >= off) v += t;
-    }
+// DPP controls (gfx9 encoding): shift right by n lanes inside each row of 16,
+// broadcast of lane 15 of each row to the next row, of lane 31 to the upper half.
+constexpr int kDppRowShr = 0x110;
+constexpr int kDppRowBcast15 = 0x142;
+constexpr int kDppRowBcast31 = 0x143;
+
+// v of the lane `CTRL` names, 0 where that lane does not exist or the row is masked off
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// inclusive prefix sum over the 64 lanes (wrapping arithmetic)
+__device__ __forceinline__ int wave_inclusive_sum(int x) {
+    uint32_t v = (uint32_t)x;
+    v += dpp_or_zero<kDppRowShr + 1, 0xf>(v);
+    v += dpp_or_zero<kDppRowShr + 2, 0xf>(v);
+    v += dpp_or_zero<kDppRowShr + 4, 0xf>(v);
+    v += dpp_or_zero<kDppRowShr + 8, 0xf>(v);
+    v += dpp_or_zero<kDppRowBcast15, 0xa>(v);
+    v += dpp_or_zero<kDppRowBcast31, 0xc>(v);
+    return (int)v;
+}
+
+// inclusive prefix maximum over the 64 lanes
+__device__ __forceinline__ uint32_t wave_inclusive_max(uint32_t v) {
+    v = max(v, dpp_or_zero<kDppRowShr + 1, 0xf>(v));
+    v = max(v, dpp_or_zero<kDppRowShr + 2, 0xf>(v));
+    v = max(v, dpp_or_zero<kDppRowShr + 4, 0xf>(v));
+    v = max(v, dpp_or_zero<kDppRowShr + 8, 0xf>(v));
+    v = max(v, dpp_or_zero<kDppRowBcast15, 0xa>(v));
+    v = max(v, dpp_or_zero<kDppRowBcast31, 0xc>(v));
     return v;
 }
 

@@ -193,6 +193,18 @@ __device__ __forceinline__ uint64_t merge_lowest_64(uint64_t list, uint64_t batc
 // below this many entering candidates in a step of 64 the one-by-one insert is cheaper
 constexpr int kBulkInsertMin = 16;
 
+// Candidates of one batch of segments that are walked per refill of a wave's
+// strip of segment marks (one byte of LDS each); a multiple of 512.
+constexpr int kMarkCap = 2048;
+
+// LDS traffic of one wave stays in program order; this keeps the compiler from
+// moving the wave's own accesses across the point where lanes exchange data.
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // q = x / w, r = x % w for 0 <= x < 2^23 and small w, without an integer divide
 __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, int &r) {
     q = (int)((float)x * inv_w);
@@ -208,9 +220,11 @@ __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, 
 
 template <int C, int S, bool MAPPED>
 __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
+    __shared__ __attribute__((aligned(8))) uint8_t mark_strips[4][kMarkCap];
     const int lane = lane_id();
     const int tile = xcd_contiguous_block(blockIdx.x, gridDim.x);
     const int q = tile * 4 + (threadIdx.x >> 6);  // one query per wave
+    uint8_t *const marks = mark_strips[threadIdx.x >> 6];
     if (q >= p.n_vert) return;
 
     const int K = p.K;
@@ -366,54 +380,62 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                 const int seg_end_off = wave_inclusive_sum(seg_len);
                 const int seg_off = seg_end_off - seg_len;
                 const int total = readlane_i32(seg_end_off, kWave - 1);
+                const int seg_delta = seg_start - seg_off;  // candidate position -> point index, for the owner
 
                 // ---- walk the concatenated candidates, 64 per step ----
-                for (int t = 0; t < total; t += kWave) {
-                    const int c = t + lane;
-                    // last segment whose offset is <= c (empty ones share the
-                    // offset of their successor, so the last one is the owner)
-                    int s_lo = 0;
-#pragma unroll
-                    for (int step = 32; step > 0; step >>= 1) {
-                        const int probe = s_lo + step;
-                        const int o = __shfl(seg_off, probe, kWave);
-                        if (o <= c) s_lo = probe;
-                    }
-                    const int j = __shfl(seg_start, s_lo, kWave) + (c - __shfl(seg_off, s_lo, kWave));
-                    bool valid = c < total && j != q;
-                    const int jj = valid ? j : q;
-                    if (p.use_direction && valid) {
-                        const int dj = p.direction[jj];
-                        if (dj == 1 || dj == 2) valid = false;  // may not be a neighbour
-                    }
-                    const float dsq = dist_sq<C>(qc, p.coord, jj, p.n_coords, qrow);
-                    if (has_radius) valid = valid && dsq <= p.radius_sq;
-                    const uint32_t id = MAPPED ? (uint32_t)p.sorting[jj] : (uint32_t)jj;
-                    const uint64_t ck = ((uint64_t)__float_as_uint(dsq) << 32) | id;
-                    const bool enters = valid && ck < thr;
-                    uint64_t beats = __ballot(enters);
-                    if (beats) {
-                        if (S == 1 && __popcll(beats) >= kBulkInsertMin) {
-                            key[0] = merge_lowest_64(key[0], wave_sort_u64(enters ? ck : kEmptyKey));
-                            beats = 0;
+                // Every non-empty segment marks its first position of the list with its
+                // lane number + 1 in this wave's strip of LDS; the owner of a position
+                // is then the prefix maximum of the marks (offsets rise with the lane).
+                uint32_t owner_carry = 0;
+                for (int c0 = 0; c0 < total; c0 += kMarkCap) {
+                    const int chunk = min(kMarkCap, total - c0);
+                    for (int base = 0; base < chunk; base += kWave * 8)
+                        *reinterpret_cast<uint64_t *>(marks + base + lane * 8) = 0;
+                    wave_lds_fence();
+                    const int rel = seg_off - c0;
+                    if (seg_len > 0 && rel >= 0 && rel < chunk) marks[rel] = (uint8_t)(lane + 1);
+                    wave_lds_fence();
+                    for (int t = 0; t < chunk; t += kWave) {
+                        const int c = c0 + t + lane;
+                        uint32_t owner = wave_inclusive_max(marks[t + lane]);
+                        owner = max(owner, owner_carry);
+                        owner_carry = (uint32_t)readlane_i32((int)owner, kWave - 1);
+                        const int j = c + __shfl(seg_delta, (int)owner - 1, kWave);
+                        bool valid = c < total && j != q;
+                        const int jj = valid ? j : q;
+                        const uint32_t id = MAPPED ? (uint32_t)p.sorting[jj] : (uint32_t)jj;
+                        const float dsq = dist_sq<C>(qc, p.coord, jj, p.n_coords, qrow);
+                        if (p.use_direction && valid) {
+                            const int dj = p.direction[jj];
+                            if (dj == 1 || dj == 2) valid = false;  // may not be a neighbour
                         }
-                        while (beats) {
-                            const int src = __ffsll((long long)beats) - 1;
-                            beats &= beats - 1;
-                            const uint64_t cand = readlane_u64(ck, src);
-                            if (!spare_rank) {  // no spare rank: re-check against the current K-th key
-                                uint64_t kth = kEmptyKey;
-#pragma unroll
-                                for (int s = 0; s < S; ++s)
-                                    if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
-                                const uint32_t ch = (uint32_t)(cand >> 32), kh = (uint32_t)(kth >> 32);
-                                if (ch > kh || (ch == kh && (uint32_t)cand >= (uint32_t)kth)) continue;
+                        valid = valid && (!has_radius || dsq <= p.radius_sq);
+                        const uint64_t ck = ((uint64_t)__float_as_uint(dsq) << 32) | id;
+                        const bool enters = valid && ck < thr;
+                        uint64_t beats = __ballot(enters);
+                        if (beats) {
+                            if (S == 1 && __popcll(beats) >= kBulkInsertMin) {
+                                key[0] = merge_lowest_64(key[0], wave_sort_u64(enters ? ck : kEmptyKey));
+                                beats = 0;
                             }
-                            sorted_insert<S>(key, cand);
-                        }
+                            while (beats) {
+                                const int src = __ffsll((long long)beats) - 1;
+                                beats &= beats - 1;
+                                const uint64_t cand = readlane_u64(ck, src);
+                                if (!spare_rank) {  // no spare rank: re-check against the current K-th key
+                                    uint64_t kth = kEmptyKey;
 #pragma unroll
-                        for (int s = 0; s < S; ++s)
-                            if (s == kth_level) thr = readlane_u64(key[s], kth_lane);
+                                    for (int s = 0; s < S; ++s)
+                                        if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
+                                    const uint32_t ch = (uint32_t)(cand >> 32), kh = (uint32_t)(kth >> 32);
+                                    if (ch > kh || (ch == kh && (uint32_t)cand >= (uint32_t)kth)) continue;
+                                }
+                                sorted_insert<S>(key, cand);
+                            }
+#pragma unroll
+                            for (int s = 0; s < S; ++s)
+                                if (s == kth_level) thr = readlane_u64(key[s], kth_lane);
+                        }
                     }
                 }
             }
