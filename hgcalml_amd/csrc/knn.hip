@@ -205,21 +205,22 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// q = x / w, r = x % w for 0 <= x < 2^23 and small w, without an integer divide
+// q = x / w, r = x % w for 0 <= x < 2^23 and small w, without an integer divide:
+// the float quotient is off by at most one, the remainder says which way
 __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, int &r) {
     q = (int)((float)x * inv_w);
     r = x - q * w;
-    if (r < 0) {
-        r += w;
-        --q;
-    } else if (r >= w) {
-        r -= w;
-        ++q;
-    }
+    const int fix = (r >= w ? 1 : 0) - (r < 0 ? 1 : 0);
+    q += fix;
+    r -= fix * w;
 }
 
-template <int C, int S, bool MAPPED>
+// C: coordinates per point, NB: binned dimensions (0 for either: taken from the
+// arguments), S: registers of the sorted list per lane, MAPPED: results in the
+// index space and at the positions of `sorting`.
+template <int C, int NB, int S, bool MAPPED>
 __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
+    constexpr int kDims = NB > 0 ? NB : kMaxBinDims;  // array extents
     __shared__ __attribute__((aligned(8))) uint8_t mark_strips[4][kMarkCap];
     const int lane = lane_id();
     const int tile = xcd_contiguous_block(blockIdx.x, gridDim.x);
@@ -252,12 +253,12 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
             for (int c = 0; c < C; ++c) qc[c] = qrow[c];
         }
 
-        const int B = p.n_bin_dim;
-        int nb[kMaxBinDims], qb[kMaxBinDims];
+        const int B = NB > 0 ? NB : p.n_bin_dim;
+        int nb[kDims], qb[kDims];
         int cells_per_event = 1;
         int reach_max = 0;  // beyond this shell distance no bin is inside the grid
 #pragma unroll
-        for (int i = 0; i < kMaxBinDims; ++i) {
+        for (int i = 0; i < kDims; ++i) {
             nb[i] = 1;
             qb[i] = 0;
             if (i < B) {
@@ -270,14 +271,15 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
         const int event_base = cells_per_event * (p.bin_idx[q] / cells_per_event);
         const int nb_last = nb[B - 1], qb_last = qb[B - 1];
         const float bw = p.bin_width[0];
+        const float bins_per_unit = 1.001f / bw;  // generous by 0.1 %, for the pruning bound only
 
         // Position of the query inside its own bin, in bin widths: to_lower[i] is a
         // lower bound of its distance to the bin's lower edge, to_upper[i] to the
         // upper edge (both 0 when the binning shift is unknown). They tighten the
         // lower bound of the distance to neighbouring bins used for pruning.
-        float to_lower[kMaxBinDims], to_upper[kMaxBinDims];
+        float to_lower[kDims], to_upper[kDims];
 #pragma unroll
-        for (int i = 0; i < kMaxBinDims; ++i) {
+        for (int i = 0; i < kDims; ++i) {
             to_lower[i] = 0.f;
             to_upper[i] = 0.f;
             if (i < B && p.shift) {
@@ -299,7 +301,17 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
         const bool spare_rank = S * kWave > Kn;
         uint64_t thr = kEmptyKey;  // current K-th key: candidates at or above it cannot enter
 
-        for (int d = 0; d <= reach_max; ++d) {
+        // Shell 0 (the query's own bin) never ends the search. When it cannot fill
+        // the list either (so that it cannot prune shell 1), it is walked together
+        // with shell 1: every row of that shell then takes its whole run of the last
+        // dimension, and the run of the centre row contains the own bin.
+        bool with_own_bin = false;
+        {
+            const int own = p.bin_idx[q];
+            if (reach_max > 0 && own + 1 < p.n_bboundaries)
+                with_own_bin = p.bin_boundaries[own + 1] - p.bin_boundaries[own] <= Kn;
+        }
+        for (int d = with_own_bin ? 1 : 0; d <= reach_max; ++d) {
             const int W = 2 * d + 1;
             const float inv_W = 1.f / (float)W;
             int n_rows = 1;
@@ -318,57 +330,54 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                 if (has_radius) reach2 = fminf(reach2, p.radius_sq);
                 if (slot < n_slots) {
                     int row = slot >> 1;
-                    const int second = slot & 1;
-                    bool inside = true, on_face = false;
-                    int off[kMaxBinDims];
-#pragma unroll
-                    for (int i = kMaxBinDims - 2; i >= 0; --i) {
-                        off[i] = 0;
-                        if (i < B - 1) {
-                            int digit;
-                            divmod_small(row, W, inv_W, row, digit);
-                            off[i] = digit - d;
-                        }
-                    }
+                    const bool second = slot & 1;
+                    bool inside = true, on_face = d == 0 || (d == 1 && with_own_bin);
                     int cell = 0;
                     float gap2 = 0.f;  // squared lower bound of the distance to this row of bins
+                    int off[kDims];
 #pragma unroll
-                    for (int i = 0; i < kMaxBinDims - 1; ++i) {
+                    for (int i = kDims - 2; i >= 0; --i) {
+                        off[i] = 0;
                         if (i < B - 1) {
-                            const int k = qb[i] + off[i];
-                            inside = inside && k >= 0 && k < nb[i];
-                            on_face = on_face || off[i] == d || off[i] == -d;
-                            cell = cell * nb[i] + k;
+                            if (i > 0) {
+                                int digit;
+                                divmod_small(row, W, inv_W, row, digit);
+                                off[i] = digit - d;
+                            } else {
+                                off[i] = row - d;  // what is left is the leading digit
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < kDims - 1; ++i) {
+                        if (i < B - 1) {
                             const int o = off[i];
-                            const float g = o > 0 ? ((float)(o - 1) + to_upper[i]) * bw
-                                                  : (o < 0 ? ((float)(-o - 1) + to_lower[i]) * bw : 0.f);
+                            const int k = qb[i] + o;
+                            inside = inside && (uint32_t)k < (uint32_t)nb[i];
+                            on_face = on_face || o == d || o == -d;
+                            cell = cell * nb[i] + k;
+                            const float edge = o > 0 ? to_upper[i] : to_lower[i];
+                            const float g = o == 0 ? 0.f : ((float)(abs(o) - 1) + edge) * bw;
                             gap2 += g * g;
                         }
                     }
-                    int lo, hi;
-                    if (on_face || d == 0) {  // the whole run of the last dimension
-                        lo = qb_last - d;
-                        hi = second ? lo - 1 : qb_last + d;
-                        // bins of the run that are provably too far are cut off
-                        // (bound generous by 0.1 % and a thousandth of a bin)
-                        const float rest = reach2 - 0.999f * gap2;
-                        if (rest < 0.f) {
-                            hi = lo - 1;
-                        } else if (rest < 1.0e37f) {
-                            const float span = sqrtf(rest) / bw * 1.001f + 1.001f;
-                            lo = max(lo, qb_last - (int)(span - tl_last));
-                            hi = min(hi, qb_last + (int)(span - tu_last));
-                        }
-                    } else {  // interior row: only the two end caps
-                        lo = second ? qb_last + d : qb_last - d;
-                        hi = lo;
-                        if (lo < 0 || lo >= nb_last) hi = lo - 1;
-                        const float g = ((float)(d - 1) + (second ? tu_last : tl_last)) * bw;
-                        if (0.999f * (gap2 + g * g) > reach2) hi = lo - 1;
-                    }
+                    // a whole run of the last dimension (rows on a face of the shell; the
+                    // second slot of such a row is unused), or one of the two end caps
+                    const float cap_gap = ((float)(d - 1) + (second ? tu_last : tl_last)) * bw;
+                    const float cap2 = gap2 + cap_gap * cap_gap;
+                    // bins of a run that are provably too far are cut off (bound
+                    // generous by 0.1 % and a thousandth of a bin)
+                    const float rest = fmaxf(reach2 - 0.999f * gap2, 0.f);
+                    const float span = rest < 1.0e37f ? __builtin_amdgcn_sqrtf(rest) * bins_per_unit + 1.001f : 3.0e9f;
+                    const int run_lo = max(qb_last - d, qb_last - (int)fminf(span - tl_last, 1.0e9f));
+                    const int run_hi = min(qb_last + d, qb_last + (int)fminf(span - tu_last, 1.0e9f));
+                    const int cap = second ? qb_last + d : qb_last - d;
+                    int lo = on_face ? run_lo : cap;
+                    int hi = on_face ? run_hi : cap;
+                    const bool too_far = on_face ? (second || 0.999f * gap2 > reach2) : 0.999f * cap2 > reach2;
                     lo = max(lo, 0);
                     hi = min(hi, nb_last - 1);
-                    if (inside && lo <= hi) {
+                    if (inside && !too_far && lo <= hi) {
                         const int first = event_base + cell * nb_last + lo;
                         const int last = event_base + cell * nb_last + hi + 1;
                         if (last < p.n_bboundaries) {
@@ -415,7 +424,9 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
                         uint64_t beats = __ballot(enters);
                         if (beats) {
                             if (S == 1 && __popcll(beats) >= kBulkInsertMin) {
-                                key[0] = merge_lowest_64(key[0], wave_sort_u64(enters ? ck : kEmptyKey));
+                                const uint64_t batch = wave_sort_u64(enters ? ck : kEmptyKey);
+                                // an empty list (its smallest key is the empty key) is replaced
+                                key[0] = readlane_u64(key[0], 0) == kEmptyKey ? batch : merge_lowest_64(key[0], batch);
                                 beats = 0;
                             }
                             while (beats) {
@@ -469,28 +480,28 @@ __global__ __launch_bounds__(256) void knn_wave_kernel(const KnnParams p) {
     }
 }
 
-template <int C, bool MAPPED>
+template <int C, int NB, bool MAPPED>
 int launch_levels(const KnnParams &p, hipStream_t s) {
     const int levels = std::max(1, ceil_div(p.K - 1, kWave));
     const dim3 grid(ceil_div(p.n_vert, 4)), block(256);
     switch (levels) {
-        case 1: knn_wave_kernel<C, 1, MAPPED><<<grid, block, 0, s>>>(p); break;
-        case 2: knn_wave_kernel<C, 2, MAPPED><<<grid, block, 0, s>>>(p); break;
+        case 1: knn_wave_kernel<C, NB, 1, MAPPED><<<grid, block, 0, s>>>(p); break;
+        case 2: knn_wave_kernel<C, NB, 2, MAPPED><<<grid, block, 0, s>>>(p); break;
         case 3:
-        case 4: knn_wave_kernel<C, 4, MAPPED><<<grid, block, 0, s>>>(p); break;
-        default: knn_wave_kernel<C, 8, MAPPED><<<grid, block, 0, s>>>(p); break;
+        case 4: knn_wave_kernel<C, NB, 4, MAPPED><<<grid, block, 0, s>>>(p); break;
+        default: knn_wave_kernel<C, NB, 8, MAPPED><<<grid, block, 0, s>>>(p); break;
     }
     return check_launch("knn_wave_kernel");
 }
 
+// The usual shapes (binned dimensions = min(3, coordinates)) get kernels with
+// both numbers fixed at compile time, anything else the one that reads them.
 template <bool MAPPED>
 int launch_coords(const KnnParams &p, hipStream_t s) {
-    switch (p.n_coords) {
-        case 2: return launch_levels<2, MAPPED>(p, s);
-        case 3: return launch_levels<3, MAPPED>(p, s);
-        case 4: return launch_levels<4, MAPPED>(p, s);
-        default: return launch_levels<0, MAPPED>(p, s);
-    }
+    if (p.n_coords == 2 && p.n_bin_dim == 2) return launch_levels<2, 2, MAPPED>(p, s);
+    if (p.n_coords == 3 && p.n_bin_dim == 3) return launch_levels<3, 3, MAPPED>(p, s);
+    if (p.n_coords == 4 && p.n_bin_dim == 3) return launch_levels<4, 3, MAPPED>(p, s);
+    return launch_levels<0, 0, MAPPED>(p, s);
 }
 
 }  // namespace
