@@ -168,6 +168,19 @@ def test_knn_neighbour_counts(oracle, K):
     run_knn_case(oracle, coords, rs, K, 7)
 
 
+@pytest.mark.parametrize("C,n_bins", [(3, 4), (4, 12), (2, 5)])
+def test_knn_dense_bins_long_candidate_lists(oracle, C, n_bins):
+    """thousands of points in a few bins: the candidate list of a batch of
+    segments is longer than what one pass over the segment marks covers, and
+    with many bins per dimension it is cut into many short segments"""
+    rng = np.random.default_rng(40 + C)
+    blob = (0.5 + 0.02 * rng.standard_normal((7000, C))).astype(np.float32)
+    spread = rng.random((1500, C), dtype=np.float32)
+    coords = np.concatenate([blob, spread])[rng.permutation(8500)]
+    rs = np.array([0, 8500], np.int32)
+    run_knn_case(oracle, coords, rs, 20, n_bins)
+
+
 def test_knn_small_events_direction_tf_compat(oracle):
     rng = np.random.default_rng(18)
     coords = rng.standard_normal((330, 3)).astype(np.float32)
