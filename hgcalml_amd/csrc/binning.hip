@@ -42,9 +42,14 @@ __global__ void iota_i32_kernel(int *p, int n) {
 // ---- grid parameters --------------------------------------------------------
 
 // stage 1: per-block column minima / maxima of the first n_dims columns
+// (also zeroes `clear[0, n_clear)` on the way, for callers that need a cleared table next)
 __global__ __launch_bounds__(256) void column_minmax_kernel(const float *__restrict__ coords, int stride,
                                                             int n_vert, int n_dims,
-                                                            float *__restrict__ partial /*[blocks][2][8]*/) {
+                                                            float *__restrict__ partial /*[blocks][2][8]*/,
+                                                            int *__restrict__ clear, long long n_clear) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n_clear;
+         i += (long long)gridDim.x * blockDim.x)
+        clear[i] = 0;
     float lo[kMaxBinDims], hi[kMaxBinDims];
 #pragma unroll
     for (int c = 0; c < kMaxBinDims; ++c) {
@@ -84,28 +89,11 @@ __global__ __launch_bounds__(256) void column_minmax_kernel(const float *__restr
     }
 }
 
-// stage 2: one wave folds the partials and derives shift / bin width / bin counts
-__global__ __launch_bounds__(64) void grid_params_kernel(const float *__restrict__ partial, int n_partial,
-                                                         int n_dims, int pre_normalized, int n_bins_scalar,
-                                                         const float *__restrict__ bin_width_in,
-                                                         float *__restrict__ shift, float *__restrict__ bin_width,
-                                                         int *__restrict__ n_bins) {
-    float lo[kMaxBinDims], hi[kMaxBinDims];
-#pragma unroll
-    for (int c = 0; c < kMaxBinDims; ++c) {
-        float a = FLT_MAX, b = -FLT_MAX;
-        for (int i = threadIdx.x; i < n_partial; i += kWave) {
-            a = fminf(a, partial[((size_t)i * 2 + 0) * kMaxBinDims + c]);
-            b = fmaxf(b, partial[((size_t)i * 2 + 1) * kMaxBinDims + c]);
-        }
-        for (int off = 32; off > 0; off >>= 1) {
-            a = fminf(a, __shfl_xor(a, off, kWave));
-            b = fmaxf(b, __shfl_xor(b, off, kWave));
-        }
-        lo[c] = a;
-        hi[c] = b;
-    }
-    if (threadIdx.x != 0) return;
+// shift, common bin width and bins per dimension from the column minima / maxima:
+// the fp32 operations of modules/bin_by_coordinates_op.py:50-65 in their order
+__device__ inline void derive_grid(const float *lo, const float *hi, int n_dims, int pre_normalized,
+                                   int n_bins_scalar, const float *bin_width_in, float *shift, float *bin_width,
+                                   int *n_bins) {
     float extent[kMaxBinDims];
     float bw = 0.f;
     for (int c = 0; c < n_dims; ++c) {
@@ -128,6 +116,31 @@ __global__ __launch_bounds__(64) void grid_params_kernel(const float *__restrict
         nb = nb + 1.f;
         n_bins[c] = (int)nb;
     }
+}
+
+// stage 2: one wave folds the partials and derives shift / bin width / bin counts
+__global__ __launch_bounds__(64) void grid_params_kernel(const float *__restrict__ partial, int n_partial,
+                                                         int n_dims, int pre_normalized, int n_bins_scalar,
+                                                         const float *__restrict__ bin_width_in,
+                                                         float *__restrict__ shift, float *__restrict__ bin_width,
+                                                         int *__restrict__ n_bins) {
+    float lo[kMaxBinDims], hi[kMaxBinDims];
+#pragma unroll
+    for (int c = 0; c < kMaxBinDims; ++c) {
+        float a = FLT_MAX, b = -FLT_MAX;
+        for (int i = threadIdx.x; i < n_partial; i += kWave) {
+            a = fminf(a, partial[((size_t)i * 2 + 0) * kMaxBinDims + c]);
+            b = fmaxf(b, partial[((size_t)i * 2 + 1) * kMaxBinDims + c]);
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            a = fminf(a, __shfl_xor(a, off, kWave));
+            b = fmaxf(b, __shfl_xor(b, off, kWave));
+        }
+        lo[c] = a;
+        hi[c] = b;
+    }
+    if (threadIdx.x != 0) return;
+    derive_grid(lo, hi, n_dims, pre_normalized, n_bins_scalar, bin_width_in, shift, bin_width, n_bins);
 }
 
 // ---- per-point assignment ---------------------------------------------------
@@ -211,6 +224,102 @@ __global__ __launch_bounds__(256) void index_replacer_kernel(const int *__restri
         out[i] = repl[v];
 }
 
+// ---- bin order in four launches (no order guarantee inside a bin) -------------
+//
+// For callers that only need the points grouped by bin: a counting sort whose
+// rank inside the bin is the order in which the points' atomic increments
+// arrive. The kernels below follow column_minmax_kernel (which also clears the
+// counters): every block folds the column minima / maxima and derives the grid
+// itself, so there is no separate launch for that.
+
+__global__ __launch_bounds__(256) void bin_points_ranked_kernel(
+    const float *__restrict__ coords, int stride, const float *__restrict__ partial, int n_partial,
+    const int *__restrict__ row_splits, int n_vert, int n_dims, int n_rs, int n_bins_scalar,
+    float *__restrict__ shift_out, float *__restrict__ bin_width_out, int *__restrict__ n_bins_out,
+    int *__restrict__ binass, int *__restrict__ flat, int *__restrict__ rank, int *__restrict__ counts,
+    int n_counts) {
+    __shared__ float s_lo[4][kMaxBinDims], s_hi[4][kMaxBinDims];
+    __shared__ float s_shift[kMaxBinDims], s_bw;
+    __shared__ int s_nb[kMaxBinDims];
+#pragma unroll
+    for (int c = 0; c < kMaxBinDims; ++c) {
+        float a = FLT_MAX, b = -FLT_MAX;
+        for (int i = threadIdx.x; i < n_partial; i += blockDim.x) {
+            a = fminf(a, partial[((size_t)i * 2 + 0) * kMaxBinDims + c]);
+            b = fmaxf(b, partial[((size_t)i * 2 + 1) * kMaxBinDims + c]);
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            a = fminf(a, __shfl_xor(a, off, kWave));
+            b = fmaxf(b, __shfl_xor(b, off, kWave));
+        }
+        if (lane_id() == 0) {
+            s_lo[threadIdx.x >> 6][c] = a;
+            s_hi[threadIdx.x >> 6][c] = b;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float lo[kMaxBinDims], hi[kMaxBinDims];
+        for (int c = 0; c < kMaxBinDims; ++c) {
+            lo[c] = fminf(fminf(s_lo[0][c], s_lo[1][c]), fminf(s_lo[2][c], s_lo[3][c]));
+            hi[c] = fmaxf(fmaxf(s_hi[0][c], s_hi[1][c]), fmaxf(s_hi[2][c], s_hi[3][c]));
+        }
+        derive_grid(lo, hi, n_dims, 0, n_bins_scalar, nullptr, s_shift, &s_bw, s_nb);
+        if (blockIdx.x == 0) {
+            for (int c = 0; c < n_dims; ++c) {
+                shift_out[c] = s_shift[c];
+                n_bins_out[c] = s_nb[c];
+            }
+            bin_width_out[0] = s_bw;
+        }
+    }
+    __syncthreads();
+    const float bw = s_bw;
+    for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < n_vert; p += gridDim.x * blockDim.x) {
+        int mul = 1, cell = 0;
+        for (int c = n_dims - 1; c >= 0; --c) {
+            const float x = coords[(size_t)p * stride + c] - s_shift[c];
+            int k = (int)(x / bw);
+            const int nb = s_nb[c];
+            if (k < 0 || k >= nb) k = 0;
+            binass[(size_t)p * (n_dims + 1) + c + 1] = k;
+            cell += k * mul;
+            mul *= nb;
+        }
+        int lo = 1, hi = n_rs;  // event: number of row splits (from the second on) that are <= p
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (row_splits[mid] > p)
+                hi = mid;
+            else
+                lo = mid + 1;
+        }
+        const int ev = lo - 1;
+        cell += ev * mul;
+        cell = min(cell, n_counts - 1);  // cannot happen for row splits that end at n_vert
+        binass[(size_t)p * (n_dims + 1)] = ev;
+        flat[p] = cell;
+        rank[p] = atomicAdd(&counts[cell], 1);
+    }
+}
+
+// every point's row of the inputs moves to its place in bin order
+__global__ __launch_bounds__(256) void scatter_to_bin_order_kernel(
+    const float *__restrict__ coords, const int *__restrict__ binass, const int *__restrict__ flat,
+    const int *__restrict__ rank, const int *__restrict__ direction, const int *__restrict__ boundaries, int n_vert,
+    int n_coords, int n_dims, int *__restrict__ sorting, float *__restrict__ scoords, int *__restrict__ sflat,
+    int *__restrict__ sbinass, int *__restrict__ sdir) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_vert) return;
+    const int cell = flat[p];
+    const int at = boundaries[cell] + rank[p];
+    sorting[at] = p;
+    sflat[at] = cell;
+    for (int c = 0; c < n_coords; ++c) scoords[(size_t)at * n_coords + c] = coords[(size_t)p * n_coords + c];
+    for (int c = 0; c <= n_dims; ++c) sbinass[(size_t)at * (n_dims + 1) + c] = binass[(size_t)p * (n_dims + 1) + c];
+    if (direction) sdir[at] = direction[p];
+}
+
 int key_bits(int n_total_bins) {
     int bits = 1;
     while (bits < 31 && (1ll << bits) < (long long)n_total_bins) ++bits;
@@ -224,6 +333,52 @@ int launch_fill_i32(int *p, int value, long long n, hipStream_t s) {
     int blocks = (int)std::min<long long>((n + 255) / 256, 4096);
     fill_i32_kernel<<<blocks, 256, 0, s>>>(p, value, n);
     return check_launch("fill_i32");
+}
+
+
+static int grouping_blocks(int n_vert) { return std::max(1, std::min(256, ceil_div(n_vert, 256))); }
+
+size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound) {
+    size_t temp = 0;
+    (void)rocprim::exclusive_scan(nullptr, temp, (const int *)nullptr, (int *)nullptr, 0,
+                                  (size_t)n_bins_bound + 1, rocprim::plus<int>(), (hipStream_t) nullptr);
+    const size_t n = std::max(n_vert, 1);
+    return align_up(temp) + align_up((size_t)grouping_blocks(n_vert) * 2 * kMaxBinDims * sizeof(float)) +
+           align_up(((size_t)n_bins_bound + 1) * sizeof(int)) + 2 * align_up(n * sizeof(int)) +
+           align_up(n * (kMaxBinDims + 1) * sizeof(int));
+}
+
+int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_direction, int n_vert, int n_coords,
+                 int n_bin_dims, int n_rs, int n_bins_scalar, int n_bins_bound, float *d_shift, float *d_bin_width,
+                 int *d_n_bins, int *d_boundaries, int *d_sorting, float *d_scoords, int *d_sflat, int *d_sbinass,
+                 int *d_sdir, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    if (!workspace || !aligned256(workspace) || workspace_bytes < bin_grouping_workspace_bytes(n_vert, n_bins_bound))
+        return fail(HGC_ERR_WORKSPACE, "bin grouping workspace missing, misaligned or too small");
+    const int blocks = grouping_blocks(n_vert);
+    Carver carve(workspace);
+    float *partial = carve.take<float>((size_t)blocks * 2 * kMaxBinDims);
+    int *counts = carve.take<int>((size_t)n_bins_bound + 1);
+    int *flat = carve.take<int>(n_vert);
+    int *rank = carve.take<int>(n_vert);
+    int *binass = carve.take<int>((size_t)n_vert * (kMaxBinDims + 1));
+    void *temp = carve.base + carve.used;
+    size_t temp_bytes = workspace_bytes - carve.used;
+    column_minmax_kernel<<<blocks, 256, 0, s>>>(d_coords, n_coords, n_vert, n_bin_dims, partial, counts,
+                                                (long long)n_bins_bound + 1);
+    int rc = check_launch("column_minmax");
+    if (rc) return rc;
+    bin_points_ranked_kernel<<<blocks, 256, 0, s>>>(d_coords, n_coords, partial, blocks, d_row_splits, n_vert,
+                                                    n_bin_dims, n_rs, n_bins_scalar, d_shift, d_bin_width, d_n_bins,
+                                                    binass, flat, rank, counts, n_bins_bound + 1);
+    rc = check_launch("bin_points_ranked");
+    if (rc) return rc;
+    // boundaries[b] = number of points in bins below b
+    HGC_HIP(rocprim::exclusive_scan(temp, temp_bytes, counts, d_boundaries, 0, (size_t)n_bins_bound + 1,
+                                    rocprim::plus<int>(), s));
+    scatter_to_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, binass, flat, rank, d_direction,
+                                                                      d_boundaries, n_vert, n_coords, n_bin_dims,
+                                                                      d_sorting, d_scoords, d_sflat, d_sbinass, d_sdir);
+    return check_launch("scatter_to_bin_order");
 }
 
 }  // namespace hgc
@@ -306,7 +461,7 @@ int hgc_bin_setup(const float *d_coords, int coord_stride, int n_vert, int n_bin
     hipStream_t s = as_stream(stream);
     const int blocks = setup_blocks(n_vert);
     float *partial = static_cast<float *>(workspace);
-    column_minmax_kernel<<<blocks, 256, 0, s>>>(d_coords, coord_stride, n_vert, n_bin_dims, partial);
+    column_minmax_kernel<<<blocks, 256, 0, s>>>(d_coords, coord_stride, n_vert, n_bin_dims, partial, nullptr, 0);
     int rc = check_launch("column_minmax");
     if (rc) return rc;
     grid_params_kernel<<<1, 64, 0, s>>>(partial, blocks, n_bin_dims, pre_normalized, n_bins_scalar, d_bin_width_in,

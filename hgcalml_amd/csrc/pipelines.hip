@@ -3,8 +3,8 @@
 // and one workspace instead of a dozen framework ops.
 //
 //   hgc_binned_select_knn_pipeline  modules/binned_select_knn_op.py:33-104
-//     (bounding box and grid, bin assignment, stable sort into bin order, gather
-//      of the sorted inputs, search, un-sort)
+//     (bounding box and grid, bin assignment, grouping by bin with the inputs
+//      moved along, search, un-sort)
 #include "hgc_common.hpp"
 
 #include <algorithm>
@@ -14,8 +14,7 @@ using namespace hgc;
 namespace {
 
 struct KnnPipelineLayout {
-    size_t shift, bin_width, n_bins, binass, flat, sorting, bounds, scoords, sflat, sbinass, sdir, setup_ws, sort_ws,
-        total;
+    size_t shift, bin_width, n_bins, sorting, bounds, scoords, sflat, sbinass, sdir, grouping_ws, total;
     int total_bins_bound;
 };
 
@@ -23,7 +22,7 @@ KnnPipelineLayout knn_layout(int n_vert, int n_coords, int n_bin_dims, int n_rs,
     KnnPipelineLayout L{};
     // every per-dimension bin count is at most n_bins_scalar + 1
     long long bound = n_rs - 1;
-    for (int i = 0; i < n_bin_dims; ++i) bound *= (n_bins_scalar + 1);
+    for (int i = 0; i < n_bin_dims; ++i) bound = std::min<long long>(bound * (n_bins_scalar + 1), 1ll << 40);
     L.total_bins_bound = (int)std::min<long long>(bound, (1ll << 31) - 2);
     const size_t n = std::max(n_vert, 1);
     size_t off = 0;
@@ -35,16 +34,13 @@ KnnPipelineLayout knn_layout(int n_vert, int n_coords, int n_bin_dims, int n_rs,
     L.shift = take(8 * sizeof(float));
     L.bin_width = take(sizeof(float));
     L.n_bins = take(8 * sizeof(int));
-    L.binass = take(n * (n_bin_dims + 1) * sizeof(int));
-    L.flat = take(n * sizeof(int));
     L.sorting = take(n * sizeof(int));
     L.bounds = take(((size_t)L.total_bins_bound + 1) * sizeof(int));
     L.scoords = take(n * n_coords * sizeof(float));
     L.sflat = take(n * sizeof(int));
     L.sbinass = take(n * (n_bin_dims + 1) * sizeof(int));
     L.sdir = take(use_direction ? n * sizeof(int) : 0);
-    L.setup_ws = take(hgc_bin_setup_workspace_bytes(n_vert, n_bin_dims));
-    L.sort_ws = take(hgc_sort_by_bin_workspace_bytes(n_vert, L.total_bins_bound));
+    L.grouping_ws = take(bin_grouping_workspace_bytes(n_vert, L.total_bins_bound));
     L.total = off;
     return L;
 }
@@ -74,15 +70,13 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
     HGC_REQUIRE(d_coords && d_row_splits && d_indices && d_dist, "null pointer");
     const int use_direction = d_direction != nullptr;
     const KnnPipelineLayout L = knn_layout(n_vert, n_coords, n_bin_dims, n_rs, n_bins_scalar, use_direction);
-    HGC_REQUIRE((long long)(n_rs - 1) * 1 <= L.total_bins_bound, "bin table overflows int32");
+    HGC_REQUIRE(L.total_bins_bound < (1ll << 31) - 2, "bin table overflows int32: fewer bins or events per call");
     if (!workspace || !aligned256(workspace) || workspace_bytes < L.total)
         return fail(HGC_ERR_WORKSPACE, "kNN pipeline workspace missing, misaligned or too small");
     char *ws = static_cast<char *>(workspace);
     float *shift = reinterpret_cast<float *>(ws + L.shift);
     float *bin_width = reinterpret_cast<float *>(ws + L.bin_width);
     int *n_bins = reinterpret_cast<int *>(ws + L.n_bins);
-    int *binass = reinterpret_cast<int *>(ws + L.binass);
-    int *flat = reinterpret_cast<int *>(ws + L.flat);
     int *sorting = d_out_sorting ? d_out_sorting : reinterpret_cast<int *>(ws + L.sorting);
     int *bounds = reinterpret_cast<int *>(ws + L.bounds);
     float *scoords = reinterpret_cast<float *>(ws + L.scoords);
@@ -90,24 +84,12 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
     int *sbinass = reinterpret_cast<int *>(ws + L.sbinass);
     int *sdir = use_direction ? reinterpret_cast<int *>(ws + L.sdir) : nullptr;
 
-    int rc = hgc_bin_setup(d_coords, n_coords, n_vert, n_bin_dims, 0, n_bins_scalar, nullptr, shift, bin_width, n_bins,
-                           ws + L.setup_ws, L.sort_ws - L.setup_ws, stream);
+    // The search needs the points grouped by bin, not a particular order inside a
+    // bin: its results are in the caller's index space and in canonical order.
+    const int rc = bin_grouping(d_coords, d_row_splits, d_direction, n_vert, n_coords, n_bin_dims, n_rs, n_bins_scalar,
+                                L.total_bins_bound, shift, bin_width, n_bins, bounds, sorting, scoords, sflat, sbinass,
+                                sdir, ws + L.grouping_ws, L.total - L.grouping_ws, as_stream(stream));
     if (rc) return rc;
-    rc = hgc_bin_by_coordinates_strided(d_coords, n_coords, shift, d_row_splits, bin_width, n_bins, binass, flat, nullptr,
-                                        nullptr, n_vert, n_bin_dims, n_rs, L.total_bins_bound, 0, stream);
-    if (rc) return rc;
-    rc = hgc_sort_by_bin(flat, n_vert, L.total_bins_bound, sorting, bounds, ws + L.sort_ws, L.total - L.sort_ws, stream);
-    if (rc) return rc;
-    rc = hgc_gather_rows(d_coords, sorting, scoords, n_vert, n_coords, stream);
-    if (rc) return rc;
-    rc = hgc_gather_rows(flat, sorting, sflat, n_vert, 1, stream);
-    if (rc) return rc;
-    rc = hgc_gather_rows(binass, sorting, sbinass, n_vert, n_bin_dims + 1, stream);
-    if (rc) return rc;
-    if (use_direction) {
-        rc = hgc_gather_rows(d_direction, sorting, sdir, n_vert, 1, stream);
-        if (rc) return rc;
-    }
     return hgc_binned_select_knn_fused(scoords, sflat, sdir, sbinass, bounds, n_bins, bin_width, sorting, shift, max_radius,
                                        d_indices, d_dist, n_vert, n_neigh, n_coords, n_bin_dims, L.total_bins_bound + 1,
                                        tf_compat, use_direction, stream);

@@ -164,8 +164,10 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
  * in the caller's order and index space: d_coords [n_vert, n_coords],
  * d_row_splits [n_rs], d_direction [n_vert] or NULL; d_indices, d_dist
  * [n_vert, n_neigh]. d_out_sorting (may be NULL) [n_vert] receives the bin
- * order of the points (original index of the i-th point in bin order), a
- * useful d_vertex_order for the accumulation. No host synchronisation. */
+ * order of the points (original index of the i-th point in bin order; the
+ * order inside a bin is unspecified and can differ from run to run, the
+ * neighbour results do not depend on it), a useful d_vertex_order for the
+ * accumulation. No host synchronisation. */
 size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, int n_rs,
                                                       int n_bins_scalar, int max_bin_dims,
                                                       int use_direction);
