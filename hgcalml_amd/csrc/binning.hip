@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void index_replacer_kernel(const int *__restri
         out[i] = repl[v];
 }
 
-// ---- bin order in four launches (no order guarantee inside a bin) -------------
+// ---- bin order in five launches (no order guarantee inside a bin) -------------
 //
 // For callers that only need the points grouped by bin: a counting sort whose
 // rank inside the bin is the order in which the points' atomic increments
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
     const int *__restrict__ row_splits, int n_vert, int n_dims, int n_rs, int n_bins_scalar,
     float *__restrict__ shift_out, float *__restrict__ bin_width_out, int *__restrict__ n_bins_out,
     int *__restrict__ binass, int *__restrict__ flat, int *__restrict__ rank, int *__restrict__ counts,
-    int n_counts) {
+    int n_bins_bound, int sub_shift) {
     __shared__ float s_lo[4][kMaxBinDims], s_hi[4][kMaxBinDims];
     __shared__ float s_shift[kMaxBinDims], s_bw;
     __shared__ int s_nb[kMaxBinDims];
@@ -296,25 +296,34 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
         }
         const int ev = lo - 1;
         cell += ev * mul;
-        cell = min(cell, n_counts - 1);  // cannot happen for row splits that end at n_vert
+        cell = min(cell, n_bins_bound - 1);  // no effect for row splits that end at n_vert
         binass[(size_t)p * (n_dims + 1)] = ev;
         flat[p] = cell;
-        rank[p] = atomicAdd(&counts[cell], 1);
+        // every bin has 2^sub_shift counters, a point takes the one its index names:
+        // the increments of a crowded bin queue up on several addresses instead of one
+        rank[p] = atomicAdd(&counts[((size_t)cell << sub_shift) | (p & ((1 << sub_shift) - 1))], 1);
     }
 }
 
-// every point's row of the inputs moves to its place in bin order
-__global__ __launch_bounds__(256) void scatter_to_bin_order_kernel(
-    const float *__restrict__ coords, const int *__restrict__ binass, const int *__restrict__ flat,
-    const int *__restrict__ rank, const int *__restrict__ direction, const int *__restrict__ boundaries, int n_vert,
-    int n_coords, int n_dims, int *__restrict__ sorting, float *__restrict__ scoords, int *__restrict__ sflat,
-    int *__restrict__ sbinass, int *__restrict__ sdir) {
+// position of every point in bin order
+__global__ __launch_bounds__(256) void place_in_bin_order_kernel(const int *__restrict__ flat,
+                                                                 const int *__restrict__ rank,
+                                                                 const int *__restrict__ boundaries, int n_vert,
+                                                                 int sub_shift, int *__restrict__ sorting) {
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
-    if (p >= n_vert) return;
-    const int cell = flat[p];
-    const int at = boundaries[cell] + rank[p];
-    sorting[at] = p;
-    sflat[at] = cell;
+    if (p < n_vert)
+        sorting[boundaries[((size_t)flat[p] << sub_shift) | (p & ((1 << sub_shift) - 1))] + rank[p]] = p;
+}
+
+// the inputs in bin order: row `at` of every output is row sorting[at] of its input
+__global__ __launch_bounds__(256) void gather_bin_order_kernel(
+    const float *__restrict__ coords, const int *__restrict__ binass, const int *__restrict__ flat,
+    const int *__restrict__ direction, const int *__restrict__ sorting, int n_vert, int n_coords, int n_dims,
+    float *__restrict__ scoords, int *__restrict__ sflat, int *__restrict__ sbinass, int *__restrict__ sdir) {
+    const int at = blockIdx.x * blockDim.x + threadIdx.x;
+    if (at >= n_vert) return;
+    const int p = sorting[at];
+    sflat[at] = flat[p];
     for (int c = 0; c < n_coords; ++c) scoords[(size_t)at * n_coords + c] = coords[(size_t)p * n_coords + c];
     for (int c = 0; c <= n_dims; ++c) sbinass[(size_t)at * (n_dims + 1) + c] = binass[(size_t)p * (n_dims + 1) + c];
     if (direction) sdir[at] = direction[p];
@@ -336,15 +345,27 @@ int launch_fill_i32(int *p, int value, long long n, hipStream_t s) {
 }
 
 
-static int grouping_blocks(int n_vert) { return std::max(1, std::min(256, ceil_div(n_vert, 256))); }
+// few blocks fold the bounding box (every binning block reads all their partial
+// results again), many assign the bins
+static int grouping_blocks(int n_vert) { return std::max(1, std::min(128, ceil_div(n_vert, 1024))); }
+
+int bin_grouping_sub_shift(int n_bins_bound) {
+    int shift = 0;
+    while (shift < 5 && (((size_t)n_bins_bound << (shift + 1)) + 1) <= ((size_t)1 << 20)) ++shift;
+    return shift;
+}
+
+static size_t grouping_counters(int n_bins_bound) {
+    return ((size_t)n_bins_bound << bin_grouping_sub_shift(n_bins_bound)) + 1;
+}
 
 size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound) {
     size_t temp = 0;
     (void)rocprim::exclusive_scan(nullptr, temp, (const int *)nullptr, (int *)nullptr, 0,
-                                  (size_t)n_bins_bound + 1, rocprim::plus<int>(), (hipStream_t) nullptr);
+                                  grouping_counters(n_bins_bound), rocprim::plus<int>(), (hipStream_t) nullptr);
     const size_t n = std::max(n_vert, 1);
     return align_up(temp) + align_up((size_t)grouping_blocks(n_vert) * 2 * kMaxBinDims * sizeof(float)) +
-           align_up(((size_t)n_bins_bound + 1) * sizeof(int)) + 2 * align_up(n * sizeof(int)) +
+           align_up(grouping_counters(n_bins_bound) * sizeof(int)) + 2 * align_up(n * sizeof(int)) +
            align_up(n * (kMaxBinDims + 1) * sizeof(int));
 }
 
@@ -357,28 +378,33 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
     const int blocks = grouping_blocks(n_vert);
     Carver carve(workspace);
     float *partial = carve.take<float>((size_t)blocks * 2 * kMaxBinDims);
-    int *counts = carve.take<int>((size_t)n_bins_bound + 1);
+    const int sub_shift = bin_grouping_sub_shift(n_bins_bound);
+    const size_t n_counters = grouping_counters(n_bins_bound);
+    int *counts = carve.take<int>(n_counters);
     int *flat = carve.take<int>(n_vert);
     int *rank = carve.take<int>(n_vert);
     int *binass = carve.take<int>((size_t)n_vert * (kMaxBinDims + 1));
     void *temp = carve.base + carve.used;
     size_t temp_bytes = workspace_bytes - carve.used;
     column_minmax_kernel<<<blocks, 256, 0, s>>>(d_coords, n_coords, n_vert, n_bin_dims, partial, counts,
-                                                (long long)n_bins_bound + 1);
+                                                (long long)n_counters);
     int rc = check_launch("column_minmax");
     if (rc) return rc;
-    bin_points_ranked_kernel<<<blocks, 256, 0, s>>>(d_coords, n_coords, partial, blocks, d_row_splits, n_vert,
+    bin_points_ranked_kernel<<<std::min(4096, ceil_div(n_vert, 256)), 256, 0, s>>>(d_coords, n_coords, partial, blocks, d_row_splits, n_vert,
                                                     n_bin_dims, n_rs, n_bins_scalar, d_shift, d_bin_width, d_n_bins,
-                                                    binass, flat, rank, counts, n_bins_bound + 1);
+                                                    binass, flat, rank, counts, n_bins_bound, sub_shift);
     rc = check_launch("bin_points_ranked");
     if (rc) return rc;
-    // boundaries[b] = number of points in bins below b
-    HGC_HIP(rocprim::exclusive_scan(temp, temp_bytes, counts, d_boundaries, 0, (size_t)n_bins_bound + 1,
-                                    rocprim::plus<int>(), s));
-    scatter_to_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, binass, flat, rank, d_direction,
-                                                                      d_boundaries, n_vert, n_coords, n_bin_dims,
-                                                                      d_sorting, d_scoords, d_sflat, d_sbinass, d_sdir);
-    return check_launch("scatter_to_bin_order");
+    // boundaries[b << sub_shift] = number of points in bins below b
+    HGC_HIP(rocprim::exclusive_scan(temp, temp_bytes, counts, d_boundaries, 0, n_counters, rocprim::plus<int>(), s));
+    place_in_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(flat, rank, d_boundaries, n_vert, sub_shift,
+                                                                    d_sorting);
+    rc = check_launch("place_in_bin_order");
+    if (rc) return rc;
+    gather_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, binass, flat, d_direction, d_sorting, n_vert,
+                                                                  n_coords, n_bin_dims, d_scoords, d_sflat, d_sbinass,
+                                                                  d_sdir);
+    return check_launch("gather_bin_order");
 }
 
 }  // namespace hgc

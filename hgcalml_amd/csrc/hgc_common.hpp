@@ -67,17 +67,27 @@ struct Carver {
 
 // ---- internal entry points shared between translation units -----------------
 
-// Groups the points by bin for the kNN search in four launches: grid from the
-// bounding box, bin of every point, bin boundary table and the inputs moved into
-// bin order (`d_sorting[i]` = original index of the i-th point). Unlike
+// Groups the points by bin for the kNN search in a handful of launches: grid from
+// the bounding box, bin of every point, bin boundary table and the inputs moved
+// into bin order (`d_sorting[i]` = original index of the i-th point). Unlike
 // hgc_sort_by_bin the order inside a bin is not specified (it can differ from
-// run to run). `n_bins_bound` bounds the number of bins of all events;
-// d_boundaries has n_bins_bound + 1 entries.
+// run to run). `n_bins_bound` bounds the number of bins of all events. The
+// boundary of bin b is d_boundaries[b << bin_grouping_sub_shift(n_bins_bound)];
+// the table has (n_bins_bound << shift) + 1 entries.
+int bin_grouping_sub_shift(int n_bins_bound);
 size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound);
 int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_direction, int n_vert, int n_coords,
                  int n_bin_dims, int n_rs, int n_bins_scalar, int n_bins_bound, float *d_shift, float *d_bin_width,
                  int *d_n_bins, int *d_boundaries, int *d_sorting, float *d_scoords, int *d_sflat, int *d_sbinass,
                  int *d_sdir, void *workspace, size_t workspace_bytes, hipStream_t s);
+
+// hgc_binned_select_knn_fused over a boundary table with stride 2^boundary_shift
+int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const int *d_direction,
+                              const int *d_dim_bin_idx, const int *d_bin_boundaries, int boundary_shift,
+                              const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
+                              const float *d_shift, float max_radius, int *d_indices, float *d_dist, int n_vert,
+                              int n_neigh, int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
+                              int use_direction, hipStream_t s);
 
 // ---- device helpers -------------------------------------------------------
 

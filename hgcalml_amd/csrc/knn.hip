@@ -48,6 +48,7 @@ struct KnnParams {
     float *out_dist;
     float radius_sq;  // < 0: no radius
     int n_vert, K, n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction;
+    int boundary_shift;  // the boundary of bin b sits at bin_boundaries[b << boundary_shift]
 };
 
 template <int C>
@@ -315,7 +316,8 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
         {
             const int own = p.bin_idx[q];
             if (reach_max > 0 && own + 1 < p.n_bboundaries)
-                with_own_bin = p.bin_boundaries[own + 1] - p.bin_boundaries[own] <= Kn;
+                with_own_bin = p.bin_boundaries[(size_t)(own + 1) << p.boundary_shift] -
+                                   p.bin_boundaries[(size_t)own << p.boundary_shift] <= Kn;
         }
         for (int d = with_own_bin ? 1 : 0; d <= reach_max; ++d) {
             const int W = 2 * d + 1;
@@ -387,8 +389,8 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                         const int first = event_base + cell * nb_last + lo;
                         const int last = event_base + cell * nb_last + hi + 1;
                         if (last < p.n_bboundaries) {
-                            seg_start = p.bin_boundaries[first];
-                            seg_len = p.bin_boundaries[last] - seg_start;
+                            seg_start = p.bin_boundaries[(size_t)first << p.boundary_shift];
+                            seg_len = p.bin_boundaries[(size_t)last << p.boundary_shift] - seg_start;
                         }
                     }
                 }
@@ -511,18 +513,13 @@ int launch_coords(const KnnParams &p, hipStream_t s) {
 }
 
 }  // namespace
-}  // namespace hgc
 
-using namespace hgc;
-
-extern "C" {
-
-int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, const int *d_direction,
-                                const int *d_dim_bin_idx, const int *d_bin_boundaries,
-                                const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
-                                const float *d_shift, float max_radius, int *d_indices, float *d_dist, int n_vert, int n_neigh,
-                                int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
-                                int use_direction, hgc_stream_t stream) {
+int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const int *d_direction,
+                              const int *d_dim_bin_idx, const int *d_bin_boundaries, int boundary_shift,
+                              const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
+                              const float *d_shift, float max_radius, int *d_indices, float *d_dist, int n_vert,
+                              int n_neigh, int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
+                              int use_direction, hipStream_t s) {
     // same conditions as the reference op (binned_select_knn_kernel.cc:336-352)
     HGC_REQUIRE(n_bin_dim > 1, "BinnedSelectKnnOp expects at least 2 binning dimensions.");
     HGC_REQUIRE(n_bin_dim < 6, "BinnedSelectKnnOp expects maximum 5 binning dimensions.");
@@ -532,6 +529,7 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
     HGC_REQUIRE(n_neigh >= 1 && n_neigh <= 8 * kWave + 1, "1 <= n_neighbours <= %d", 8 * kWave + 1);
     HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neighbours overflows int32");
     HGC_REQUIRE(n_bboundaries >= 2, "bin boundary table too short");
+    HGC_REQUIRE(boundary_shift >= 0 && boundary_shift < 8, "bad boundary stride");
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_coord && d_bin_idx && d_dim_bin_idx && d_bin_boundaries && d_n_bins && d_bin_width &&
                     d_indices && d_dist,
@@ -561,8 +559,25 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
     p.n_bboundaries = n_bboundaries;
     p.tf_compat = tf_compat;
     p.use_direction = use_direction;
-    hipStream_t s = as_stream(stream);
+    p.boundary_shift = boundary_shift;
     return d_sorting ? launch_coords<true>(p, s) : launch_coords<false>(p, s);
+}
+
+}  // namespace hgc
+
+using namespace hgc;
+
+extern "C" {
+
+int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, const int *d_direction,
+                                const int *d_dim_bin_idx, const int *d_bin_boundaries,
+                                const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
+                                const float *d_shift, float max_radius, int *d_indices, float *d_dist, int n_vert, int n_neigh,
+                                int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
+                                int use_direction, hgc_stream_t stream) {
+    return binned_select_knn_strided(d_coord, d_bin_idx, d_direction, d_dim_bin_idx, d_bin_boundaries, 0, d_n_bins,
+                                     d_bin_width, d_sorting, d_shift, max_radius, d_indices, d_dist, n_vert, n_neigh,
+                                     n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction, as_stream(stream));
 }
 
 int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int *d_direction,

@@ -35,7 +35,7 @@ KnnPipelineLayout knn_layout(int n_vert, int n_coords, int n_bin_dims, int n_rs,
     L.bin_width = take(sizeof(float));
     L.n_bins = take(8 * sizeof(int));
     L.sorting = take(n * sizeof(int));
-    L.bounds = take(((size_t)L.total_bins_bound + 1) * sizeof(int));
+    L.bounds = take((((size_t)L.total_bins_bound << bin_grouping_sub_shift(L.total_bins_bound)) + 1) * sizeof(int));
     L.scoords = take(n * n_coords * sizeof(float));
     L.sflat = take(n * sizeof(int));
     L.sbinass = take(n * (n_bin_dims + 1) * sizeof(int));
@@ -90,9 +90,10 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
                                 L.total_bins_bound, shift, bin_width, n_bins, bounds, sorting, scoords, sflat, sbinass,
                                 sdir, ws + L.grouping_ws, L.total - L.grouping_ws, as_stream(stream));
     if (rc) return rc;
-    return hgc_binned_select_knn_fused(scoords, sflat, sdir, sbinass, bounds, n_bins, bin_width, sorting, shift, max_radius,
-                                       d_indices, d_dist, n_vert, n_neigh, n_coords, n_bin_dims, L.total_bins_bound + 1,
-                                       tf_compat, use_direction, stream);
+    return binned_select_knn_strided(scoords, sflat, sdir, sbinass, bounds, bin_grouping_sub_shift(L.total_bins_bound),
+                                     n_bins, bin_width, sorting, shift, max_radius, d_indices, d_dist, n_vert, n_neigh,
+                                     n_coords, n_bin_dims, L.total_bins_bound + 1, tf_compat, use_direction,
+                                     as_stream(stream));
 }
 
 }  // extern "C"
