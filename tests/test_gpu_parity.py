@@ -640,6 +640,32 @@ def test_neighbour_covariance(oracle):
     assert np.abs(cov.cpu().numpy() - rcov).max() <= 1e-5 * np.abs(rcov).max()
 
 
+@pytest.mark.parametrize("case", ["clusters", "one_bin", "ragged"])
+def test_knn_pipeline_bin_order_groups_points_by_bin(oracle, case):
+    """the order the kNN pipeline hands out is a permutation of the points along
+    which the flat bin index (oracle binning, same grid) never decreases; the
+    order inside a bin is free"""
+    from hgcalml_amd import BinnedSelectKnn, ops
+    rng = np.random.default_rng(84)
+    if case == "clusters":
+        coords = workloads.cfg2(scale=0.05)["coords"]
+        rs = np.array([0, len(coords)], np.int32)
+        n_bins = 12
+    elif case == "one_bin":  # all points but two in one bin: every counter increment hits the same bin
+        coords = np.concatenate([0.5 + 1e-4 * rng.standard_normal((5000, 3)), [[0, 0, 0]], [[1, 1, 1]]]).astype(np.float32)
+        rs = np.array([0, len(coords)], np.int32)
+        n_bins = 9
+    else:
+        coords = rng.random((4000, 3), dtype=np.float32)
+        rs = np.array([0, 900, 900, 2500, 4000], np.int32)
+        n_bins = 6
+    idx, _ = run_knn_case(oracle, coords, rs, 8, n_bins, max_ties=len(coords))
+    order = ops.vertex_order_of(idx).cpu().numpy()
+    assert sorted(order.tolist()) == list(range(len(coords)))
+    _, flat, _, _ = oracle.BinByCoordinates(coords[:, :3], rs, n_bins=n_bins, calc_n_per_bin=False)
+    assert (np.diff(flat[order]) >= 0).all()
+
+
 def test_vertex_processing_order_changes_nothing(oracle):
     """the kNN hands its bin order to the accumulation as a processing order:
     same bits with it, without it and with an arbitrary permutation"""
