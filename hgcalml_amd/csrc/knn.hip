@@ -135,6 +135,15 @@ __device__ __forceinline__ void sorted_insert(uint64_t (&key)[S], uint64_t c) {
     }
 }
 
+// value of lane `src` (taken modulo 64); one LDS crossbar pass, no bounds logic
+__device__ __forceinline__ int from_lane_i32(int v, int src) { return __builtin_amdgcn_ds_bpermute(src << 2, v); }
+
+__device__ __forceinline__ uint64_t from_lane_u64(uint64_t v, int src) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(src << 2, (int)(uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
 // ---- bulk insert: sort a batch of 64 keys across the lanes and merge it into the list ----
 //
 // A compare-exchange step of the bitonic network between lanes i and i^J. Which
@@ -152,9 +161,7 @@ constexpr uint64_t keeps_min_mask(int k, int j) {
 template <int K, int J>
 __device__ __forceinline__ uint64_t compare_exchange(uint64_t key) {
     constexpr uint64_t kMin = keeps_min_mask(K, J);
-    const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)key, J, kWave);
-    const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(key >> 32), J, kWave);
-    const uint64_t other = ((uint64_t)hi << 32) | lo;
+    const uint64_t other = from_lane_u64(key, lane_id() ^ J);
     const uint64_t lt = __ballot(other < key);
     // the lane that keeps the smaller key swaps when the other one is smaller, its partner when not
     const bool swap = __builtin_amdgcn_inverse_ballot_w64(lt ^ ~kMin);
@@ -184,10 +191,7 @@ __device__ __forceinline__ uint64_t wave_sort_u64(uint64_t key) {
 // the 64 smallest of an ascending list and an ascending batch, ascending:
 // min(list[i], batch[63-i]) is a bitonic sequence, six more steps sort it
 __device__ __forceinline__ uint64_t merge_lowest_64(uint64_t list, uint64_t batch) {
-    const int mirror = (kWave - 1) - lane_id();
-    const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)batch, mirror, kWave);
-    const uint32_t hi = (uint32_t)__shfl((int)(uint32_t)(batch >> 32), mirror, kWave);
-    const uint64_t rev = ((uint64_t)hi << 32) | lo;
+    const uint64_t rev = from_lane_u64(batch, (kWave - 1) - lane_id());
     return bitonic_merge_steps<128>(rev < list ? rev : list);
 }
 
@@ -278,7 +282,8 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
         const int event_base = cells_per_event * (p.bin_idx[q] / cells_per_event);
         const int nb_last = nb[B - 1], qb_last = qb[B - 1];
         const float bw = p.bin_width[0];
-        const float bins_per_unit = 1.001f / bw;  // generous by 0.1 %, for the pruning bound only
+        const float inv_bw = 1.f / bw;
+        const float bins_per_unit = 1.001f * inv_bw;  // generous by 0.1 %, for the pruning bound only
 
         // Position of the query inside its own bin, in bin widths: to_lower[i] is a
         // lower bound of its distance to the bin's lower edge, to_upper[i] to the
@@ -290,7 +295,7 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
             to_lower[i] = 0.f;
             to_upper[i] = 0.f;
             if (i < B && p.shift) {
-                const float frac = (qrow[i] - p.shift[i]) / bw - (float)qb[i];
+                const float frac = (qrow[i] - p.shift[i]) * inv_bw - (float)qb[i];
                 if (frac >= 0.f && frac <= 1.f) {
                     to_lower[i] = fmaxf(frac - 1e-3f, 0.f);
                     to_upper[i] = fmaxf(1.f - frac - 1e-3f, 0.f);
@@ -417,7 +422,7 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                         uint32_t owner = wave_inclusive_max(marks[t + lane]);
                         owner = max(owner, owner_carry);
                         owner_carry = (uint32_t)readlane_i32((int)owner, kWave - 1);
-                        const int j = c + __shfl(seg_delta, (int)owner - 1, kWave);
+                        const int j = c + from_lane_i32(seg_delta, (int)owner - 1);
                         bool valid = c < total && j != q;
                         const int jj = valid ? j : q;
                         const uint32_t id = MAPPED ? (uint32_t)p.sorting[jj] : (uint32_t)jj;
