@@ -56,7 +56,9 @@ __device__ __forceinline__ float dist_sq(const float (&q)[C > 0 ? C : 1], const 
                                          int n_coords, const float *__restrict__ qrow) {
     float acc = 0.f;
     if constexpr (C > 0) {
-        const float *r = coord + (size_t)j * C;
+        // uniform base + 32-bit byte offset: the load takes its base from scalar registers
+        const float *r = reinterpret_cast<const float *>(reinterpret_cast<const char *>(coord) +
+                                                         (uint32_t)j * (uint32_t)(C * sizeof(float)));
         float x[C];
         if constexpr (C == 4) {
             const float4 v = *reinterpret_cast<const float4 *>(r);
@@ -109,7 +111,7 @@ __device__ __forceinline__ void sorted_insert(uint64_t (&key)[S], uint64_t c) {
     if constexpr (S == 1) {
         const uint64_t old = key[0];
         const bool larger = old > c;
-        const uint64_t run = __ballot(larger);  // contiguous upper lanes, the list is sorted
+        const uint64_t run = __builtin_amdgcn_ballot_w64(larger);  // contiguous upper lanes, the list is sorted
         if (run) {
             if (larger) key[0] = wave_shift_up1_zero(old);
             key[0] = writelane_u64(c, __ffsll((long long)run) - 1, key[0]);
@@ -122,7 +124,7 @@ __device__ __forceinline__ void sorted_insert(uint64_t (&key)[S], uint64_t c) {
             const uint64_t old = key[s];
             const uint64_t last = readlane_u64(old, kWave - 1);
             const bool larger = placed || old > c;
-            const uint64_t run = __ballot(larger);
+            const uint64_t run = __builtin_amdgcn_ballot_w64(larger);
             if (run) {
                 if (larger) key[s] = wave_shift_up1_u64(old, carry);
                 if (!placed) {
@@ -162,7 +164,7 @@ template <int K, int J>
 __device__ __forceinline__ uint64_t compare_exchange(uint64_t key) {
     constexpr uint64_t kMin = keeps_min_mask(K, J);
     const uint64_t other = from_lane_u64(key, lane_id() ^ J);
-    const uint64_t lt = __ballot(other < key);
+    const uint64_t lt = __builtin_amdgcn_ballot_w64(other < key);
     // the lane that keeps the smaller key swaps when the other one is smaller, its partner when not
     const bool swap = __builtin_amdgcn_inverse_ballot_w64(lt ^ ~kMin);
     return swap ? other : key;
@@ -312,6 +314,9 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
         // ranks. Then the K-th key is re-read once per batch instead of per insert.
         const bool spare_rank = S * kWave > Kn;
         uint64_t thr = kEmptyKey;  // current K-th key: candidates at or above it cannot enter
+        // first key beyond the radius: d² <= r² <=> key < (bits(r²) + 1) << 32 for the non-negative r²
+        const uint64_t radius_limit = has_radius ? (uint64_t)(__float_as_uint(p.radius_sq) + 1u) << 32 : kEmptyKey;
+        uint64_t cut = radius_limit;  // min(thr, radius_limit): what a candidate's key has to stay below
 
         // Shell 0 (the query's own bin) never ends the search. When it cannot fill
         // the list either (so that it cannot prune shell 1), it is walked together
@@ -402,7 +407,10 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                 const int seg_end_off = wave_inclusive_sum(seg_len);
                 const int seg_off = seg_end_off - seg_len;
                 const int total = readlane_i32(seg_end_off, kWave - 1);
-                const int seg_delta = seg_start - seg_off;  // candidate position -> point index, for the owner
+                // candidate position -> point index for the owning segment; kept one lane up,
+                // so that the mark (lane number + 1) is the lane to read it from
+                // (DPP wave_ror:1; lane 63's value goes to lane 0, which is where mark 64 reads)
+                const int seg_delta = __builtin_amdgcn_update_dpp(0, seg_start - seg_off, 0x13c, 0xf, 0xf, false);
 
                 // ---- walk the concatenated candidates, 64 per step ----
                 // Every non-empty segment marks its first position of the list with its
@@ -422,21 +430,25 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                         uint32_t owner = wave_inclusive_max(marks[t + lane]);
                         owner = max(owner, owner_carry);
                         owner_carry = (uint32_t)readlane_i32((int)owner, kWave - 1);
-                        const int j = c + from_lane_i32(seg_delta, (int)owner - 1);
-                        bool valid = c < total && j != q;
-                        const int jj = valid ? j : q;
-                        const uint32_t id = MAPPED ? (uint32_t)p.sorting[jj] : (uint32_t)jj;
+                        const int j = c + from_lane_i32(seg_delta, (int)owner);
+                        // lane masks are combined as integers on the scalar side
+                        const bool in_list = c < total;
+                        uint64_t valid = __builtin_amdgcn_ballot_w64(in_list) & __builtin_amdgcn_ballot_w64(j != q);
+                        const int jj = in_list ? j : q;
+                        const uint32_t id = MAPPED ? *reinterpret_cast<const uint32_t *>(
+                                                         reinterpret_cast<const char *>(p.sorting) + ((uint32_t)jj << 2))
+                                                   : (uint32_t)jj;
                         const float dsq = dist_sq<C>(qc, p.coord, jj, p.n_coords, qrow);
-                        if (p.use_direction && valid) {
+                        if (p.use_direction) {
                             const int dj = p.direction[jj];
-                            if (dj == 1 || dj == 2) valid = false;  // may not be a neighbour
+                            valid &= ~__builtin_amdgcn_ballot_w64(dj == 1 || dj == 2);  // may not be a neighbour
                         }
-                        valid = valid && (!has_radius || dsq <= p.radius_sq);
                         const uint64_t ck = ((uint64_t)__float_as_uint(dsq) << 32) | id;
-                        const bool enters = valid && ck < thr;
-                        uint64_t beats = __ballot(enters);
+                        // below the K-th key and (keys compare like distances) within the radius
+                        uint64_t beats = valid & __builtin_amdgcn_ballot_w64(ck < cut);
                         if (beats) {
-                            if (S == 1 && __popcll(beats) >= kBulkInsertMin) {
+                            if (S == 1 && (int)__popcll(beats) >= kBulkInsertMin) {
+                                const bool enters = __builtin_amdgcn_inverse_ballot_w64(beats);
                                 const uint64_t batch = wave_sort_u64(enters ? ck : kEmptyKey);
                                 // an empty list (its smallest key is the empty key) is replaced
                                 key[0] = readlane_u64(key[0], 0) == kEmptyKey ? batch : merge_lowest_64(key[0], batch);
@@ -459,6 +471,8 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
 #pragma unroll
                             for (int s = 0; s < S; ++s)
                                 if (s == kth_level) thr = readlane_u64(key[s], kth_lane);
+                            // the low word of radius_limit is 0: the high words decide
+                            cut = (uint32_t)(thr >> 32) < (uint32_t)(radius_limit >> 32) ? thr : radius_limit;
                         }
                     }
                 }
