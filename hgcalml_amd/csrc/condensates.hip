@@ -120,8 +120,14 @@ struct TakenFlags {
 
 constexpr int kHitsPerThread = 4;
 
-template <bool LDS_FLAGS>
-__global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondParams p, int flag_words) {
+// LDS_FLAGS: claimed flags of the high-beta hits in LDS. ASSIGNED_BITS (max-beta
+// mode only, where an assigned hit is never looked at again): one bit per hit of
+// the event in LDS says whether it is assigned, so that the claim step loads
+// coordinates and masks of unassigned hits only; most hits of a box belong to
+// earlier condensates, and one CU's load bandwidth is what the step waits for.
+template <bool LDS_FLAGS, bool ASSIGNED_BITS>
+__global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondParams p, int flag_words,
+                                                                  int assigned_words) {
     extern __shared__ uint32_t s_bits[];
     __shared__ int s_first[kWavesPerBlock];
     __shared__ int s_pick, s_alpha;
@@ -144,6 +150,9 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
     }
     if (LDS_FLAGS)
         for (int i = tid; i < flag_words; i += kBlock) s_bits[i] = 0;
+    uint32_t *const s_assigned = s_bits + flag_words;
+    if (ASSIGNED_BITS)
+        for (int i = tid; i < assigned_words; i += kBlock) s_assigned[i] = 0;
     for (int i = first + tid; i < last; i += kBlock) {
         p.assignment[i] = -1;
         p.association[i] = -1;
@@ -308,12 +317,24 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
                     }
                     hit[k] = live[k] ? s_row_start[lo_r] + (h - s_row_off[lo_r]) : first;
                 }
+                if (ASSIGNED_BITS) {
+#pragma unroll
+                    for (int k = 0; k < kHitsPerThread; ++k) {
+                        const int local = hit[k] - first;
+                        live[k] = live[k] && !((s_assigned[local >> 5] >> (local & 31)) & 1u);
+                    }
+                }
                 int asg[kHitsPerThread], filt[kHitsPerThread], msk[kHitsPerThread];
                 float dsq[kHitsPerThread];
 #pragma unroll
                 for (int k = 0; k < kHitsPerThread; ++k) {
                     const int i = hit[k];
-                    asg[k] = p.assignment[i];
+                    asg[k] = -1;
+                    filt[k] = -1;
+                    msk[k] = 1;
+                    dsq[k] = 0.f;
+                    if (ASSIGNED_BITS && !live[k]) continue;
+                    if (!ASSIGNED_BITS && p.by_max_beta) asg[k] = p.assignment[i];
                     filt[k] = p.to_filtered[i];
                     msk[k] = p.mask[i];
                     float acc = 0.f;
@@ -337,6 +358,7 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
                     }
                     p.assignment[i] = shower;
                     p.association[i] = shower_orig;
+                    if (ASSIGNED_BITS) atomicOr(&s_assigned[(i - first) >> 5], 1u << ((i - first) & 31));
                     if (filt[k] != -1) taken.set(filt[k] - first_h);
                 }
             }
@@ -467,13 +489,22 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int
         p.n_vert_h = n_vert_h;
         p.order_h = order;
         p.event_count = event_count;
-        // one claimed-flag bit per high-beta hit of an event lives in LDS when it fits
-        // (n_vert_h bounds every event); 48 KB = 393k hits
+        // One claimed-flag bit per high-beta hit of an event and, in max-beta mode, one
+        // assigned bit per hit live in LDS when they fit (n_vert_h and n_vert bound
+        // every event; the event sizes themselves are device data).
         const int flag_words = ceil_div(std::max(n_vert_h, 1), 32);
-        if ((size_t)flag_words * 4 <= 48 * 1024)
-            condensate_event_kernel<true><<<num_rows, kBlock, (size_t)flag_words * 4, s>>>(p, flag_words);
-        else
-            condensate_event_kernel<false><<<num_rows, kBlock, 0, s>>>(p, 0);
+        const int assigned_words = ceil_div(std::max(n_vert, 1), 32);
+        constexpr size_t kDynamicLdsLimit = 144 * 1024;  // of 160 KB; the kernel has ~9 KB of static tables
+        const size_t flag_bytes = (size_t)flag_words * 4, both_bytes = flag_bytes + (size_t)assigned_words * 4;
+        if (assign_by_max_beta && both_bytes <= kDynamicLdsLimit) {
+            HGC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&condensate_event_kernel<true, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamicLdsLimit));
+            condensate_event_kernel<true, true><<<num_rows, kBlock, both_bytes, s>>>(p, flag_words, assigned_words);
+        } else if (flag_bytes <= 48 * 1024) {
+            condensate_event_kernel<true, false><<<num_rows, kBlock, flag_bytes, s>>>(p, flag_words, 0);
+        } else {
+            condensate_event_kernel<false, false><<<num_rows, kBlock, 0, s>>>(p, 0, 0);
+        }
         int rc = check_launch("condensate_event_kernel");
         if (rc) return rc;
     }
