@@ -801,6 +801,16 @@ def test_condensates_cfg5_full(oracle, by_max_beta):
 
 
 @pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensates_more_hits_than_the_lds_flags_hold(oracle, by_max_beta):
+    """1.3 M hits with ~0.9 M above the beta threshold: neither the assigned bits nor
+    the claimed flags fit into LDS, the kernel keeps its flags in global memory"""
+    cfg = workloads.cfg5(scale=5.2, n_events=4)
+    cfg["beta_threshold"] = 0.02
+    assert (cfg["betas"] > 0.02).sum() > 48 * 1024 * 8
+    run_condensates(oracle, cfg, by_max_beta)
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
 def test_condensates_per_hit_radii_and_ties(oracle, by_max_beta):
     cfg = workloads.cfg5(scale=0.05, n_events=5)
     rng = np.random.default_rng(24)
