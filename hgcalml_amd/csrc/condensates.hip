@@ -130,7 +130,8 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
                                                                   int assigned_words) {
     extern __shared__ uint32_t s_bits[];
     __shared__ int s_first[kWavesPerBlock];
-    __shared__ int s_pick, s_alpha;
+    __shared__ int s_pick, s_alpha, s_alpha_mask, s_alpha_orig;
+    __shared__ float s_alpha_centre[kMaxDims], s_alpha_dist;
     __shared__ int s_row_off[kBlock + 1];
     __shared__ int s_row_start[kBlock];
     __shared__ int s_wave_tot[kWavesPerBlock];
@@ -176,6 +177,12 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
     int window = -1;       // start of the 1024 order entries cached in registers
     int my_q = -1;
     bool my_selectable = false;
+    // what a claim step needs of this thread's entry, fetched with the window so that
+    // the step does not wait for a load that depends on the pick
+    float my_centre[kMaxDims], my_dist = 0.f;
+    int my_mask = 0, my_orig = -1;
+#pragma unroll
+    for (int c = 0; c < kMaxDims; ++c) my_centre[c] = 0.f;
     int shower = 0;
     while (cursor < last_h) {
         // ---- next unclaimed hit in selection order ----
@@ -184,6 +191,14 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
             const int pos = window + tid;
             my_q = pos < last_h ? p.order_h[pos] : -1;
             my_selectable = my_q >= 0 && (always_first(p.mask_h, p.n_vert_h, my_q) || p.beta_h[my_q] > -1.f);
+            if (my_q >= 0) {
+#pragma unroll
+                for (int c = 0; c < kMaxDims; ++c)
+                    if (c < C) my_centre[c] = p.ccoords_h[(size_t)my_q * C + c];
+                my_dist = p.dist_h[my_q];
+                my_mask = p.mask_h[my_q];
+                my_orig = p.orig_h[my_q];
+            }
         }
         const bool open = my_selectable && window + tid >= cursor && !taken.test(my_q - first_h);
         const uint64_t b = __ballot(open);
@@ -201,7 +216,14 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
             __syncthreads();
             continue;
         }
-        if (tid == pick) s_alpha = my_q;
+        if (tid == pick) {
+            s_alpha = my_q;
+            s_alpha_dist = my_dist;
+            s_alpha_mask = my_mask;
+            s_alpha_orig = my_orig;
+#pragma unroll
+            for (int c = 0; c < kMaxDims; ++c) s_alpha_centre[c] = my_centre[c];
+        }
         __syncthreads();
         cursor = window + pick;
         const int alpha = s_alpha;
@@ -209,10 +231,10 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         // ---- claim step ----
         float centre[kMaxDims];
 #pragma unroll
-        for (int c = 0; c < kMaxDims; ++c) centre[c] = c < C ? p.ccoords_h[(size_t)alpha * C + c] : 0.f;
-        float radius = p.dist_h[alpha];
+        for (int c = 0; c < kMaxDims; ++c) centre[c] = s_alpha_centre[c];
+        float radius = s_alpha_dist;
         const float radius_sq = radius * radius;
-        const bool solitary = p.mask_h[alpha] > 0;
+        const bool solitary = s_alpha_mask > 0;
         if (solitary) radius = 0.f;
         const float reach_sq = radius * radius * 1.0001f;  // pruning bound, slightly generous
 
@@ -236,7 +258,7 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
             }
         }
         const int run_lo = lo_bin[B - 1], run_hi = lo_bin[B - 1] + width[B - 1] - 1;
-        const int shower_orig = p.orig_h[alpha];
+        const int shower_orig = s_alpha_orig;
 
         for (int row0 = 0; row0 < n_rows; row0 += kBlock) {
             // -- every thread resolves one row of the box into a run of hits --
