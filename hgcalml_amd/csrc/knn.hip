@@ -7,11 +7,14 @@
 //   modules/compiled/select_knn_kernel.cc:158,244-245   (radius rule)
 //
 // Design (gfx950, wave64):
-//   * Points arrive sorted by bin, so the bins of one row of the grid (last
+//   * Points arrive grouped by bin, so the bins of one row of the grid (last
 //     binned dimension running) are one contiguous range of points. A shell of
 //     half-width d is cut into such ranges ("segments"); the 64 lanes look up 64
-//     segments at once, prefix-sum their lengths, and the wave then walks the
-//     concatenated candidate list 64 points per step, fully coalesced.
+//     segments at once (cutting each against the current K-th distance) and
+//     prefix-sum their lengths. Every non-empty segment marks the position of
+//     its first candidate in a strip of LDS; the wave then walks the
+//     concatenated candidate list 64 points per step, fully coalesced, and finds
+//     the segment of a position as the prefix maximum of the marks.
 //   * Each lane evaluates one candidate: serial fp32 sum of squared coordinate
 //     differences in coordinate order (no FMA contraction), packed with the
 //     candidate's index into a 64-bit key (distance bits high, index low), so a
@@ -25,7 +28,8 @@
 //     list in one go instead.
 //   * The shell loop stops exactly as the reference does: list full and
 //     ((bw*d)*bw)*d > K-th distance, or no bin of the shell inside the grid.
-//   * No LDS, no atomics, no barriers; every wave exits on its own.
+//   * The kernel is bound by vector ALU issue; LDS holds only the marks. No
+//     atomics, no barriers; every wave is its own workgroup and exits on its own.
 #include "hgc_common.hpp"
 
 namespace hgc {
