@@ -27,11 +27,12 @@
 namespace hgc {
 
 int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
-// accumulate_grad_fused.hip; returns 1 when the shape is not covered
+// accumulate_grad_fused.hip; returns 1 when the shape is not covered. gw == nullptr:
+// feature gradient only (feat and idx are then not read).
 int launch_accumulate_grad_fused(const float *g, const float *w, const float *feat, const int *maxidx,
                                  const unsigned char *maxslot, const int *inv_off, const int *inv_slots, float *gw,
                                  float *gfeat, int n_vert, int K, int F, int g_cols, bool mean_and_max, const int *idx,
-                                 const int *order, hipStream_t s);
+                                 const int *order, float divisor, hipStream_t s);
 
 namespace {
 
@@ -834,11 +835,12 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
     if (n_feat >= kWave && fits_32bit) {  // one wave per vertex, rows addressed through 32-bit buffer offsets
         const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
         // both gradients from one gather pass where that kernel covers the shape
-        if (want_w && want_f && divisor == (float)n_neigh) {
+        // (or the mean-only feature gradient alone: the gather without the dot products)
+        if (want_f && (want_w || !mean_and_max)) {
             const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
                                                         d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
                                                         d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat,
-                                                        mean_and_max != 0, d_neigh_indices, d_order, s);
+                                                        mean_and_max != 0, d_neigh_indices, d_order, divisor, s);
             if (rc <= 0) return rc;  // 1: shape not covered, use the two-kernel path
         }
         const int vec = wave_vec(n_feat, align_or);

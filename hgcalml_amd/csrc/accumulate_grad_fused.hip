@@ -112,7 +112,7 @@ constexpr uint32_t kOutOfRange = 0xfffffff0u;
 // subnormal), and the max part is formed as (hit ? g_max : 0) * w, whose zero
 // may carry the weight's sign, which cannot change a sum that started at +0
 // (it would differ for an infinite weight only).
-template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool FAST>
+template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool FAST, bool WGRAD>
 __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix &MI, __amdgpu_buffer_rsrc_t MS,
                                            const uint32_t (&lane_bytes)[NB], uint32_t max_col_bytes, int c, int cnt,
                                            uint64_t repmask, int self_key, int m, uint32_t offkey_v, float w_v,
@@ -181,11 +181,11 @@ __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix 
                     const float g = gm[u][b][e];
                     const float part = POW2K ? g * swk[u] : (g / kf) * sw[u];
                     // weight gradient of slot (v, n): partial dot products with the wave's own row
-                    val[h + u] = __builtin_fmaf(g, xk[b][e], val[h + u]);
+                    if (WGRAD) val[h + u] = __builtin_fmaf(g, xk[b][e], val[h + u]);
                     if (MAX) {
                         // a lane with one hit among its VEC features has loaded all of them
                         const float gsel = (VEC == 1 || hit[u][b][e]) ? gx[u][b][e] : 0.f;
-                        val[h + u] = __builtin_fmaf(gsel, xo[b][e], val[h + u]);
+                        if (WGRAD) val[h + u] = __builtin_fmaf(gsel, xo[b][e], val[h + u]);
                         // repeated self references carry the max part once, at the first self slot
                         const float part_max = (!FAST && rep[u]) ? 0.f : gsel * sw[u];
                         const float add = part + part_max;
@@ -201,16 +201,17 @@ __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix 
     }
 }
 
-template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS>
+// WGRAD false: feature gradient only (feat, idx and gw are not touched); kf is
+// what the mean part is divided by (K for the accumulation, 1 for a plain push).
+template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool WGRAD>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) void accumulate_grad_fused_kernel(
     const float *__restrict__ g, const float *__restrict__ w, const float *__restrict__ feat,
     const int *__restrict__ maxidx, const unsigned char *__restrict__ maxslot, const int *__restrict__ inv_off,
     const int *__restrict__ inv_slots, float *__restrict__ gw, float *__restrict__ gfeat, int n_vert, int K, int F,
-    int g_cols, const FastDiv div_k, const int *__restrict__ idx, const int *__restrict__ order) {
+    int g_cols, const FastDiv div_k, const int *__restrict__ idx, const int *__restrict__ order, const float kf) {
     const int m = wave_vertex(order, n_vert);
     if (m >= n_vert) return;
     const int lane = lane_id();
-    const float kf = (float)K;
     const float inv_kf = 1.f / kf;  // exact when K is a power of two
     const double inv_kd = 1.0 / (double)kf;
     const int begin = inv_off[m], end = inv_off[m + 1];
@@ -227,7 +228,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
     for (int b = 0; b < NB; ++b) {
         const int fb = (b * kWave + lane) * VEC;
         lane_bytes[b] = (uint32_t)fb * 4u;
-        load_vec<VEC>(feat + (size_t)m * F + fb, xo[b]);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) xo[b][e] = 0.f;
+        if (WGRAD) load_vec<VEC>(feat + (size_t)m * F + fb, xo[b]);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) xk[b][e] = (float)((double)xo[b][e] * inv_kd);
 #pragma unroll
@@ -237,7 +240,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
     // first slot of the target's own row that names the target itself (-1: none);
     // later entries naming it are repeated self references
     int self_key = -1;
-    for (int n0 = 0; n0 < K && self_key < 0; n0 += kWave) {
+    for (int n0 = 0; MAX && n0 < K && self_key < 0; n0 += kWave) {
         const int n = n0 + lane;
         const uint64_t is_self = __ballot(n < K && idx[(size_t)m * K + min(n, K - 1)] == m);
         if (is_self != 0) self_key = n0 + __ffsll((unsigned long long)is_self) - 1;
@@ -252,22 +255,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
         // row offset of the entry's vertex, with the entry's slot in its low bits
         const uint32_t offkey_v = (uint32_t)v * g_row_bytes | ((MAX && SLOTS) ? (uint32_t)key_v : 0u);
         const float wk_v = w_v * inv_kf;
-        const uint64_t repmask = __ballot(v == m && key_v != self_key && lane < cnt);
+        const uint64_t repmask = MAX ? __ballot(v == m && key_v != self_key && lane < cnt) : 0ull;
         for (int c = 0; c < cnt; c += kGroup) {
             float val[kGroup];
 #pragma unroll
             for (int i = 0; i < kGroup; ++i) val[i] = 0.f;
             const bool fast = (c + kGroup <= cnt) && ((repmask >> c) & ((1ull << kGroup) - 1)) == 0;
             if (fast)
-                grad_group<VEC, NB, MAX, POW2K, SLOTS, true>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
-                                                             self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
+                grad_group<VEC, NB, MAX, POW2K, SLOTS, true, WGRAD>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
+                                                                    self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
             else
-                grad_group<VEC, NB, MAX, POW2K, SLOTS, false>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
-                                                              self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
-            const float r = transpose_reduce_16(val);  // lane L: entry c + (L & 15)
-            const int dst = __shfl(slot_v, c + (lane & (kGroup - 1)), kWave);
-            if (lane < kGroup && c + lane < cnt) {
-                gw[dst] = r;
+                grad_group<VEC, NB, MAX, POW2K, SLOTS, false, WGRAD>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
+                                                                     self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
+            if (WGRAD) {
+                const float r = transpose_reduce_16(val);  // lane L: entry c + (L & 15)
+                const int dst = __shfl(slot_v, c + (lane & (kGroup - 1)), kWave);
+                if (lane < kGroup && c + lane < cnt) gw[dst] = r;
             }
         }
     }
@@ -289,18 +292,19 @@ __global__ __launch_bounds__(256) void zero_padded_weight_grad_kernel(const int 
 template <int VEC, int NB>
 int launch_fused(const float *g, const float *w, const float *feat, const int *maxidx, const unsigned char *maxslot,
                  const int *inv_off, const int *inv_slots, float *gw, float *gfeat, int n_vert, int K, int F, int g_cols,
-                 bool mean_and_max, const int *idx, const int *order, hipStream_t s) {
+                 bool mean_and_max, const int *idx, const int *order, float divisor, bool want_w, hipStream_t s) {
     const dim3 grid(ceil_div(n_vert, 4)), block(256);
     const FastDiv div_k = make_fast_div(K);
-    const bool pow2k = is_pow2(K);
+    const bool pow2k = divisor == (float)(int)divisor && is_pow2((int)divisor);
     const bool slots = mean_and_max && maxslot != nullptr;
-#define HGC_FUSED(MAX, P2, SL)                                                                                      \
-    accumulate_grad_fused_kernel<VEC, NB, MAX, P2, SL><<<grid, block, 0, s>>>(g, w, feat, maxidx, maxslot, inv_off, \
-                                                                              inv_slots, gw, gfeat, n_vert, K, F,    \
-                                                                              g_cols, div_k, idx, order)
-    if (mean_and_max && slots) { if (pow2k) HGC_FUSED(true, true, true); else HGC_FUSED(true, false, true); }
-    else if (mean_and_max) { if (pow2k) HGC_FUSED(true, true, false); else HGC_FUSED(true, false, false); }
-    else { if (pow2k) HGC_FUSED(false, true, false); else HGC_FUSED(false, false, false); }
+#define HGC_FUSED(MAX, P2, SL, WG)                                                                                       \
+    accumulate_grad_fused_kernel<VEC, NB, MAX, P2, SL, WG><<<grid, block, 0, s>>>(g, w, feat, maxidx, maxslot, inv_off, \
+                                                                                  inv_slots, gw, gfeat, n_vert, K, F,    \
+                                                                                  g_cols, div_k, idx, order, divisor)
+    if (!want_w) { if (pow2k) HGC_FUSED(false, true, false, false); else HGC_FUSED(false, false, false, false); }
+    else if (mean_and_max && slots) { if (pow2k) HGC_FUSED(true, true, true, true); else HGC_FUSED(true, false, true, true); }
+    else if (mean_and_max) { if (pow2k) HGC_FUSED(true, true, false, true); else HGC_FUSED(true, false, false, true); }
+    else { if (pow2k) HGC_FUSED(false, true, false, true); else HGC_FUSED(false, false, false, true); }
 #undef HGC_FUSED
     return check_launch("accumulate_grad_fused_kernel");
 }
@@ -310,8 +314,10 @@ int launch_fused(const float *g, const float *w, const float *feat, const int *m
 int launch_accumulate_grad_fused(const float *g, const float *w, const float *feat, const int *maxidx,
                                  const unsigned char *maxslot, const int *inv_off, const int *inv_slots, float *gw,
                                  float *gfeat, int n_vert, int K, int F, int g_cols, bool mean_and_max, const int *idx,
-                                 const int *order, hipStream_t s) {
-    if (F % kWave != 0) return 1;
+                                 const int *order, float divisor, hipStream_t s) {
+    // gw == nullptr: the feature gradient alone (mean only; with the max part the two-kernel path does it)
+    const bool want_w = gw != nullptr;
+    if (F % kWave != 0 || (!want_w && mean_and_max)) return 1;
     const uintptr_t align_or = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(feat) |
                                reinterpret_cast<uintptr_t>(maxidx) | reinterpret_cast<uintptr_t>(gfeat);
     // rows are addressed through 32-bit buffer offsets
@@ -322,12 +328,15 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
     // wider rows would not fit the register budget that keeps 5+ waves per SIMD resident
     if (nb < 1 || vec * nb > 4) return 1;
 
-    const long long total = (long long)n_vert * K;
-    zero_padded_weight_grad_kernel<<<256, 256, 0, s>>>(inv_off, inv_slots, gw, n_vert, total);
-    int rc = check_launch("zero_padded_weight_grad_kernel");
-    if (rc) return rc;
-#define HGC_ARGS \
-    g, w, feat, maxidx, maxslot, inv_off, inv_slots, gw, gfeat, n_vert, K, F, g_cols, mean_and_max, idx, order, s
+    if (want_w) {
+        const long long total = (long long)n_vert * K;
+        zero_padded_weight_grad_kernel<<<256, 256, 0, s>>>(inv_off, inv_slots, gw, n_vert, total);
+        const int rc = check_launch("zero_padded_weight_grad_kernel");
+        if (rc) return rc;
+    }
+#define HGC_ARGS                                                                                                   \
+    g, w, feat, maxidx, maxslot, inv_off, inv_slots, gw, gfeat, n_vert, K, F, g_cols, mean_and_max, idx, order, divisor, \
+        want_w, s
     switch (vec * 10 + nb) {
         case 11: return launch_fused<1, 1>(HGC_ARGS);
         case 12: return launch_fused<1, 2>(HGC_ARGS);

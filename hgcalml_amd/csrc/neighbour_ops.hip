@@ -113,6 +113,104 @@ __global__ __launch_bounds__(256) void local_distance_kernel(const int *__restri
     dist[t] = dsq;
 }
 
+// Gradient of push_knn, both outputs from one gather: a wave owns vertex v,
+// fetches the upstream gradient rows of its K neighbours once and forms
+//   feat_grad[v, f] = sum_n grad[idx[v,n], f] * w[v,n]   (serial, slot order: the reference's sum)
+//   w_grad[v, n]    = sum_f grad[idx[v,n], f] * feat[v, f]
+// the second as per-lane partial dot products that a fixed transpose-butterfly
+// reduces for 32 slots at a time. Lane l owns features [l*VEC, l*VEC+VEC) of each
+// of the NB blocks of 64*VEC features.
+template <int VEC, int NB>
+__global__ __launch_bounds__(256) void push_grad_wave_kernel(const float *__restrict__ grad, const float *__restrict__ w,
+                                                             const float *__restrict__ feat, const int *__restrict__ idx,
+                                                             float *__restrict__ feat_grad, float *__restrict__ w_grad,
+                                                             int n_vert, int K, int F) {
+    using namespace acc;
+    constexpr int G = 32;  // slots per reduction
+    constexpr int U = 8;   // gathered rows in flight
+    const int v = wave_vertex(nullptr, n_vert);
+    if (v >= n_vert) return;
+    const int lane = lane_id();
+    const int *irow = idx + (size_t)v * K;
+    const float *wrow = w + (size_t)v * K;
+    const RowMatrix X(grad, n_vert, F);
+    uint32_t lane_bytes[NB];
+    float own[NB][VEC], sum[NB][VEC];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int fb = (b * kWave + lane) * VEC;
+        lane_bytes[b] = (uint32_t)fb * 4u;
+        load_vec<VEC>(feat + (size_t)v * F + fb, own[b]);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) sum[b][e] = 0.f;
+    }
+    for (int l0 = 0; l0 < K; l0 += G) {
+        float val[G];
+#pragma unroll
+        for (int i = 0; i < G; ++i) val[i] = 0.f;
+#pragma unroll
+        for (int u0 = 0; u0 < G; u0 += U) {
+            if (l0 + u0 >= K) break;  // wave-uniform
+            int j[U];
+            float wl[U];
+            float x[U][NB][VEC];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int l = min(l0 + u0 + u, K - 1);
+                j[u] = l0 + u0 + u < K ? irow[l] : -1;
+                wl[u] = wrow[l];
+            }
+            // slots without a neighbour read row 0 and are left out of the sum; their
+            // weight gradient is overwritten with 0 below
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+                    X.load<VEC>((uint32_t)j[u] < (uint32_t)n_vert ? j[u] : 0, lane_bytes[b], x[u][b]);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool valid = (uint32_t)j[u] < (uint32_t)n_vert;  // wave-uniform
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        val[u0 + u] = __builtin_fmaf(own[b][e], x[u][b][e], val[u0 + u]);
+                        if (valid) sum[b][e] = sum[b][e] + x[u][b][e] * wl[u];
+                    }
+            }
+        }
+        const float r = transpose_reduce_32(val);  // lane L: slot l0 + (L & 31)
+        const int l = l0 + lane;
+        if (lane < G && l < K) w_grad[(size_t)v * K + l] = (uint32_t)irow[l] < (uint32_t)n_vert ? r : 0.f;
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) store_vec<VEC>(feat_grad + (size_t)v * F + (lane_bytes[b] >> 2), sum[b]);
+}
+
+// returns 1 when the shape is not covered
+int launch_push_grad_wave(const float *grad, const float *w, const float *feat, const int *idx, float *feat_grad,
+                          float *w_grad, int n_vert, int K, int F, hipStream_t s) {
+    using namespace acc;
+    if (F % kWave != 0 || (unsigned long long)n_vert * (unsigned long long)F * 4ull >= (1ull << 32)) return 1;
+    const uintptr_t align_or = reinterpret_cast<uintptr_t>(grad) | reinterpret_cast<uintptr_t>(feat) |
+                               reinterpret_cast<uintptr_t>(feat_grad);
+    const int vec = wave_vec(F, align_or);
+    const int nb = F / (kWave * vec);
+    const dim3 grid(ceil_div(n_vert, 4)), block(256);
+#define HGC_PUSH_GRAD(VEC, NB) \
+    push_grad_wave_kernel<VEC, NB><<<grid, block, 0, s>>>(grad, w, feat, idx, feat_grad, w_grad, n_vert, K, F)
+    switch (vec * 10 + nb) {
+        case 11: HGC_PUSH_GRAD(1, 1); break;
+        case 12: HGC_PUSH_GRAD(1, 2); break;
+        case 13: HGC_PUSH_GRAD(1, 3); break;
+        case 21: HGC_PUSH_GRAD(2, 1); break;
+        case 41: HGC_PUSH_GRAD(4, 1); break;
+        default: return 1;
+    }
+#undef HGC_PUSH_GRAD
+    return check_launch("push_grad_wave_kernel");
+}
+
 }  // namespace
 }  // namespace hgc
 
@@ -161,6 +259,16 @@ int hgc_push_knn(const float *d_weights, const float *d_feat, const int *d_idxs,
 int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *d_feat, const int *d_idxs,
                       float *d_feat_grad, float *d_w_grad, int n_vert, int n_neigh, int n_feat, hgc_stream_t stream) {
     HGC_REQUIRE(n_vert <= 0 || (d_feat_grad && d_w_grad), "null pointer");
+    HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
+    HGC_REQUIRE((long long)n_vert * std::max(n_neigh, n_feat) < (1ll << 31), "tensor too large for int32 indexing");
+    if (n_vert == 0) return HGC_OK;
+    HGC_REQUIRE(d_grad && d_weights && d_feat && d_idxs, "null pointer");
+    {
+        // both gradients from one gather pass where that kernel covers the shape
+        const int rc = launch_push_grad_wave(d_grad, d_weights, d_feat, d_idxs, d_feat_grad, d_w_grad, n_vert, n_neigh,
+                                             n_feat, as_stream(stream));
+        if (rc <= 0) return rc;
+    }
     // feat_grad[v, f] = sum_n grad[idx[v,n], f] * w[v,n]: the mean-only forward over `grad`, not divided by K
     int rc = accumulate_forward(d_weights, d_grad, d_idxs, d_feat_grad, nullptr, nullptr, n_vert, n_neigh, n_feat,
                                 n_feat, 0, 1.f, nullptr, stream);
