@@ -201,8 +201,31 @@ __device__ __forceinline__ uint64_t merge_lowest_64(uint64_t list, uint64_t batc
     return bitonic_merge_steps<128>(rev < list ? rev : list);
 }
 
+// Merges an ascending batch of 64 keys into the list of S ascending runs of 64
+// (run s holds ranks 64 s .. 64 s + 63): run by run, min(run[i], carry[63-i])
+// and max(run[i], carry[63-i]) are bitonic sequences that hold the 64 smallest
+// and the 64 largest of the two; six steps sort each, the smaller half stays,
+// the larger one is carried to the next run. What falls off the last run is dropped.
+template <int S>
+__device__ __forceinline__ void merge_batch(uint64_t (&key)[S], uint64_t batch) {
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        if (s + 1 == S) {
+            key[s] = merge_lowest_64(key[s], batch);
+        } else {
+            const uint64_t rev = from_lane_u64(batch, (kWave - 1) - lane_id());
+            const bool take = rev < key[s];
+            const uint64_t low = take ? rev : key[s], high = take ? key[s] : rev;
+            key[s] = bitonic_merge_steps<128>(low);
+            batch = bitonic_merge_steps<128>(high);
+        }
+    }
+}
+
 // below this many entering candidates in a step of 64 the one-by-one insert is cheaper
 constexpr int kBulkInsertMin = 16;
+// lists of more runs than this would insert one by one (a merge costs 12 more steps per run)
+constexpr int kBulkInsertMaxRuns = 8;
 
 // Candidates of one batch of segments that are walked per refill of a wave's
 // strip of segment marks (one byte of LDS each); a multiple of 512.
@@ -451,11 +474,12 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                         // below the K-th key and (keys compare like distances) within the radius
                         uint64_t beats = valid & __builtin_amdgcn_ballot_w64(ck < cut);
                         if (beats) {
-                            if (S == 1 && (int)__popcll(beats) >= kBulkInsertMin) {
+                            if (S <= kBulkInsertMaxRuns && (int)__popcll(beats) >= kBulkInsertMin) {
                                 const bool enters = __builtin_amdgcn_inverse_ballot_w64(beats);
                                 const uint64_t batch = wave_sort_u64(enters ? ck : kEmptyKey);
                                 // an empty list (its smallest key is the empty key) is replaced
-                                key[0] = readlane_u64(key[0], 0) == kEmptyKey ? batch : merge_lowest_64(key[0], batch);
+                                if (readlane_u64(key[0], 0) == kEmptyKey) key[0] = batch;
+                                else merge_batch<S>(key, batch);
                                 beats = 0;
                             }
                             while (beats) {
