@@ -489,14 +489,11 @@ __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__re
 
 // ------------------------------------------------------------------ inverse index
 
-__global__ __launch_bounds__(256) void inverse_keys_kernel(const int *__restrict__ idx, unsigned int *__restrict__ keys,
-                                                           int *__restrict__ slots, long long total, int n_vert) {
-    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= total) return;
-    const int j = idx[i];
-    keys[i] = (unsigned)j < (unsigned)n_vert ? (unsigned)j : (unsigned)n_vert;  // invalid -> sorts last
-    slots[i] = (int)i;
-}
+// sort key of a neighbour slot: its target, or n_vert for "no neighbour" (sorts last)
+struct InverseKey {
+    unsigned n_vert;
+    __host__ __device__ unsigned operator()(int j) const { return (unsigned)j < n_vert ? (unsigned)j : n_vert; }
+};
 
 __global__ __launch_bounds__(256) void inverse_offsets_kernel(const unsigned int *__restrict__ sorted_keys,
                                                               long long total, int *__restrict__ offsets, int n_vert) {
@@ -768,10 +765,10 @@ int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int 
 size_t hgc_inverse_neighbour_index_workspace_bytes(int n_vert, int n_neigh) {
     const size_t total = std::max<size_t>((size_t)n_vert * n_neigh, 1);
     size_t temp = 0;
-    (void)rocprim::radix_sort_pairs(nullptr, temp, (const unsigned int *)nullptr, (unsigned int *)nullptr,
-                                    (const int *)nullptr, (int *)nullptr, total, 0,
+    (void)rocprim::radix_sort_pairs(nullptr, temp, rocprim::make_transform_iterator((const int *)nullptr, InverseKey{1u}),
+                                    (unsigned int *)nullptr, rocprim::counting_iterator<int>(0), (int *)nullptr, total, 0,
                                     inverse_key_bits(std::max(n_vert, 1)), (hipStream_t) nullptr);
-    return align_up(temp) + 3 * align_up(total * sizeof(int));
+    return align_up(temp) + align_up(total * sizeof(int));
 }
 
 int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh, int *d_inv_offsets, int *d_inv_slots,
@@ -787,16 +784,15 @@ int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh, int 
         return fail(HGC_ERR_WORKSPACE, "inverse_neighbour_index workspace missing, misaligned or too small");
     const long long total = (long long)n_vert * n_neigh;
     Carver carve(workspace);
-    unsigned int *keys = carve.take<unsigned int>(total);
     unsigned int *keys_sorted = carve.take<unsigned int>(total);
-    int *slots = carve.take<int>(total);
     void *temp = carve.base + carve.used;
     size_t temp_bytes = workspace_bytes - carve.used;
-    inverse_keys_kernel<<<ceil_div(total, 256), 256, 0, s>>>(d_idxs, keys, slots, total, n_vert);
-    int rc = check_launch("inverse_keys");
-    if (rc) return rc;
-    // stable: inside one target the flat slots stay ascending, i.e. (vertex, slot) order
-    HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, slots, d_inv_slots, (size_t)total, 0,
+    // Keys and values are generated on the fly: key = the slot's target (invalid
+    // ones sort last), value = the flat slot itself. Stable: inside one target the
+    // flat slots stay ascending, i.e. (vertex, slot) order.
+    const auto keys_in = rocprim::make_transform_iterator(d_idxs, InverseKey{(unsigned)n_vert});
+    const rocprim::counting_iterator<int> slots_in(0);
+    HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_sorted, slots_in, d_inv_slots, (size_t)total, 0,
                                       inverse_key_bits(n_vert), s));
     inverse_offsets_kernel<<<ceil_div((long long)n_vert + 1, 256), 256, 0, s>>>(keys_sorted, total, d_inv_offsets, n_vert);
     return check_launch("inverse_offsets");
