@@ -105,6 +105,19 @@ __device__ __forceinline__ int xcd_contiguous_block(int bid, int nblocks) {
     return (bid % kNumXcd) * per + bid / kNumXcd;
 }
 
+// Same idea in chunks: tiles [c*CHUNK, (c+1)*CHUNK) go to XCD c % 8, so that an
+// XCD's concurrent workgroups still work on neighbouring tiles while every XCD
+// gets its share of every part of the tile range. For work whose cost varies
+// along the range (one XCD-sized contiguous piece would finish long after
+// another).
+template <int CHUNK>
+__device__ __forceinline__ int xcd_chunked_block(int bid, int nblocks) {
+    const int body = nblocks / (kNumXcd * CHUNK) * (kNumXcd * CHUNK);
+    if (bid >= body) return bid;  // ragged tail keeps its index
+    const int xcd = bid % kNumXcd, k = bid / kNumXcd;  // the k-th block this XCD receives
+    return ((k / CHUNK) * kNumXcd + xcd) * CHUNK + k % CHUNK;
+}
+
 __device__ __forceinline__ int readlane_i32(int v, int lane) {
     return __builtin_amdgcn_readlane(v, lane);
 }

@@ -263,7 +263,9 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
     constexpr int kDims = NB > 0 ? NB : kMaxBinDims;  // array extents
     __shared__ __attribute__((aligned(8))) uint8_t mark_strips[kQueriesPerBlock][kMarkCap];
     const int lane = lane_id();
-    const int tile = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    // queries come in bin order and differ a lot in cost from region to region:
+    // chunks of 512 of them are dealt to the XCDs in turn
+    const int tile = xcd_chunked_block<512>(blockIdx.x, gridDim.x);
     const int q = tile * kQueriesPerBlock + (threadIdx.x >> 6);  // one query per wave
     uint8_t *const marks = mark_strips[threadIdx.x >> 6];
     if (q >= p.n_vert) return;
