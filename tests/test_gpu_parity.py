@@ -149,6 +149,28 @@ def test_knn_cfg3_ragged_radius(oracle):
     assert (dist.cpu().numpy()[:, 1:][pad] == 0).all()
 
 
+def test_knn_cfg3_full_size_properties(oracle):
+    """16 ragged events, 1.1 M points, K=32, radius 0.1 at full size: structure of
+    every row, and sampled rows against a brute force inside their event"""
+    from hgcalml_amd import BinnedSelectKnn
+    c = workloads.cfg3()
+    idx, dist = BinnedSelectKnn(c["K"], t(c["coords"]), t(c["row_splits"]), n_bins=c["n_bins"], max_radius=c["max_radius"])
+    i, d = idx.cpu().numpy(), dist.cpu().numpy()
+    n = len(c["coords"])
+    assert (i[:, 0] == np.arange(n)).all() and (d[:, 0] == 0).all()
+    pad = i[:, 1:] < 0
+    assert (np.diff(pad.astype(np.int8), axis=1) >= 0).all() and (d[:, 1:][pad] == 0).all()
+    r2 = np.float32(np.float32(c["max_radius"]) * np.float32(c["max_radius"]))
+    assert (d <= r2).all()
+    filled = np.where(pad, np.float32(3e38), d[:, 1:])
+    assert (np.diff(filled, axis=1) >= 0)[~pad[:, 1:]].all()  # ascending distances up to the padding
+    ev = np.searchsorted(c["row_splits"][1:], np.arange(n), side="right")
+    nb = np.where(pad, np.arange(n)[:, None], i[:, 1:])
+    assert (ev[nb] == ev[:, None]).all()  # neighbours stay inside the event
+    rows = np.random.default_rng(19).choice(n, 200, replace=False)
+    assert check_knn_rows(oracle, i, d, c["coords"], c["row_splits"], c["K"], rows, radius=c["max_radius"]) == 0
+
+
 @pytest.mark.parametrize("C,B", [(2, 2), (3, 3), (3, 2), (4, 3), (5, 3), (6, 4), (5, 5)])
 def test_knn_dimensions(oracle, C, B):
     from hgcalml_amd import BinnedSelectKnn
