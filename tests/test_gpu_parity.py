@@ -688,6 +688,40 @@ def test_knn_pipeline_bin_order_groups_points_by_bin(oracle, case):
     assert (np.diff(flat[order]) >= 0).all()
 
 
+def test_knn_and_accumulate_replay_from_a_hip_graph():
+    """the kNN pipeline + accumulate forward make no host round trip, so one step
+    can be captured into a HIP graph; every replay (with eager work and
+    synchronisations in between) returns the eager bits"""
+    from hgcalml_amd import AccumulateKnn, BinnedSelectKnn
+    cfg = workloads.cfg2(scale=0.1)
+    coords, rs, feat = t(cfg["coords"]), t(cfg["row_splits"]), t(cfg["features"])
+
+    def step():
+        idx, dist = BinnedSelectKnn(32, coords, rs, n_bins=12)
+        out, arg = AccumulateKnn(dist, feat, idx)
+        return idx, dist, out, arg
+
+    with torch.no_grad():
+        ref = [x.clone() for x in step()]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = step()
+        for _ in range(4):
+            for x in outs:
+                x.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert all(torch.equal(a, b) for a, b in zip(outs, ref))
+            eager = step()
+            torch.cuda.synchronize()
+            assert all(torch.equal(a, b) for a, b in zip(eager, ref))
+
+
 def test_vertex_processing_order_changes_nothing(oracle):
     """the kNN hands its bin order to the accumulation as a processing order:
     same bits with it, without it and with an arbitrary permutation"""
