@@ -518,9 +518,15 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int
         const int assigned_words = ceil_div(std::max(n_vert, 1), 32);
         constexpr size_t kDynamicLdsLimit = 144 * 1024;  // of 160 KB; the kernel has ~9 KB of static tables
         const size_t flag_bytes = (size_t)flag_words * 4, both_bytes = flag_bytes + (size_t)assigned_words * 4;
-        if (assign_by_max_beta && both_bytes <= kDynamicLdsLimit) {
-            HGC_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&condensate_event_kernel<true, true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamicLdsLimit));
+        // more than the default 64 KB of dynamic LDS has to be granted per kernel; without
+        // the grant the variant without assigned bits runs
+        const bool with_assigned_bits =
+            assign_by_max_beta && both_bytes <= kDynamicLdsLimit &&
+            (both_bytes <= 48 * 1024 ||
+             hipFuncSetAttribute(reinterpret_cast<const void *>(&condensate_event_kernel<true, true>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamicLdsLimit) == hipSuccess);
+        (void)hipGetLastError();  // a refused grant is not an error of this call
+        if (with_assigned_bits) {
             condensate_event_kernel<true, true><<<num_rows, kBlock, both_bytes, s>>>(p, flag_words, assigned_words);
         } else if (flag_bytes <= 48 * 1024) {
             condensate_event_kernel<true, false><<<num_rows, kBlock, flag_bytes, s>>>(p, flag_words, 0);
