@@ -84,3 +84,32 @@ def test_random_configuration(oracle, seed):
                                                  assign_by_max_beta=mode)
     for a, b in zip(got, ref):
         assert (a.cpu().numpy() == b).all()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_knn_long_lists_and_dense_blobs(oracle, seed):
+    """neighbour lists of several runs of 64 (K > 65) and points crowded into a
+    few bins; rows that differ from the oracle must be exact ties at the K-th
+    boundary (a dense blob produces a few)"""
+    from helpers import check_knn_rows
+    from hgcalml_amd import BinnedSelectKnn
+    rng = np.random.default_rng(3000 + seed)
+    n = int(rng.integers(400, 7000))
+    C = int(rng.integers(2, 6))
+    K = int(rng.choice([66, 129, 130, 200, 300]))
+    n_ev = int(rng.integers(1, 3))
+    rs = np.concatenate([[0], np.sort(rng.integers(0, n + 1, n_ev - 1)), [n]]).astype(np.int32)
+    kind = int(rng.integers(0, 3))
+    coords = (rng.random((n, C), dtype=np.float32) if kind == 0 else
+              rng.standard_normal((n, C)).astype(np.float32) if kind == 1 else
+              np.concatenate([0.5 + 0.01 * rng.standard_normal((n - n // 5, C)),
+                              rng.random((n // 5, C))]).astype(np.float32)[rng.permutation(n)])
+    nb = int(rng.integers(3, 16))
+    radius = None if rng.random() < 0.7 else float(rng.random() * 0.5 + 0.05)
+    idx, dist = BinnedSelectKnn(K, t(coords), t(rs), n_bins=nb, max_radius=radius)
+    ri, rd = oracle.canonical_knn(*oracle.BinnedSelectKnn(K, coords, rs, n_bins=nb, max_radius=radius))
+    gi, gd = idx.cpu().numpy(), dist.cpu().numpy()
+    differ = np.nonzero((gi != ri).any(1) | (bits(gd) != bits(rd)).any(1))[0]
+    kw = {} if radius is None else {"radius": radius}
+    assert check_knn_rows(oracle, gi, gd, coords, rs, K, differ, **kw) == len(differ)
+    assert len(differ) <= n // 100
