@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void index_replacer_kernel(const int *__restri
         out[i] = repl[v];
 }
 
-// ---- bin order in five launches (no order guarantee inside a bin) -------------
+// ---- bin order by counting (no order guarantee inside a bin) -------------------
 //
 // For callers that only need the points grouped by bin: a counting sort whose
 // rank inside the bin is the order in which the points' atomic increments
