@@ -72,8 +72,20 @@ def event_ms(fn, steps, warmup):
     return float(np.mean(times)), float(np.median(times)), float(np.min(times))
 
 
-def cpu_baseline_knn(cfg, reps=5):
-    """the oracle's binned kNN kernel over all queries of cfg2, `reps` passes, one thread"""
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline_knn(cfg, reps=5, opt_level_0=False):
+    """the oracle's binned kNN kernel over all queries of cfg2, `reps` passes, one thread
+    (opt_level_0: built without optimisation, the flags of the reference's own Makefile)"""
     import oracle
     coords, rs, K = cfg["coords"], cfg["row_splits"], cfg["K"]
     dbin, flat, nb, bw, nper = oracle.BinByCoordinates(coords[:, :3], rs, n_bins=cfg["n_bins"])
@@ -82,7 +94,7 @@ def cpu_baseline_knn(cfg, reps=5):
     sc, sf, sd = coords[order], flat[order], dbin[order]
     t0 = time.perf_counter()
     for _ in range(reps):
-        oracle.binned_select_knn_kernel(K, sc, sf, sd, bb, nb, bw)
+        oracle.binned_select_knn_kernel(K, sc, sf, sd, bb, nb, bw, opt_level_0=opt_level_0)
     dt = time.perf_counter() - t0
     return reps * len(coords) / dt, dt
 
@@ -256,6 +268,11 @@ def main():
     if not args.skip_cpu_baseline:
         log("bench: CPU baseline (oracle, 1 thread): binned kNN kernel over cfg2 ...")
         qps, secs = cpu_baseline_knn(c2)
+        try:
+            qps_o0, _ = cpu_baseline_knn(c2, reps=1, opt_level_0=True)
+        except Exception as e:  # no compiler on this box and no prebuilt -O0 library
+            log("bench: -O0 oracle unavailable (%r)" % (e,))
+            qps_o0 = None
         small = workloads.cfg4(scale=0.1)
         f_s, b_s = cpu_baseline_accumulate(small)
         ns = len(small["indices"])
@@ -274,7 +291,9 @@ def main():
                "condensates_cfg5_ms": round(cond_s * 1e3, 1),
                "condensates_sample": "all of cfg5 (8 events, 500k hits, max-beta mode) through the oracle's wrapper "
                                      "(numpy glue + C kernel)",
-               "host_cpus": os.cpu_count()}
+               "value_unoptimised_build": None if qps_o0 is None else round(qps_o0, 1),
+               "unoptimised_note": "same kernel built -O0 (the reference's Makefile passes no -O flag), one pass",
+               "host_cpus": os.cpu_count(), "cpu_model": cpu_model()}
         log("bench: CPU oracle kNN %.0f queries/s (%.1f s)" % (qps, secs))
 
     line = {
