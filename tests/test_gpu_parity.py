@@ -131,6 +131,25 @@ def test_knn_cfg1_full(oracle):
     run_knn_case(oracle, c["coords"], c["row_splits"], c["K"], c["n_bins"])
 
 
+def test_cfg1_knn_then_accumulate(oracle):
+    """the reference's own CPU-runnable case end to end: kNN over 20,000 uniform 3-D points,
+    K=16, then the accumulation of F=32 features over the full table (self
+    included) and over the table without its self column (the GravNet convention)"""
+    from hgcalml_amd import AccumulateKnn, AccumulateLinKnn, BinnedSelectKnn
+    c = workloads.cfg1()
+    idx, dist = BinnedSelectKnn(c["K"], t(c["coords"]), t(c["row_splits"]), n_bins=c["n_bins"])
+    ri, rd = oracle.canonical_knn(*oracle.BinnedSelectKnn(c["K"], c["coords"], c["row_splits"], n_bins=c["n_bins"]))
+    assert (idx.cpu().numpy() == ri).all() and (bits(dist.cpu().numpy()) == bits(rd)).all()
+    for table, d2 in ((ri, rd), (ri[:, 1:].copy(), rd[:, 1:].copy())):
+        w = np.exp(-10 * d2).astype(np.float32)
+        ro, ra = oracle.AccumulateLinKnn(w, c["features"], table)
+        out, arg = AccumulateLinKnn(t(w), t(c["features"]), t(table))
+        assert (bits(out.cpu().numpy()) == bits(ro)).all() and (arg.cpu().numpy() == ra).all()
+        # exp(-x) from torch on the device against numpy's: 1e-5 relative, as for every wrapper with exp
+        out2, _ = AccumulateKnn(t(10 * d2), t(c["features"]), t(table))
+        assert np.abs(out2.cpu().numpy() - ro).max() <= 1e-5 * np.abs(ro).max()
+
+
 def test_knn_cfg2_full(oracle):
     c = workloads.cfg2()
     idx, dist = run_knn_case(oracle, c["coords"], c["row_splits"], c["K"], c["n_bins"])
