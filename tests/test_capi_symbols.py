@@ -75,7 +75,8 @@ def test_host_side_argument_checks(capi):
     capi.hgc_sort_by_bin_workspace_bytes.restype = ctypes.c_size_t
     capi.hgc_inverse_neighbour_index_workspace_bytes.restype = ctypes.c_size_t
     assert capi.hgc_sort_by_bin_workspace_bytes(150000, 27000) >= 2 * 150000 * 4
-    assert capi.hgc_inverse_neighbour_index_workspace_bytes(1000, 64) >= 3 * 64000 * 4
+    # the sorted keys, plus whatever rocPRIM asks for itself
+    assert capi.hgc_inverse_neighbour_index_workspace_bytes(1000, 64) >= 64000 * 4
     # missing workspace is reported, not dereferenced
     h = capi.hgc_sort_by_bin
     h.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
