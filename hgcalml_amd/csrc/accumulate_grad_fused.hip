@@ -14,6 +14,9 @@
 // result is bit-identical to it) and reduces the dot products of 16 entries at
 // a time across its lanes, writing each weight gradient to its own slot.
 //
+// The same kernel without the dot products (no weight gradient wanted, mean
+// only) is the ordered gather push_knn needs: out[m] = sum of w[v,n] * feat[v].
+//
 // Scalar-unit economy: the per-entry metadata (flat slot -> vertex, row offset,
 // weight, arg-max key) is computed by the 64 lanes for 64 entries at once and
 // broadcast per entry with v_readlane; the hot loop carries no scalar loads and
