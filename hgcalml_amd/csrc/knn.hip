@@ -64,9 +64,18 @@ __device__ __forceinline__ float dist_sq(const float (&q)[C > 0 ? C : 1], const 
         const float *r = reinterpret_cast<const float *>(reinterpret_cast<const char *>(coord) +
                                                          (uint32_t)j * (uint32_t)(C * sizeof(float)));
         float x[C];
-        if constexpr (C == 4) {
-            const float4 v = *reinterpret_cast<const float4 *>(r);
-            x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+        if constexpr (C == 4 || C == 8) {  // rows are 16-byte aligned (checked on the host)
+#pragma unroll
+            for (int c = 0; c < C; c += 4) {
+                const float4 v = *reinterpret_cast<const float4 *>(r + c);
+                x[c] = v.x; x[c + 1] = v.y; x[c + 2] = v.z; x[c + 3] = v.w;
+            }
+        } else if constexpr (C == 6) {     // 8-byte aligned
+#pragma unroll
+            for (int c = 0; c < C; c += 2) {
+                const float2 v = *reinterpret_cast<const float2 *>(r + c);
+                x[c] = v.x; x[c + 1] = v.y;
+            }
         } else if constexpr (C == 2) {
             const float2 v = *reinterpret_cast<const float2 *>(r);
             x[0] = v.x; x[1] = v.y;
@@ -551,13 +560,17 @@ int launch_levels(const KnnParams &p, hipStream_t s) {
     return check_launch("knn_wave_kernel");
 }
 
-// The usual shapes (binned dimensions = min(3, coordinates)) get kernels with
+// The usual shapes (binned dimensions = min(3, coordinates), up to 8 coordinates) get kernels with
 // both numbers fixed at compile time, anything else the one that reads them.
 template <bool MAPPED>
 int launch_coords(const KnnParams &p, hipStream_t s) {
     if (p.n_coords == 2 && p.n_bin_dim == 2) return launch_levels<2, 2, MAPPED>(p, s);
     if (p.n_coords == 3 && p.n_bin_dim == 3) return launch_levels<3, 3, MAPPED>(p, s);
     if (p.n_coords == 4 && p.n_bin_dim == 3) return launch_levels<4, 3, MAPPED>(p, s);
+    if (p.n_coords == 5 && p.n_bin_dim == 3) return launch_levels<5, 3, MAPPED>(p, s);
+    if (p.n_coords == 6 && p.n_bin_dim == 3) return launch_levels<6, 3, MAPPED>(p, s);
+    if (p.n_coords == 7 && p.n_bin_dim == 3) return launch_levels<7, 3, MAPPED>(p, s);
+    if (p.n_coords == 8 && p.n_bin_dim == 3) return launch_levels<8, 3, MAPPED>(p, s);
     return launch_levels<0, 0, MAPPED>(p, s);
 }
 
@@ -585,7 +598,8 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
                 "null pointer");
     HGC_REQUIRE(!use_direction || d_direction,
                 "BinnedSelectKnnOp needs a direction tensor (0,1,2,other) with length nvert if use_direction=True.");
-    HGC_REQUIRE((n_coords != 4 && n_coords != 2) || (reinterpret_cast<uintptr_t>(d_coord) & 15u) == 0,
+    HGC_REQUIRE((n_coords != 4 && n_coords != 2 && n_coords != 6 && n_coords != 8) ||
+                    (reinterpret_cast<uintptr_t>(d_coord) & 15u) == 0,
                 "coordinate matrix must be 16-byte aligned");
 
     KnnParams p;

@@ -190,7 +190,7 @@ def test_knn_cfg3_full_size_properties(oracle):
     assert check_knn_rows(oracle, i, d, c["coords"], c["row_splits"], c["K"], rows, radius=c["max_radius"]) == 0
 
 
-@pytest.mark.parametrize("C,B", [(2, 2), (3, 3), (3, 2), (4, 3), (5, 3), (6, 4), (5, 5)])
+@pytest.mark.parametrize("C,B", [(2, 2), (3, 3), (3, 2), (4, 3), (5, 3), (6, 3), (7, 3), (8, 3), (9, 3), (6, 4), (5, 5)])
 def test_knn_dimensions(oracle, C, B):
     from hgcalml_amd import BinnedSelectKnn
     rng = np.random.default_rng(16 + C * 10 + B)
