@@ -704,7 +704,7 @@ int accumulate_forward(const float *d_distances, const float *d_feat, const int 
                               reinterpret_cast<uintptr_t>(d_out_maxidxs);
     // the wave kernels address rows through 32-bit buffer offsets
     const bool fits_32bit = (unsigned long long)n_vert * (unsigned long long)n_out_feat * 4ull < (1ull << 32);
-    if (n_feat >= kWave && fits_32bit) {  // one wave per vertex
+    if (n_feat >= 16 && fits_32bit) {  // one wave per vertex (lanes beyond a short row stay idle)
         const int vec = wave_vec(n_feat, align_or);
         const dim3 grid(ceil_div(n_vert, 4)), block(256);
 #define HGC_FWD(VEC, MAX)                                                                                         \
@@ -828,17 +828,18 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
     const bool pow2k = divisor == (float)(int)divisor && is_pow2((int)divisor);
 
     const bool fits_32bit = (unsigned long long)n_vert * (unsigned long long)(2 * n_feat) * 4ull < (1ull << 32);
+    // both gradients from one gather pass where that kernel covers the shape (rows of
+    // 16 to 256 features), or the mean-only feature gradient alone: the gather without
+    // the dot products
+    if (fits_32bit && want_f && (want_w || !mean_and_max)) {
+        const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
+                                                    d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
+                                                    d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat,
+                                                    mean_and_max != 0, d_neigh_indices, d_order, divisor, s);
+        if (rc <= 0) return rc;  // 1: shape not covered, use the two-kernel path
+    }
     if (n_feat >= kWave && fits_32bit) {  // one wave per vertex, rows addressed through 32-bit buffer offsets
         const bool use_slots = d_max_slots != nullptr && n_neigh <= 254;
-        // both gradients from one gather pass where that kernel covers the shape
-        // (or the mean-only feature gradient alone: the gather without the dot products)
-        if (want_f && (want_w || !mean_and_max)) {
-            const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
-                                                        d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
-                                                        d_out_grad_features, n_vert, n_neigh, n_feat, n_grad_from_out_feat,
-                                                        mean_and_max != 0, d_neigh_indices, d_order, divisor, s);
-            if (rc <= 0) return rc;  // 1: shape not covered, use the two-kernel path
-        }
         const int vec = wave_vec(n_feat, align_or);
         const dim3 grid(ceil_div(n_vert, 4)), block(256);
         const FastDiv div_k = make_fast_div(n_neigh);

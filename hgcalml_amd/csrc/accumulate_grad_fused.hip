@@ -100,7 +100,8 @@ __device__ __forceinline__ float transpose_reduce_16(float (&val)[kGroup]) {
 
 // With arg-max slots a row's byte offset (a multiple of 512) and the entry's
 // slot share one word, so that one cross-lane read brings both.
-constexpr uint32_t kKeyMask = 511u;
+constexpr int kKeyBits = 9;
+constexpr uint32_t kKeyMask = (1u << kKeyBits) - 1u;
 // a per-lane buffer offset no matrix reaches: the hardware range check turns
 // the load into "return 0" without a memory access
 constexpr uint32_t kOutOfRange = 0xfffffff0u;
@@ -115,9 +116,10 @@ constexpr uint32_t kOutOfRange = 0xfffffff0u;
 // subnormal), and the max part is formed as (hit ? g_max : 0) * w, whose zero
 // may carry the weight's sign, which cannot change a sum that started at +0
 // (it would differ for an infinite weight only).
-template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool FAST, bool WGRAD>
+template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool FAST, bool WGRAD, bool PARTIAL>
 __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix &MI, __amdgpu_buffer_rsrc_t MS,
-                                           const uint32_t (&lane_bytes)[NB], uint32_t max_col_bytes, int c, int cnt,
+                                           const uint32_t (&lane_bytes)[NB], uint32_t max_col_bytes,
+                                           uint32_t g_row_bytes, int c, int cnt,
                                            uint64_t repmask, int self_key, int m, uint32_t offkey_v, float w_v,
                                            float wk_v, const float (&xo)[NB][VEC], const float (&xk)[NB][VEC],
                                            float (&acc)[NB][VEC], float kf, float (&val)[kGroup]) {
@@ -130,8 +132,13 @@ __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix 
         for (int u = 0; u < kRows; ++u) {
             const int li = c + h + u;  // lanes past the end of the list hold a copy of its last entry
             const uint32_t ok = (uint32_t)__builtin_amdgcn_readlane((int)offkey_v, li);
-            soff[u] = (MAX && SLOTS) ? (ok & ~kKeyMask) : ok;
-            skey[u] = (MAX && SLOTS) ? (ok & kKeyMask) : (uint32_t)m;
+            if (MAX && SLOTS && PARTIAL) {  // vertex and slot share the word, the row offset is a scalar multiply away
+                soff[u] = (ok >> kKeyBits) * g_row_bytes;
+                skey[u] = ok & kKeyMask;
+            } else {
+                soff[u] = (MAX && SLOTS) ? (ok & ~kKeyMask) : ok;
+                skey[u] = (MAX && SLOTS) ? (ok & kKeyMask) : (uint32_t)m;
+            }
             sw[u] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(w_v), li));
             swk[u] = POW2K ? __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(wk_v), li)) : 0.f;
             rep[u] = false;
@@ -171,6 +178,9 @@ __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix 
                     bool any = false;
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) any = any || hit[u][b][e];
+                    // a lane beyond the last feature (rows that do not fill their last block of
+                    // 64) aims every load out of range and so only ever holds zeros
+                    if (PARTIAL) any = any && lane_bytes[b] != kOutOfRange;
                     Gm.load_at<VEC>(soff[u], any ? lane_bytes[b] + max_col_bytes : kOutOfRange, gx[u][b]);
                 }
         }
@@ -206,7 +216,9 @@ __device__ __forceinline__ void grad_group(const RowMatrix &Gm, const RowMatrix 
 
 // WGRAD false: feature gradient only (feat, idx and gw are not touched); kf is
 // what the mean part is divided by (K for the accumulation, 1 for a plain push).
-template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool WGRAD>
+// PARTIAL: F is not a multiple of 64 (VEC is 1 then); the lanes of the last block
+// beyond F stay idle.
+template <int VEC, int NB, bool MAX, bool POW2K, bool SLOTS, bool WGRAD, bool PARTIAL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) void accumulate_grad_fused_kernel(
     const float *__restrict__ g, const float *__restrict__ w, const float *__restrict__ feat,
     const int *__restrict__ maxidx, const unsigned char *__restrict__ maxslot, const int *__restrict__ inv_off,
@@ -230,10 +242,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const int fb = (b * kWave + lane) * VEC;
-        lane_bytes[b] = (uint32_t)fb * 4u;
+        const bool in_row = !PARTIAL || fb < F;
+        lane_bytes[b] = in_row ? (uint32_t)fb * 4u : kOutOfRange;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) xo[b][e] = 0.f;
-        if (WGRAD) load_vec<VEC>(feat + (size_t)m * F + fb, xo[b]);
+        if (WGRAD && in_row) load_vec<VEC>(feat + (size_t)m * F + fb, xo[b]);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) xk[b][e] = (float)((double)xo[b][e] * inv_kd);
 #pragma unroll
@@ -256,7 +269,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
         const int v = fast_div(slot_v, div_k);
         const int key_v = slot_v - v * K;
         // row offset of the entry's vertex, with the entry's slot in its low bits
-        const uint32_t offkey_v = (uint32_t)v * g_row_bytes | ((MAX && SLOTS) ? (uint32_t)key_v : 0u);
+        // (rows that are no multiple of 512 bytes have no free low bits: vertex and slot are packed instead)
+        const uint32_t offkey_v = (MAX && SLOTS && PARTIAL)
+                                      ? ((uint32_t)v << kKeyBits) | (uint32_t)key_v
+                                      : (uint32_t)v * g_row_bytes | ((MAX && SLOTS) ? (uint32_t)key_v : 0u);
         const float wk_v = w_v * inv_kf;
         const uint64_t repmask = MAX ? __ballot(v == m && key_v != self_key && lane < cnt) : 0ull;
         for (int c = 0; c < cnt; c += kGroup) {
@@ -265,10 +281,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
             for (int i = 0; i < kGroup; ++i) val[i] = 0.f;
             const bool fast = (c + kGroup <= cnt) && ((repmask >> c) & ((1ull << kGroup) - 1)) == 0;
             if (fast)
-                grad_group<VEC, NB, MAX, POW2K, SLOTS, true, WGRAD>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
+                grad_group<VEC, NB, MAX, POW2K, SLOTS, true, WGRAD, PARTIAL>(Gm, MI, MS, lane_bytes, max_col_bytes, g_row_bytes, c, cnt, repmask,
                                                                     self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
             else
-                grad_group<VEC, NB, MAX, POW2K, SLOTS, false, WGRAD>(Gm, MI, MS, lane_bytes, max_col_bytes, c, cnt, repmask,
+                grad_group<VEC, NB, MAX, POW2K, SLOTS, false, WGRAD, PARTIAL>(Gm, MI, MS, lane_bytes, max_col_bytes, g_row_bytes, c, cnt, repmask,
                                                                      self_key, m, offkey_v, w_v, wk_v, xo, xk, acc, kf, val);
             if (WGRAD) {
                 const float r = transpose_reduce_16(val);  // lane L: entry c + (L & 15)
@@ -278,7 +294,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
         }
     }
 #pragma unroll
-    for (int b = 0; b < NB; ++b) store_vec<VEC>(gfeat + (size_t)m * F + (lane_bytes[b] >> 2), acc[b]);
+    for (int b = 0; b < NB; ++b)
+        if (!PARTIAL || lane_bytes[b] != kOutOfRange) store_vec<VEC>(gfeat + (size_t)m * F + (lane_bytes[b] >> 2), acc[b]);
 }
 
 // weight gradient of padded slots (index < 0 or out of range): they sort to the
@@ -292,7 +309,7 @@ __global__ __launch_bounds__(256) void zero_padded_weight_grad_kernel(const int 
         gw[inv_slots[i]] = 0.f;
 }
 
-template <int VEC, int NB>
+template <int VEC, int NB, bool PARTIAL>
 int launch_fused(const float *g, const float *w, const float *feat, const int *maxidx, const unsigned char *maxslot,
                  const int *inv_off, const int *inv_slots, float *gw, float *gfeat, int n_vert, int K, int F, int g_cols,
                  bool mean_and_max, const int *idx, const int *order, float divisor, bool want_w, hipStream_t s) {
@@ -301,7 +318,7 @@ int launch_fused(const float *g, const float *w, const float *feat, const int *m
     const bool pow2k = divisor == (float)(int)divisor && is_pow2((int)divisor);
     const bool slots = mean_and_max && maxslot != nullptr;
 #define HGC_FUSED(MAX, P2, SL, WG)                                                                                       \
-    accumulate_grad_fused_kernel<VEC, NB, MAX, P2, SL, WG><<<grid, block, 0, s>>>(g, w, feat, maxidx, maxslot, inv_off, \
+    accumulate_grad_fused_kernel<VEC, NB, MAX, P2, SL, WG, PARTIAL><<<grid, block, 0, s>>>(g, w, feat, maxidx, maxslot, inv_off, \
                                                                                   inv_slots, gw, gfeat, n_vert, K, F,    \
                                                                                   g_cols, div_k, idx, order, divisor)
     if (!want_w) { if (pow2k) HGC_FUSED(false, true, false, false); else HGC_FUSED(false, false, false, false); }
@@ -320,14 +337,16 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
                                  const int *order, float divisor, hipStream_t s) {
     // gw == nullptr: the feature gradient alone (mean only; with the max part the two-kernel path does it)
     const bool want_w = gw != nullptr;
-    if (F % kWave != 0 || (!want_w && mean_and_max)) return 1;
+    if (F < 16 || (!want_w && mean_and_max)) return 1;
+    const bool partial = F % kWave != 0;  // the last block of 64 lanes is not full
+    if (partial && n_vert >= (1 << (32 - kKeyBits))) return 1;  // vertex and slot share one word there
     const uintptr_t align_or = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(feat) |
                                reinterpret_cast<uintptr_t>(maxidx) | reinterpret_cast<uintptr_t>(gfeat);
     // rows are addressed through 32-bit buffer offsets
     if ((unsigned long long)n_vert * (unsigned long long)g_cols * 4ull >= (1ull << 32)) return 1;
     if (maxslot && K > 254) maxslot = nullptr;
-    const int vec = wave_vec(F, align_or);
-    const int nb = F / (kWave * vec);
+    const int vec = partial ? 1 : wave_vec(F, align_or);
+    const int nb = ceil_div(F, kWave * vec);
     // wider rows would not fit the register budget that keeps 5+ waves per SIMD resident
     if (nb < 1 || vec * nb > 4) return 1;
 
@@ -340,13 +359,21 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
 #define HGC_ARGS                                                                                                   \
     g, w, feat, maxidx, maxslot, inv_off, inv_slots, gw, gfeat, n_vert, K, F, g_cols, mean_and_max, idx, order, divisor, \
         want_w, s
+    if (partial) {
+        switch (nb) {
+            case 1: return launch_fused<1, 1, true>(HGC_ARGS);
+            case 2: return launch_fused<1, 2, true>(HGC_ARGS);
+            case 3: return launch_fused<1, 3, true>(HGC_ARGS);
+        }
+        return 1;
+    }
     switch (vec * 10 + nb) {
-        case 11: return launch_fused<1, 1>(HGC_ARGS);
-        case 12: return launch_fused<1, 2>(HGC_ARGS);
-        case 13: return launch_fused<1, 3>(HGC_ARGS);
-        case 21: return launch_fused<2, 1>(HGC_ARGS);
-        case 22: return launch_fused<2, 2>(HGC_ARGS);
-        case 41: return launch_fused<4, 1>(HGC_ARGS);
+        case 11: return launch_fused<1, 1, false>(HGC_ARGS);
+        case 12: return launch_fused<1, 2, false>(HGC_ARGS);
+        case 13: return launch_fused<1, 3, false>(HGC_ARGS);
+        case 21: return launch_fused<2, 1, false>(HGC_ARGS);
+        case 22: return launch_fused<2, 2, false>(HGC_ARGS);
+        case 41: return launch_fused<4, 1, false>(HGC_ARGS);
     }
 #undef HGC_ARGS
     return 1;

@@ -217,7 +217,7 @@ int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int 
  * adjacent in memory share no neighbours and every gathered row misses L2;
  * given the kNN's bin order (d_out_sorting of hgc_binned_select_knn_pipeline)
  * concurrent waves work on spatial neighbours and share their rows (measured
- * 1.9x on the forward, N=150k, K=64, F=64). Honoured for n_feat >= 64. */
+ * 1.9x on the forward, N=150k, K=64, F=64). Honoured for n_feat >= 16. */
 int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, const int *d_idxs,
                              float *d_out_feat, int *d_out_maxidxs, unsigned char *d_out_maxslots,
                              const int *d_vertex_order,

@@ -316,7 +316,8 @@ def grad_tolerance(g, x, idx, w, K):
     return 1e-5 * scale + 1e-30
 
 
-@pytest.mark.parametrize("K,F", [(8, 4), (16, 32), (64, 64), (12, 128), (5, 7), (64, 96), (9, 384), (260, 64), (255, 128)])
+@pytest.mark.parametrize("K,F", [(8, 4), (16, 32), (64, 64), (12, 128), (5, 7), (64, 96), (9, 384), (260, 64), (255, 128),
+                                  (16, 16), (12, 48), (33, 160), (7, 20)])
 def test_accumulate_gradient(oracle, K, F):
     rng = np.random.default_rng(20 + K + F)
     d, x, idx = make_acc_case(rng, 300, K, F)
@@ -336,7 +337,7 @@ def test_accumulate_gradient(oracle, K, F):
         assert (gw.cpu().numpy()[idx < 0] == 0).all()
 
 
-@pytest.mark.parametrize("K,F", [(16, 32), (64, 64), (64, 128), (20, 192), (12, 256), (10, 512)])
+@pytest.mark.parametrize("K,F", [(16, 32), (64, 64), (64, 128), (20, 192), (12, 256), (10, 512), (24, 48), (9, 160), (64, 17)])
 def test_accumulate_slot_table_path(oracle, K, F):
     """forward with arg-max slots + gradient fed with them: same bits as the
     index-comparing path and as the oracle, including repeated self references"""
