@@ -162,6 +162,38 @@ __device__ __forceinline__ void fwd_slot(const float (&x)[VEC], float wn, int sl
     }
 }
 
+// Up to U slots [n_begin, n_end) of a vertex's row where some have no neighbour,
+// or the short last chunk of a row: index and weight of slot n_begin + l sit in
+// lane l and are broadcast with v_readlane (no arrays of scalars to keep alive),
+// all rows are in flight together, a slot without a neighbour fetches row 0 and
+// is skipped. Returns n_begin so that the caller's loop advances as for a full chunk.
+template <int VEC, bool MAX, int U>
+__device__ __forceinline__ int partial_chunk(const RowMatrix &X, const int *__restrict__ irow,
+                                             const float *__restrict__ wrow, int n_begin, int n_end, int n_vert,
+                                             uint32_t lane_bytes, float (&sum)[VEC], float (&best)[VEC], int (&arg)[VEC]) {
+    const int lane = lane_id();
+    const int n_mine = min(n_begin + lane, n_end - 1);
+    const int j_lane = n_begin + lane < n_end ? irow[n_mine] : -1;
+    const float w_lane = wrow[n_mine];
+    const uint64_t valid = __ballot((uint32_t)j_lane < (uint32_t)n_vert);  // bit l: slot n_begin + l has a neighbour
+    float x[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int j = __builtin_amdgcn_readlane(j_lane, u);
+        X.load<VEC>((valid >> u) & 1ull ? j : 0, lane_bytes, x[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        if (!((valid >> u) & 1ull)) continue;  // wave-uniform
+        const float w = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(w_lane), u));
+        if (n_begin + u == 0)
+            fwd_slot<VEC, MAX, true>(x[u], w, 0, sum, best, arg);
+        else
+            fwd_slot<VEC, MAX, false>(x[u], w, n_begin + u, sum, best, arg);
+    }
+    return n_begin;
+}
+
 template <int VEC, bool MAX>
 __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *__restrict__ w,
                                                                   const float *__restrict__ feat,
@@ -220,28 +252,21 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                     for (int u = 0; u < U; ++u) fwd_slot<VEC, MAX, false>(x[u], wn[u], n0 + u, sum, best, arg);
                 }
             } else {
-                for (int u = 0; u < U; ++u) {
-                    const int jj = irow[n0 + u];
-                    if ((unsigned)jj >= (unsigned)n_vert) continue;
-                    float xs[VEC];
-                    X.load<VEC>(jj, lane_bytes, xs);
-                    if (n0 + u == 0)
-                        fwd_slot<VEC, MAX, true>(xs, wrow[0], 0, sum, best, arg);
-                    else
-                        fwd_slot<VEC, MAX, false>(xs, wrow[n0 + u], n0 + u, sum, best, arg);
-                }
+                n0 = partial_chunk<VEC, MAX, U>(X, irow, wrow, n0, n0 + U, n_vert, lane_bytes, sum, best, arg);
             }
         }
-        for (; n0 < K; ++n0) {  // K not a multiple of U
-            const int jj = irow[n0];
-            if ((unsigned)jj >= (unsigned)n_vert) continue;
-            if (jj == v && first_self < 0) first_self = n0;
-            float xs[VEC];
-            X.load<VEC>(jj, lane_bytes, xs);
-            if (n0 == 0)
-                fwd_slot<VEC, MAX, true>(xs, wrow[0], 0, sum, best, arg);
+        if (n0 < K) {  // K not a multiple of U
+            if (MAX) {
+                const int n_mine = min(n0 + lane_id(), K - 1);
+                const uint64_t self = __ballot(n0 + lane_id() < K && irow[n_mine] == v);
+                if (first_self < 0 && self) first_self = n0 + __builtin_ctzll(self);
+            }
+            if (K - n0 <= 4)
+                partial_chunk<VEC, MAX, 4>(X, irow, wrow, n0, K, n_vert, lane_bytes, sum, best, arg);
+            else if (K - n0 <= 8 || U == 8)
+                partial_chunk<VEC, MAX, 8>(X, irow, wrow, n0, K, n_vert, lane_bytes, sum, best, arg);
             else
-                fwd_slot<VEC, MAX, false>(xs, wrow[n0], n0, sum, best, arg);
+                partial_chunk<VEC, MAX, 16>(X, irow, wrow, n0, K, n_vert, lane_bytes, sum, best, arg);
         }
         float mean[VEC];
 #pragma unroll
