@@ -7,19 +7,38 @@
 //   modules/compiled/binstepper.h:100-165                           (box of bins)
 //
 // The reference picks, again and again, the unclaimed high-beta hit with the
-// largest beta (first one in bin order on ties) by a linear scan. That order
-// is static, so here the high-beta hits of every event are sorted ONCE by
-// (event, beta descending, position ascending) with a stable radix sort, and
-// one workgroup per event walks its list: the next hit that is still unclaimed
-// becomes a condensation point and all 1024 threads test the hits of its box of
-// bins (contiguous runs of the bin-sorted hits) in parallel. Only distances
-// (serial fp32 over the coordinates, no FMA contraction) and comparisons are
-// involved, so the result is the reference's bit for bit.
+// largest beta (first one in bin order on ties) by a linear scan, and lets it
+// claim the hits of its box of bins that lie inside its sphere. Two facts turn
+// that chain of claim steps into wide kernels:
+//   * the order of the picks is static: the high-beta hits of every event are
+//     sorted once by (event, beta descending, position ascending);
+//   * a high-beta hit becomes a condensation point exactly if no condensation
+//     point EARLIER in that order covers it, in both assignment modes (the
+//     first condensation point that covers a hit always claims it), and only
+//     a few hundred of tens of thousands do.
+// So the condensation points are found first, from the sorted candidates alone:
+// one workgroup per event walks the list in windows, one candidate per thread;
+// a window is resolved wave after wave (inside a wave: the first open lane is
+// a condensation point, the lanes it covers close), every later wave dropping
+// what the new points cover. Between a few launches of that kernel, whose
+// share of the list grows geometrically, a grid-wide kernel drops every
+// remaining candidate that the points found so far cover, so that the event's
+// workgroup only ever tests its candidates against the points of its own launch
+// (kept in LDS). Finally every hit looks for the points of its event that cover
+// it, in selection order: the first one (max-beta mode) or the reference's
+// running comparison over all of them (min-distance mode).
 //
-// This is latency-bound (a chain of a few hundred dependent claim steps per
-// event), not bandwidth-bound: compulsory traffic is about N*(4C+16) bytes.
+// "Covers" is the reference's claim test: inside the sphere (serial fp32 over
+// the coordinates, no FMA contraction), the hit's bin inside the point's box
+// of bins (floor((c-r)/bw) .. ceil((c+r)/bw) per binned dimension), mask rules
+// as in the reference. The reference checks only the flat index of a box cell,
+// so a box that sticks out of the grid also walks cells of the neighbouring
+// row; their hits lie outside the sphere, which makes the per-dimension test
+// here equivalent. Only comparisons and order-independent writes are involved,
+// so the result is the reference's bit for bit.
 #include "hgc_common.hpp"
 
+#include <climits>
 #include <cstring>
 #include <algorithm>
 
@@ -33,8 +52,13 @@ namespace {
 
 constexpr int kMaxDims = 16;     // coordinate dimensions
 constexpr int kMaxBinDims = 6;   // binned dimensions
-constexpr int kBlock = 1024;
+constexpr int kBlock = 1024;     // threads of an event's workgroup
 constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kFill = 4;         // windows of the sorted list looked at per refill of the queue
+constexpr int kQueueCap = kBlock + kFill * kBlock;
+constexpr int kScanBlock = 256;  // threads of the grid-wide kernels
+constexpr int kTile = 128;       // condensation points staged in LDS at a time there
+constexpr int kMaxLaunches = 4;  // launches of the event kernel
 
 struct CondParams {
     int C, B;
@@ -58,9 +82,35 @@ struct CondParams {
     const float *bin_widths;
     const int *row_splits;
     int num_rows, by_max_beta, n_vert, n_vert_h;
-    const int *order_h;   // high-beta hits in selection order, grouped by event
-    int *event_count;     // condensates found per event
+    // workspace
+    const int *order_h;  // high-beta hits in selection order, grouped by event
+    int *pos_h;          // [n_vert_h] position of a high-beta hit among all hits, -1 unknown
+    int *hit_bin;        // [n_vert] bin of a hit inside its event's grid, INT_MIN unknown
+    uint32_t *cand;      // [n_vert_h] candidate records in selection order
+    int *closed;         // [n_vert_h] by selection position: never a condensation point (cannot be
+                         // picked at all, or a point of an earlier launch covers it)
+    uint32_t *points;    // [n_vert_h] an event's condensation points in selection order, from
+                         // row_splits_h[event] on
+    int *cursor_at;      // [kMaxLaunches][num_rows] selection position an event's walk stopped at
+    int *n_alpha_at;     // [kMaxLaunches][num_rows] points of the event after that launch
 };
+
+// A candidate record (CMAX = coordinate slots, unused ones hold 0 and add an
+// exact 0 to every distance):
+//   [0, CMAX)          coordinates of its hit
+//   [CMAX, CMAX+6)     per-dimension bins of its hit, saturated to 16 bits (-32768: unknown)
+//   CMAX+6             1: its hit is masked (or unknown), no sphere claims it
+//   CMAX+7             unused
+//   [CMAX+8, ...)      the condensation point it would be:
+//     [0, CMAX) centre, CMAX radius^2, CMAX+1 q | solitary << 31, CMAX+2 original index,
+//     CMAX+3 unused, [CMAX+4, CMAX+10) box of bins per dimension, lo | hi << 16 (saturated to 16
+//     bits; dimensions that are not binned hold the full range); padded to 16 bytes
+// The box test is exact up to 16383 bins per dimension (the sphere test is what decides beyond
+// fp32 rounding at a bin boundary).
+__host__ __device__ constexpr int alpha_words(int cmax) { return (cmax + 4 + kMaxBinDims + 3) / 4 * 4; }
+__host__ __device__ constexpr int cand_words(int cmax) { return cmax + 8 + alpha_words(cmax); }
+
+__device__ __forceinline__ int saturate16(int v) { return max(-32768, min(32767, v)); }
 
 // the reference indexes the high-beta mask with the truth value of (q > 0)
 __device__ __forceinline__ bool always_first(const int *mask_h, int n_vert_h, int q) {
@@ -68,29 +118,31 @@ __device__ __forceinline__ bool always_first(const int *mask_h, int n_vert_h, in
     return slot < n_vert_h && mask_h[slot] != 0;
 }
 
-// ascending sort key == selection order
-__global__ __launch_bounds__(256) void selection_keys_kernel(const float *__restrict__ beta_h,
-                                                             const int *__restrict__ mask_h,
-                                                             const int *__restrict__ row_splits_h, int num_rows,
-                                                             int n_vert_h, uint64_t *__restrict__ keys,
-                                                             int *__restrict__ values) {
-    const int q = blockIdx.x * blockDim.x + threadIdx.x;
-    if (q >= n_vert_h) return;
-    int lo = 1, hi = num_rows + 1;  // event = last r with row_splits_h[r] <= q
+// r with splits[r] <= i < splits[r+1]
+__device__ __forceinline__ int event_of(const int *__restrict__ splits, int num_rows, int i) {
+    int lo = 1, hi = num_rows + 1;
     while (lo < hi) {
-        int mid = (lo + hi) >> 1;
-        if (row_splits_h[mid] > q)
+        const int mid = (lo + hi) >> 1;
+        if (splits[mid] > i)
             hi = mid;
         else
             lo = mid + 1;
     }
-    const uint64_t ev = (uint64_t)(lo - 1);
+    return min(lo - 1, num_rows - 1);
+}
+
+// ascending sort key == selection order; clears the per-candidate outputs
+__global__ __launch_bounds__(256) void selection_keys_kernel(const CondParams p, uint64_t *__restrict__ keys,
+                                                             int *__restrict__ values) {
+    const int q = blockIdx.x * blockDim.x + threadIdx.x;
+    if (q >= p.n_vert_h) return;
+    const uint64_t ev = (uint64_t)event_of(p.row_splits_h, p.num_rows, q);
     uint64_t cls, low;
-    if (always_first(mask_h, n_vert_h, q)) {
+    if (always_first(p.mask_h, p.n_vert_h, q)) {
         cls = 0;  // chosen as soon as it is the first unclaimed one, in position order
         low = 0;
     } else {
-        const float b = beta_h[q];
+        const float b = p.beta_h[q];
         uint32_t u = __float_as_uint(b);
         u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // monotone map float -> uint
         low = (uint32_t)~u;                               // larger beta first
@@ -98,304 +150,458 @@ __global__ __launch_bounds__(256) void selection_keys_kernel(const float *__rest
     }
     keys[q] = (ev << 34) | (cls << 32) | low;
     values[q] = q;
+    p.is_alpha_h[q] = 0;
+    p.taken_h[q] = 0;
+    p.alpha_indices[q] = -1;
+    p.pos_h[q] = -1;
 }
 
-// claimed flags of the event's high-beta hits: one bit each, in LDS when they
-// fit (LDS_FLAGS), else the caller's int array in global memory
-template <bool LDS_FLAGS>
-struct TakenFlags {
-    uint32_t *bits;  // LDS
-    int *global;     // taken_h + first_h
-    __device__ __forceinline__ bool test(int local) const {
-        if (LDS_FLAGS) return (bits[local >> 5] >> (local & 31)) & 1u;
-        return global[local] != 0;
-    }
-    __device__ __forceinline__ void set(int local) const {
-        if (LDS_FLAGS)
-            atomicOr(&bits[local >> 5], 1u << (local & 31));
+// bin of every hit inside its event's grid (from the bin boundaries), and the
+// position of every high-beta hit among all hits
+__global__ __launch_bounds__(256) void hit_prepare_kernel(const CondParams p) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= p.n_vert) return;
+    const int r = event_of(p.row_splits, p.num_rows, i);
+    int cells = 1;
+    for (int d = 0; d < p.B; ++d) cells *= p.n_bins[d];
+    const int *splits = p.bin_splits + (size_t)cells * r;
+    int lo = 0, hi = cells;  // last bin whose first hit is <= i
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (splits[mid] <= i)
+            lo = mid;
         else
-            global[local] = 1;
+            hi = mid;
+    }
+    p.hit_bin[i] = (cells > 0 && splits[lo] <= i && i < splits[lo + 1]) ? lo : INT_MIN;
+    const int q = p.to_filtered[i];
+    if (q >= 0 && q < p.n_vert_h) p.pos_h[q] = i;
+}
+
+struct Grid {
+    int nb[kMaxBinDims];
+    float bw;
+    __device__ __forceinline__ void load(const CondParams &p) {
+#pragma unroll
+        for (int d = 0; d < kMaxBinDims; ++d) nb[d] = d < p.B ? p.n_bins[d] : 1;
+        bw = p.bin_widths[0];
+    }
+    // per-dimension bin indices of a bin of the event's grid, as the box test wants them
+    __device__ __forceinline__ void split(int bin, int B, int (&k)[kMaxBinDims]) const {
+        const bool known = bin != INT_MIN;
+#pragma unroll
+        for (int d = kMaxBinDims - 1; d >= 0; --d) {
+            k[d] = d < B ? -32768 : 0;
+            if (d < B && known) {
+                k[d] = saturate16(bin % nb[d]);
+                bin /= nb[d];
+            }
+        }
     }
 };
 
-constexpr int kHitsPerThread = 4;
+// everything a candidate needs, gathered into selection order
+template <int CMAX>
+__global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams p) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= p.n_vert_h) return;
+    const int C = p.C, B = p.B;
+    Grid g;
+    g.load(p);
+    const int q = p.order_h[i];
+    const int at = p.pos_h[q];
+    uint32_t *rec = p.cand + (size_t)i * cand_words(CMAX);
+    uint32_t *point = rec + CMAX + 8;
+    float centre[CMAX];
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) {
+        centre[c] = c < C ? p.ccoords_h[(size_t)q * C + c] : 0.f;
+        rec[c] = (c < C && at >= 0) ? __float_as_uint(p.ccoords[(size_t)at * C + c]) : 0u;
+        point[c] = __float_as_uint(centre[c]);
+    }
+    int k[kMaxBinDims];
+    g.split(at >= 0 ? p.hit_bin[at] : INT_MIN, B, k);
+#pragma unroll
+    for (int d = 0; d < kMaxBinDims; ++d) rec[CMAX + d] = (uint32_t)k[d];
+    rec[CMAX + 6] = (at < 0 || p.mask[at] != 0) ? 1u : 0u;
+    rec[CMAX + 7] = 0u;
+    float radius = p.dist_h[q];
+    const bool solitary = p.mask_h[q] > 0;
+    point[CMAX] = __float_as_uint(radius * radius);
+    point[CMAX + 1] = (uint32_t)q | (solitary ? 0x80000000u : 0u);
+    point[CMAX + 2] = (uint32_t)p.orig_h[q];
+    point[CMAX + 3] = 0u;
+    if (solitary) radius = 0.f;
+#pragma unroll
+    for (int d = 0; d < kMaxBinDims; ++d) {
+        int lo = -32768, hi = 32767;
+        if (d < B) {
+            float fl = floorf((centre[d] - radius) / g.bw), fh = ceilf((centre[d] + radius) / g.bw);
+            // keep the box finite for absurd radii; the clamped range still covers
+            // every bin of the grid in this dimension
+            fl = fminf(fmaxf(fl, (float)(-g.nb[d])), (float)(2 * g.nb[d]));
+            fh = fminf(fmaxf(fh, (float)(-g.nb[d])), (float)(2 * g.nb[d]));
+            lo = saturate16((int)fl);
+            hi = saturate16((int)fh);
+        }
+        point[CMAX + 4 + d] = ((uint32_t)lo & 0xffffu) | ((uint32_t)hi << 16);
+    }
+    for (int w = CMAX + 4 + kMaxBinDims; w < alpha_words(CMAX); ++w) point[w] = 0u;
+    const bool selectable = always_first(p.mask_h, p.n_vert_h, q) || p.beta_h[q] > -1.f;
+    p.closed[i] = selectable ? 0 : 1;
+}
 
-// LDS_FLAGS: claimed flags of the high-beta hits in LDS. ASSIGNED_BITS (max-beta
-// mode only, where an assigned hit is never looked at again): one bit per hit of
-// the event in LDS says whether it is assigned, so that the claim step loads
-// coordinates and masks of unassigned hits only; most hits of a box belong to
-// earlier condensates, and one CU's load bandwidth is what the step waits for.
-template <bool LDS_FLAGS, bool ASSIGNED_BITS>
-__global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondParams p, int flag_words,
-                                                                  int assigned_words) {
-    extern __shared__ uint32_t s_bits[];
-    __shared__ int s_first[kWavesPerBlock];
-    __shared__ int s_pick, s_alpha, s_alpha_mask, s_alpha_orig;
-    __shared__ float s_alpha_centre[kMaxDims], s_alpha_dist;
-    __shared__ int s_row_off[kBlock + 1];
-    __shared__ int s_row_start[kBlock];
-    __shared__ int s_wave_tot[kWavesPerBlock];
+// The reference's claim test of one hit against one condensation point, in two
+// parts: sphere and mask rules on the first CMAX+2 words of the point ...
+template <int CMAX>
+__device__ __forceinline__ bool in_sphere(const uint32_t (&a)[CMAX + 2], const float (&x)[CMAX], bool uncoverable,
+                                          int self_q, float &dsq) {
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) {
+        const float t = __uint_as_float(a[c]) - x[c];
+        acc = acc + t * t;
+    }
+    dsq = acc;
+    if (a[CMAX + 1] >> 31) return self_q == (int)(a[CMAX + 1] & 0x7fffffffu);
+    return !uncoverable && acc <= __uint_as_float(a[CMAX]);
+}
+
+// ... and the hit's bin against the point's box of bins
+__device__ __forceinline__ bool in_box(const uint32_t (&box)[kMaxBinDims], const int (&k)[kMaxBinDims]) {
+    bool inside = true;
+#pragma unroll
+    for (int d = 0; d < kMaxBinDims; ++d)
+        inside = inside && k[d] >= (int)(int16_t)(box[d] & 0xffffu) && k[d] <= ((int)box[d] >> 16);
+    return inside;
+}
+
+// the whole test against a point in LDS (16-byte aligned); the box is only read for hits inside the sphere
+template <int CMAX>
+__device__ __forceinline__ bool covers(const uint32_t *a, const float (&x)[CMAX], bool uncoverable, int self_q,
+                                       const int (&k)[kMaxBinDims], float &dsq) {
+    uint32_t head[CMAX + 2];
+#pragma unroll
+    for (int c4 = 0; c4 < CMAX; c4 += 4) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(a + c4);
+        head[c4] = v.x, head[c4 + 1] = v.y, head[c4 + 2] = v.z, head[c4 + 3] = v.w;
+    }
+    const uint2 rs = *reinterpret_cast<const uint2 *>(a + CMAX);
+    head[CMAX] = rs.x, head[CMAX + 1] = rs.y;
+    if (!in_sphere<CMAX>(head, x, uncoverable, self_q, dsq)) return false;
+    const uint4 b0 = *reinterpret_cast<const uint4 *>(a + CMAX + 4);
+    const uint2 b1 = *reinterpret_cast<const uint2 *>(a + CMAX + 8);
+    const uint32_t box[kMaxBinDims] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y};
+    return in_box(box, k);
+}
+
+__device__ __forceinline__ int coherent_load(const int *ptr) {
+    return __hip_atomic_load(ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Finds the condensation points among the next `budget` candidates (all that are
+// left: budget < 0) of one event per workgroup. The walk over the sorted list
+// collects the candidates that are still open in a queue; `window` of them are
+// resolved at a time, one per thread; `capacity` points of this launch fit into
+// the LDS list.
+template <int CMAX>
+__global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondParams p, int launch, int budget,
+                                                                  int window, int capacity) {
+    extern __shared__ __align__(16) uint32_t s_list[];
+    __shared__ int s_queue[kQueueCap];
+    __shared__ int s_fill[kFill][kWavesPerBlock];
+    __shared__ int s_open[kWavesPerBlock], s_cnt[kWavesPerBlock];
+    constexpr int aw = alpha_words(CMAX), cw = cand_words(CMAX);
 
     const int r = blockIdx.x;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
-    const int first = p.row_splits[r], last = p.row_splits[r + 1];
     const int first_h = p.row_splits_h[r], last_h = p.row_splits_h[r + 1];
-    const TakenFlags<LDS_FLAGS> taken{s_bits, p.taken_h + first_h};
 
-    for (int q = first_h + tid; q < last_h; q += kBlock) {
-        p.is_alpha_h[q] = 0;
-        p.taken_h[q] = 0;
-        p.alpha_indices[q] = -1;
-    }
-    if (LDS_FLAGS)
-        for (int i = tid; i < flag_words; i += kBlock) s_bits[i] = 0;
-    uint32_t *const s_assigned = s_bits + flag_words;
-    if (ASSIGNED_BITS)
-        for (int i = tid; i < assigned_words; i += kBlock) s_assigned[i] = 0;
-    for (int i = first + tid; i < last; i += kBlock) {
-        p.assignment[i] = -1;
-        p.association[i] = -1;
-        if (!p.by_max_beta) p.best_dsq[i] = 10e20f;
-    }
+    int cur = launch == 0 ? first_h : p.cursor_at[(launch - 1) * p.num_rows + r];
+    int n_alpha = launch == 0 ? 0 : p.n_alpha_at[(launch - 1) * p.num_rows + r];
+    const int end = budget < 0 ? last_h : (int)min((long long)last_h, (long long)cur + budget);
+    int n_list = 0;  // points of this launch, all in s_list
+    int n_queue = 0;
+    int stopped_at = -1;
 
-    const int C = p.C, B = p.B;
-    int nb[kMaxBinDims];
-    int cells = 1;
+    for (;;) {
+        // ---- refill the queue with the open candidates of the next windows, in order ----
+        while (n_queue < window && cur < end) {
+            uint64_t open_mask[kFill];
 #pragma unroll
-    for (int d = 0; d < kMaxBinDims; ++d) {
-        nb[d] = d < B ? p.n_bins[d] : 1;
-        cells *= nb[d];
-    }
-    const int *bin_splits = p.bin_splits + (size_t)cells * r;
-    const float bw = p.bin_widths[0];
-    const float edge_slack = 1e-3f * bw;  // bins are cut by a rounded fp32 divide
-    __syncthreads();
-
-    int cursor = first_h;  // everything before it in the selection order is claimed
-    int window = -1;       // start of the 1024 order entries cached in registers
-    int my_q = -1;
-    bool my_selectable = false;
-    // what a claim step needs of this thread's entry, fetched with the window so that
-    // the step does not wait for a load that depends on the pick
-    float my_centre[kMaxDims], my_dist = 0.f;
-    int my_mask = 0, my_orig = -1;
-#pragma unroll
-    for (int c = 0; c < kMaxDims; ++c) my_centre[c] = 0.f;
-    int shower = 0;
-    while (cursor < last_h) {
-        // ---- next unclaimed hit in selection order ----
-        if (window < 0 || cursor >= window + kBlock) {
-            window = cursor;
-            const int pos = window + tid;
-            my_q = pos < last_h ? p.order_h[pos] : -1;
-            my_selectable = my_q >= 0 && (always_first(p.mask_h, p.n_vert_h, my_q) || p.beta_h[my_q] > -1.f);
-            if (my_q >= 0) {
-#pragma unroll
-                for (int c = 0; c < kMaxDims; ++c)
-                    if (c < C) my_centre[c] = p.ccoords_h[(size_t)my_q * C + c];
-                my_dist = p.dist_h[my_q];
-                my_mask = p.mask_h[my_q];
-                my_orig = p.orig_h[my_q];
+            for (int j = 0; j < kFill; ++j) {
+                const int pos = cur + j * kBlock + tid;
+                const bool open = pos < end && coherent_load(p.closed + pos) == 0;
+                open_mask[j] = __ballot(open);
+                if (lane == 0) s_fill[j][wave] = __popcll(open_mask[j]);
             }
-        }
-        const bool open = my_selectable && window + tid >= cursor && !taken.test(my_q - first_h);
-        const uint64_t b = __ballot(open);
-        if (lane == 0) s_first[wave] = b ? wave * kWave + (__ffsll((long long)b) - 1) : kBlock;
-        __syncthreads();
-        if (tid == 0) {
-            int best = kBlock;
-            for (int w = 0; w < kWavesPerBlock; ++w) best = min(best, s_first[w]);
-            s_pick = best;
-        }
-        __syncthreads();
-        const int pick = s_pick;
-        if (pick == kBlock) {  // nothing open in this window
-            cursor = window + kBlock;
             __syncthreads();
+            int at = n_queue, total = 0;
+            int mine[kFill];
+#pragma unroll
+            for (int j = 0; j < kFill; ++j) {
+#pragma unroll
+                for (int w = 0; w < kWavesPerBlock; ++w) {
+                    if (w == wave) mine[j] = at + total;
+                    total += s_fill[j][w];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kFill; ++j)
+                if ((open_mask[j] >> lane) & 1ull)
+                    s_queue[mine[j] + __popcll(open_mask[j] & ((1ull << lane) - 1ull))] = cur + j * kBlock + tid;
+            n_queue += total;
+            cur = (int)min((long long)end, (long long)cur + kFill * kBlock);
+            __syncthreads();
+        }
+        if (n_queue == 0) break;
+        const int take = min(n_queue, window);
+        if (n_list + take > capacity) {
+            // the list may not hold what this window adds
+            const int front = s_queue[0];
+            if (budget >= 0) {  // the grid-wide kernel after this launch takes the list over
+                stopped_at = front;
+                break;
+            }
+            // last launch: this workgroup closes what the list covers among the rest of
+            // its candidates itself, then starts a new list and walks on from the
+            // front of the queue
+            __syncthreads();
+            for (int i = front + tid; i < last_h; i += kBlock) {
+                if (coherent_load(p.closed + i)) continue;
+                const uint32_t *ri = p.cand + (size_t)i * cw;
+                if (ri[CMAX + 6]) continue;
+                float xi[CMAX];
+                int ki[kMaxBinDims];
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c) xi[c] = __uint_as_float(ri[c]);
+#pragma unroll
+                for (int d = 0; d < kMaxBinDims; ++d) ki[d] = (int)ri[CMAX + d];
+                for (int s = 0; s < n_list; ++s) {
+                    float dsq;
+                    if (covers<CMAX>(s_list + (size_t)s * aw, xi, false, -1, ki, dsq)) {
+                        p.closed[i] = 1;
+                        break;
+                    }
+                }
+            }
+            __threadfence();
+            __syncthreads();
+            n_list = 0;
+            n_queue = 0;
+            cur = front;
             continue;
         }
-        if (tid == pick) {
-            s_alpha = my_q;
-            s_alpha_dist = my_dist;
-            s_alpha_mask = my_mask;
-            s_alpha_orig = my_orig;
+
+        // ---- this thread's candidate ----
+        const bool valid = tid < take;
+        const int pos = valid ? s_queue[tid] : first_h;
+        float x[CMAX];
+        int k[kMaxBinDims];
+        uint32_t point[aw];
+        bool uncoverable = false;
+        {
+            const uint32_t *rec = p.cand + (size_t)pos * cw;
 #pragma unroll
-            for (int c = 0; c < kMaxDims; ++c) s_alpha_centre[c] = my_centre[c];
+            for (int c4 = 0; c4 < CMAX; c4 += 4) {
+                const float4 v = valid ? *reinterpret_cast<const float4 *>(rec + c4) : float4{0.f, 0.f, 0.f, 0.f};
+                x[c4] = v.x, x[c4 + 1] = v.y, x[c4 + 2] = v.z, x[c4 + 3] = v.w;
+            }
+#pragma unroll
+            for (int d = 0; d < kMaxBinDims; ++d) k[d] = valid ? (int)rec[CMAX + d] : INT_MIN;
+            uncoverable = valid && rec[CMAX + 6] != 0;
+#pragma unroll
+            for (int w4 = 0; w4 < aw; w4 += 4) {
+                const uint4 v = valid ? *reinterpret_cast<const uint4 *>(rec + CMAX + 8 + w4) : uint4{0u, 0u, 0u, 0u};
+                point[w4] = v.x, point[w4 + 1] = v.y, point[w4 + 2] = v.z, point[w4 + 3] = v.w;
+            }
+        }
+        bool open = valid;
+
+        // ---- points found earlier in this launch ----
+        if (__ballot(open && !uncoverable)) {
+            for (int s = 0; s < n_list; ++s) {
+                float dsq;
+                if (open && !uncoverable && covers<CMAX>(s_list + (size_t)s * aw, x, false, -1, k, dsq))
+                    open = false;
+                if ((s & 15) == 15 && !__ballot(open && !uncoverable)) break;
+            }
+        }
+        const uint64_t wave_open = __ballot(open);
+        if (lane == 0) {
+            s_open[wave] = wave_open != 0;
+            s_cnt[wave] = 0;
         }
         __syncthreads();
-        cursor = window + pick;
-        const int alpha = s_alpha;
 
-        // ---- claim step ----
-        float centre[kMaxDims];
+        // ---- the window, wave after wave ----
+        const int n_waves = (take + kWave - 1) / kWave;
+        for (int w = 0; w < n_waves; ++w) {
+            if (!s_open[w]) continue;  // uniform
+            if (wave == w) {
+                int cnt = 0;
+                while (true) {
+                    const uint64_t m = __ballot(open);
+                    if (!m) break;
+                    const int first = __builtin_ctzll(m);  // the next condensation point
+                    if (lane == first) {
+                        // for the later waves (LDS) and the grid-wide kernels (global memory)
+                        uint32_t *slot = s_list + (size_t)(n_list + cnt) * aw;
+                        const int rank = n_alpha + cnt;
+                        uint32_t *out = p.points + (size_t)(first_h + rank) * aw;
 #pragma unroll
-        for (int c = 0; c < kMaxDims; ++c) centre[c] = s_alpha_centre[c];
-        float radius = s_alpha_dist;
-        const float radius_sq = radius * radius;
-        const bool solitary = s_alpha_mask > 0;
-        if (solitary) radius = 0.f;
-        const float reach_sq = radius * radius * 1.0001f;  // pruning bound, slightly generous
-
-        int lo_bin[kMaxBinDims], width[kMaxBinDims];
-        int n_rows = 1;
-#pragma unroll
-        for (int d = 0; d < kMaxBinDims; ++d) {
-            lo_bin[d] = 0;
-            width[d] = 1;
-            if (d < B) {
-                const float lo = centre[d] - radius;
-                const float hi = centre[d] + radius;
-                float fl = floorf(lo / bw), fh = ceilf(hi / bw);
-                // keep the walk finite for absurd radii; the clamped range still
-                // covers every bin of the grid in this dimension
-                fl = fminf(fmaxf(fl, (float)(-nb[d])), (float)(2 * nb[d]));
-                fh = fminf(fmaxf(fh, (float)(-nb[d])), (float)(2 * nb[d]));
-                lo_bin[d] = (int)fl;
-                width[d] = (int)fh - (int)fl + 1;
-                if (d < B - 1) n_rows *= width[d];
-            }
-        }
-        const int run_lo = lo_bin[B - 1], run_hi = lo_bin[B - 1] + width[B - 1] - 1;
-        const int shower_orig = s_alpha_orig;
-
-        for (int row0 = 0; row0 < n_rows; row0 += kBlock) {
-            // -- every thread resolves one row of the box into a run of hits --
-            int start = 0, len = 0;
-            const int row = row0 + tid;
-            if (row < n_rows) {
-                // per-dimension indices are not range checked (only the flat index
-                // is), like the reference
-                long long base = 0;
-                int rem = row;
-                long long stride = nb[B - 1];
-                bool in_grid = true;
-                float gap_sq = 0.f;
-                for (int d = B - 2; d >= 0; --d) {
-                    const int k = lo_bin[d] + rem % width[d];
-                    rem /= width[d];
-                    base += (long long)k * stride;
-                    stride *= nb[d];
-                    in_grid = in_grid && k >= 0 && k < nb[d];
-                    // distance from the centre to the slab of bin k in this dimension
-                    const float below = (float)k * bw - edge_slack - centre[d];
-                    const float above = centre[d] - ((float)(k + 1) * bw + edge_slack);
-                    const float gap = fmaxf(0.f, fmaxf(below, above));
-                    gap_sq += gap * gap;
-                }
-                int k_lo = run_lo, k_hi = run_hi;
-                bool keep = true;
-                if (in_grid && !solitary) {
-                    // rows of real bins can be pruned against the sphere: no hit of a
-                    // skipped bin can pass d^2 <= radius^2 (slack covers fp rounding)
-                    const float rest = reach_sq - gap_sq;
-                    if (rest < 0.f) {
-                        keep = false;
-                    } else {
-                        const float half = sqrtf(rest) + edge_slack;
-                        k_lo = max(k_lo, (int)floorf((centre[B - 1] - half) / bw) - 1);
-                        k_hi = min(k_hi, (int)floorf((centre[B - 1] + half) / bw) + 1);
+                        for (int t = 0; t < aw; t += 4) {
+                            const uint4 v{point[t], point[t + 1], point[t + 2], point[t + 3]};
+                            *reinterpret_cast<uint4 *>(slot + t) = v;
+                            *reinterpret_cast<uint4 *>(out + t) = v;
+                        }
+                        const int q = (int)(point[CMAX + 1] & 0x7fffffffu);
+                        p.alpha_indices[first_h + rank] = (int)point[CMAX + 2];
+                        p.is_alpha_h[q] = 1;
+                        p.taken_h[q] = 1;
+                        open = false;
                     }
+                    // its lanes get the point from the lane's registers
+                    uint32_t head[CMAX + 2], box[kMaxBinDims];
+#pragma unroll
+                    for (int t = 0; t < CMAX + 2; ++t) head[t] = (uint32_t)__builtin_amdgcn_readlane((int)point[t], first);
+#pragma unroll
+                    for (int d = 0; d < kMaxBinDims; ++d)
+                        box[d] = (uint32_t)__builtin_amdgcn_readlane((int)point[CMAX + 4 + d], first);
+                    float dsq;
+                    if (open && !uncoverable && in_sphere<CMAX>(head, x, false, -1, dsq) && in_box(box, k)) open = false;
+                    ++cnt;
                 }
-                long long a = base + k_lo, z = base + k_hi;
-                if (a < 0) a = 0;
-                if (z > cells - 1) z = cells - 1;
-                if (keep && a <= z) {
-                    start = bin_splits[a];
-                    len = bin_splits[z + 1] - start;
-                }
+                if (lane == 0) s_cnt[w] = cnt;
             }
-            // -- exclusive scan of the run lengths over the workgroup --
-            const int incl = wave_inclusive_sum(len);
-            if (lane == kWave - 1) s_wave_tot[wave] = incl;
             __syncthreads();
-            int wave_off = 0, total = 0;
-#pragma unroll
-            for (int w = 0; w < kWavesPerBlock; ++w) {
-                const int t = s_wave_tot[w];
-                if (w < wave) wave_off += t;
-                total += t;
+            const int added = s_cnt[w];
+            if (wave > w && __ballot(open && !uncoverable)) {
+                for (int s = n_list; s < n_list + added; ++s) {
+                    float dsq;
+                    if (open && !uncoverable && covers<CMAX>(s_list + (size_t)s * aw, x, false, -1, k, dsq))
+                        open = false;
+                }
             }
-            s_row_off[tid] = wave_off + incl - len;
-            s_row_start[tid] = start;
-            if (tid == 0) s_row_off[kBlock] = total;
-            __syncthreads();
+            n_list += added;
+            n_alpha += added;
+        }
 
-            // -- all hits of all runs, kHitsPerThread per thread with their loads batched --
-            for (int h0 = 0; h0 < total; h0 += kBlock * kHitsPerThread) {
-                int hit[kHitsPerThread];
-                bool live[kHitsPerThread];
+        // ---- the rest of the queue moves to its front ----
+        const int rest = n_queue - take;
+        int moved[kFill];
 #pragma unroll
-                for (int k = 0; k < kHitsPerThread; ++k) {
-                    const int h = h0 + k * kBlock + tid;
-                    live[k] = h < total;
-                    // last row whose offset is <= h (empty rows share their successor's offset)
-                    int lo_r = 0;
+        for (int j = 0; j < kFill; ++j) moved[j] = j * kBlock + tid < rest ? s_queue[take + j * kBlock + tid] : 0;
+        __syncthreads();
 #pragma unroll
-                    for (int step = kBlock / 2; step > 0; step >>= 1) {
-                        const int probe = lo_r + step;
-                        if (s_row_off[probe] <= h) lo_r = probe;
-                    }
-                    hit[k] = live[k] ? s_row_start[lo_r] + (h - s_row_off[lo_r]) : first;
-                }
-                if (ASSIGNED_BITS) {
-#pragma unroll
-                    for (int k = 0; k < kHitsPerThread; ++k) {
-                        const int local = hit[k] - first;
-                        live[k] = live[k] && !((s_assigned[local >> 5] >> (local & 31)) & 1u);
-                    }
-                }
-                int asg[kHitsPerThread], filt[kHitsPerThread], msk[kHitsPerThread];
-                float dsq[kHitsPerThread];
-#pragma unroll
-                for (int k = 0; k < kHitsPerThread; ++k) {
-                    const int i = hit[k];
-                    asg[k] = -1;
-                    filt[k] = -1;
-                    msk[k] = 1;
-                    dsq[k] = 0.f;
-                    if (ASSIGNED_BITS && !live[k]) continue;
-                    if (!ASSIGNED_BITS && p.by_max_beta) asg[k] = p.assignment[i];
-                    filt[k] = p.to_filtered[i];
-                    msk[k] = p.mask[i];
-                    float acc = 0.f;
-                    for (int c = 0; c < C; ++c) {
-                        const float t = centre[c] - p.ccoords[(size_t)i * C + c];
-                        acc = acc + t * t;
-                    }
-                    dsq[k] = acc;
-                }
-#pragma unroll
-                for (int k = 0; k < kHitsPerThread; ++k) {
-                    if (!live[k]) continue;
-                    const int i = hit[k];
-                    if (p.by_max_beta && asg[k] != -1) continue;
-                    const bool inside = (dsq[k] <= radius_sq && !solitary && msk[k] == 0) || (solitary && filt[k] == alpha);
-                    if (!inside) continue;
-                    if (!p.by_max_beta) {
-                        const float lhs = p.best_dsq[i] * radius_sq;
-                        if (!(lhs >= dsq[k])) continue;
-                        p.best_dsq[i] = dsq[k];
-                    }
-                    p.assignment[i] = shower;
-                    p.association[i] = shower_orig;
-                    if (ASSIGNED_BITS) atomicOr(&s_assigned[(i - first) >> 5], 1u << ((i - first) & 31));
-                    if (filt[k] != -1) taken.set(filt[k] - first_h);
-                }
-            }
-            __syncthreads();  // LDS row tables are reused by the next tile / condensate
-        }
-        if (tid == 0) {
-            p.is_alpha_h[alpha] = 1;
-            taken.set(alpha - first_h);
-            p.alpha_indices[first_h + shower] = shower_orig;
-        }
-        ++shower;
-        ++cursor;
-        __syncthreads();  // claims visible to the whole workgroup before the next pick
+        for (int j = 0; j < kFill; ++j)
+            if (j * kBlock + tid < rest) s_queue[j * kBlock + tid] = moved[j];
+        n_queue = rest;
+        __syncthreads();
     }
-    if (tid == 0) p.event_count[r] = shower;
+    if (tid == 0) {
+        p.cursor_at[launch * p.num_rows + r] = stopped_at >= 0 ? stopped_at : end;
+        p.n_alpha_at[launch * p.num_rows + r] = n_alpha;
+    }
+}
+
+// Grid-wide pass over items of all events against the condensation points of
+// their event, a tile of points in LDS at a time.
+//   MODE 0: items = candidates from the event's cursor on, points = those the last
+//           launch of the event kernel added; closes what they cover
+//   MODE 1: items = all hits, all points; first point that covers the hit (max-beta)
+//   MODE 2: items = all hits, all points; the reference's running comparison (min-distance)
+template <int CMAX, int MODE>
+__global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams p, int launch) {
+    constexpr int aw = alpha_words(CMAX), cw = cand_words(CMAX);
+    __shared__ __align__(16) uint32_t s_tile[kTile * aw];
+    const int tid = threadIdx.x;
+    const int C = p.C, B = p.B;
+    const int n_items = MODE == 0 ? p.n_vert_h : p.n_vert;
+    const int *splits = MODE == 0 ? p.row_splits_h : p.row_splits;
+    const int i_first = blockIdx.x * kScanBlock;
+    const int i = i_first + tid;
+    const bool valid = i < n_items;
+    const int ev_lo = event_of(splits, p.num_rows, i_first);
+    const int ev_hi = event_of(splits, p.num_rows, min(i_first + kScanBlock, n_items) - 1);
+    const int my_ev = valid ? event_of(splits, p.num_rows, i) : -1;
+
+    // ---- this thread's item ----
+    float x[CMAX];
+    int k[kMaxBinDims];
+    bool alive = valid, uncoverable = false;
+    int self_q = -1;
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) x[c] = 0.f;
+#pragma unroll
+    for (int d = 0; d < kMaxBinDims; ++d) k[d] = INT_MIN;
+    if (MODE == 0) {
+        if (valid) {
+            const uint32_t *rec = p.cand + (size_t)i * cw;
+            alive = p.closed[i] == 0 && i >= p.cursor_at[launch * p.num_rows + my_ev] && rec[CMAX + 6] == 0;
+            if (alive) {
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c) x[c] = __uint_as_float(rec[c]);
+#pragma unroll
+                for (int d = 0; d < kMaxBinDims; ++d) k[d] = (int)rec[CMAX + d];
+            }
+        }
+    } else if (valid) {
+        Grid g;
+        g.load(p);
+#pragma unroll
+        for (int c = 0; c < CMAX; ++c)
+            if (c < C) x[c] = p.ccoords[(size_t)i * C + c];
+        uncoverable = p.mask[i] != 0;
+        self_q = p.to_filtered[i];
+        g.split(p.hit_bin[i], B, k);
+    }
+
+    int shower = -1, asso = -1;
+    float best = 10e20f;
+
+    for (int ev = ev_lo; ev <= ev_hi; ++ev) {
+        const int first_h = p.row_splits_h[ev];
+        const int rank_lo = (MODE == 0 && launch > 0) ? p.n_alpha_at[(launch - 1) * p.num_rows + ev] : 0;
+        const int rank_hi = p.n_alpha_at[launch * p.num_rows + ev];
+        bool mine = alive && my_ev == ev;
+        for (int base = rank_lo; base < rank_hi; base += kTile) {
+            if (!__syncthreads_or(mine)) break;  // also: everyone is done with the previous tile
+            const int n_tile = min(kTile, rank_hi - base);
+            const uint4 *src = reinterpret_cast<const uint4 *>(p.points + (size_t)(first_h + base) * aw);
+            for (int e = tid; e < n_tile * (aw / 4); e += kScanBlock) reinterpret_cast<uint4 *>(s_tile)[e] = src[e];
+            __syncthreads();
+            if (mine) {
+                for (int t = 0; t < n_tile; ++t) {
+                    const uint32_t *a = s_tile + (size_t)t * aw;
+                    float dsq;
+                    if (!covers<CMAX>(a, x, uncoverable, self_q, k, dsq)) continue;
+                    if (MODE == 2) {
+                        const float lhs = best * __uint_as_float(a[CMAX]);
+                        if (!(lhs >= dsq)) continue;
+                        best = dsq;
+                    }
+                    shower = base + t;
+                    asso = (int)a[CMAX + 2];
+                    if (MODE != 2) {
+                        mine = alive = false;
+                        break;
+                    }
+                }
+            }
+        }
+    }
+    if (!valid) return;
+    if (MODE == 0) {
+        if (shower >= 0) p.closed[i] = 1;
+    } else {
+        p.assignment[i] = shower;
+        p.association[i] = asso;
+        if (MODE == 2) p.best_dsq[i] = best;
+        if (shower >= 0 && self_q >= 0 && self_q < p.n_vert_h) p.taken_h[self_q] = 1;
+    }
 }
 
 __global__ void cumulative_counts_kernel(const int *__restrict__ event_count, int num_rows,
@@ -416,6 +622,83 @@ int selection_key_bits(int num_rows) {
     return 34 + bits;
 }
 
+struct Workspace {
+    uint64_t *keys, *keys_sorted;
+    int *values, *order, *pos_h, *hit_bin, *closed, *cursor_at, *n_alpha_at;
+    uint32_t *cand, *points;
+    size_t used;
+};
+
+Workspace carve_workspace(void *base, int n_vert, int n_vert_h, int num_rows) {
+    const size_t nh = std::max(n_vert_h, 1), n = std::max(n_vert, 1), rows = std::max(num_rows, 1);
+    Carver carve(base);
+    Workspace w;
+    w.keys = carve.take<uint64_t>(nh);
+    w.keys_sorted = carve.take<uint64_t>(nh);
+    w.values = carve.take<int>(nh);
+    w.order = carve.take<int>(nh);
+    w.pos_h = carve.take<int>(nh);
+    w.hit_bin = carve.take<int>(n);
+    w.closed = carve.take<int>(nh);
+    w.points = carve.take<uint32_t>(nh * (size_t)alpha_words(kMaxDims));
+    w.cursor_at = carve.take<int>(kMaxLaunches * rows);
+    w.n_alpha_at = carve.take<int>(kMaxLaunches * rows);
+    w.cand = carve.take<uint32_t>(nh * (size_t)cand_words(kMaxDims));
+    w.used = carve.used;
+    return w;
+}
+
+// returns through `last_launch` which launch of the event kernel holds the final counts
+template <int CMAX>
+int run(const CondParams &p, hipStream_t s, int &last_launch) {
+    int rc;
+    if (p.n_vert > 0) {
+        hit_prepare_kernel<<<ceil_div(p.n_vert, 256), 256, 0, s>>>(p);
+        if ((rc = check_launch("hit_prepare"))) return rc;
+    }
+    if (p.n_vert_h > 0) {
+        candidate_records_kernel<CMAX><<<ceil_div(p.n_vert_h, 256), 256, 0, s>>>(p);
+        if ((rc = check_launch("candidate_records"))) return rc;
+    }
+    // the event kernel's list of condensation points lives in dynamic LDS; more than
+    // the default has to be granted per kernel
+    const size_t point_bytes = (size_t)alpha_words(CMAX) * sizeof(uint32_t);
+    size_t list_bytes = 40 * 1024;
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&condensate_event_kernel<CMAX>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) == hipSuccess)
+        list_bytes = 128 * 1024;
+    (void)hipGetLastError();  // a refused grant is not an error of this call
+    const int capacity = (int)(list_bytes / point_bytes);
+    const int window = std::min(kBlock, capacity / 2 / kWave * kWave);
+    // geometric shares of the sorted candidates, the last launch takes what is left;
+    // n_vert_h bounds every event
+    int budgets[kMaxLaunches];
+    int n_launches = 0;
+    long long reach = 0;
+    for (int share = 1024; n_launches < kMaxLaunches - 1 && reach + share < p.n_vert_h; share *= 4) {
+        budgets[n_launches++] = share;
+        reach += share;
+    }
+    budgets[n_launches++] = -1;
+    for (int l = 0; l < n_launches; ++l) {
+        condensate_event_kernel<CMAX><<<p.num_rows, kBlock, list_bytes, s>>>(p, l, budgets[l], window, capacity);
+        if ((rc = check_launch("condensate_event_kernel"))) return rc;
+        if (l + 1 < n_launches && p.n_vert_h > 0) {
+            cover_scan_kernel<CMAX, 0><<<ceil_div(p.n_vert_h, kScanBlock), kScanBlock, 0, s>>>(p, l);
+            if ((rc = check_launch("cover_scan_kernel (candidates)"))) return rc;
+        }
+    }
+    if (p.n_vert > 0) {
+        if (p.by_max_beta)
+            cover_scan_kernel<CMAX, 1><<<ceil_div(p.n_vert, kScanBlock), kScanBlock, 0, s>>>(p, n_launches - 1);
+        else
+            cover_scan_kernel<CMAX, 2><<<ceil_div(p.n_vert, kScanBlock), kScanBlock, 0, s>>>(p, n_launches - 1);
+        if ((rc = check_launch("cover_scan_kernel (hits)"))) return rc;
+    }
+    last_launch = n_launches - 1;
+    return HGC_OK;
+}
+
 }  // namespace
 }  // namespace hgc
 
@@ -424,14 +707,12 @@ using namespace hgc;
 extern "C" {
 
 size_t hgc_binned_assign_to_condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows) {
-    (void)n_vert;
     const size_t nh = std::max(n_vert_h, 1);
     size_t temp = 0;
     (void)rocprim::radix_sort_pairs(nullptr, temp, (const uint64_t *)nullptr, (uint64_t *)nullptr,
                                     (const int *)nullptr, (int *)nullptr, nh, 0,
                                     selection_key_bits(std::max(num_rows, 1)), (hipStream_t) nullptr);
-    return align_up(temp) + 2 * align_up(nh * sizeof(uint64_t)) + 2 * align_up(nh * sizeof(int)) +
-           align_up((size_t)std::max(num_rows, 1) * sizeof(int));
+    return align_up(temp) + carve_workspace(nullptr, n_vert, n_vert_h, num_rows).used;
 }
 
 int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,
@@ -464,79 +745,61 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int
                         d_high_assigned_status_h && d_original_indices_h && d_alpha_indices,
                     "null pointer");
 
-    const size_t nh = std::max(n_vert_h, 1);
-    Carver carve(workspace);
-    uint64_t *keys = carve.take<uint64_t>(nh);
-    uint64_t *keys_sorted = carve.take<uint64_t>(nh);
-    int *values = carve.take<int>(nh);
-    int *order = carve.take<int>(nh);
-    int *event_count = carve.take<int>(std::max(num_rows, 1));
-    void *temp = carve.base + carve.used;
-    size_t temp_bytes = workspace_bytes - carve.used;
+    const Workspace w = carve_workspace(workspace, n_vert, n_vert_h, num_rows);
+    void *temp = static_cast<char *>(workspace) + w.used;
+    size_t temp_bytes = workspace_bytes - w.used;
 
-    if (n_vert_h > 0) {
-        selection_keys_kernel<<<ceil_div(n_vert_h, 256), 256, 0, s>>>(d_beta_h, d_no_condensation_mask_h,
-                                                                      d_row_splits_h, num_rows, n_vert_h, keys, values);
-        int rc = check_launch("selection_keys");
-        if (rc) return rc;
-        HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys, keys_sorted, values, order, (size_t)n_vert_h, 0,
-                                          selection_key_bits(num_rows), s));
-    }
+    CondParams p;
+    p.C = dimensions;
+    p.B = dimensions_binning;
+    p.taken_h = d_condensates_assigned_h;
+    p.ccoords_h = d_ccoords_h;
+    p.dist_h = d_dist_h;
+    p.beta_h = d_beta_h;
+    p.mask_h = d_no_condensation_mask_h;
+    p.is_alpha_h = d_high_assigned_status_h;
+    p.orig_h = d_original_indices_h;
+    p.row_splits_h = d_row_splits_h;
+    p.ccoords = d_ccoords;
+    p.mask = d_no_condensation_mask;
+    p.to_filtered = d_indices_to_filtered;
+    p.best_dsq = d_assignment_min_distance;
+    p.assignment = d_assignment;
+    p.association = d_association;
+    p.alpha_indices = d_alpha_indices;
+    p.bin_splits = d_bin_splits;
+    p.n_bins = d_n_bins;
+    p.bin_widths = d_bin_widths;
+    p.row_splits = d_row_splits;
+    p.num_rows = num_rows;
+    p.by_max_beta = assign_by_max_beta;
+    p.n_vert = n_vert;
+    p.n_vert_h = n_vert_h;
+    p.order_h = w.order;
+    p.pos_h = w.pos_h;
+    p.hit_bin = w.hit_bin;
+    p.cand = w.cand;
+    p.closed = w.closed;
+    p.points = w.points;
+    p.cursor_at = w.cursor_at;
+    p.n_alpha_at = w.n_alpha_at;
+
+    int last_launch = 0;
     if (num_rows > 0) {
-        CondParams p;
-        p.C = dimensions;
-        p.B = dimensions_binning;
-        p.taken_h = d_condensates_assigned_h;
-        p.ccoords_h = d_ccoords_h;
-        p.dist_h = d_dist_h;
-        p.beta_h = d_beta_h;
-        p.mask_h = d_no_condensation_mask_h;
-        p.is_alpha_h = d_high_assigned_status_h;
-        p.orig_h = d_original_indices_h;
-        p.row_splits_h = d_row_splits_h;
-        p.ccoords = d_ccoords;
-        p.mask = d_no_condensation_mask;
-        p.to_filtered = d_indices_to_filtered;
-        p.best_dsq = d_assignment_min_distance;
-        p.assignment = d_assignment;
-        p.association = d_association;
-        p.alpha_indices = d_alpha_indices;
-        p.bin_splits = d_bin_splits;
-        p.n_bins = d_n_bins;
-        p.bin_widths = d_bin_widths;
-        p.row_splits = d_row_splits;
-        p.num_rows = num_rows;
-        p.by_max_beta = assign_by_max_beta;
-        p.n_vert = n_vert;
-        p.n_vert_h = n_vert_h;
-        p.order_h = order;
-        p.event_count = event_count;
-        // One claimed-flag bit per high-beta hit of an event and, in max-beta mode, one
-        // assigned bit per hit live in LDS when they fit (n_vert_h and n_vert bound
-        // every event; the event sizes themselves are device data).
-        const int flag_words = ceil_div(std::max(n_vert_h, 1), 32);
-        const int assigned_words = ceil_div(std::max(n_vert, 1), 32);
-        constexpr size_t kDynamicLdsLimit = 144 * 1024;  // of 160 KB; the kernel has ~9 KB of static tables
-        const size_t flag_bytes = (size_t)flag_words * 4, both_bytes = flag_bytes + (size_t)assigned_words * 4;
-        // more than the default 64 KB of dynamic LDS has to be granted per kernel; without
-        // the grant the variant without assigned bits runs
-        const bool with_assigned_bits =
-            assign_by_max_beta && both_bytes <= kDynamicLdsLimit &&
-            (both_bytes <= 48 * 1024 ||
-             hipFuncSetAttribute(reinterpret_cast<const void *>(&condensate_event_kernel<true, true>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynamicLdsLimit) == hipSuccess);
-        (void)hipGetLastError();  // a refused grant is not an error of this call
-        if (with_assigned_bits) {
-            condensate_event_kernel<true, true><<<num_rows, kBlock, both_bytes, s>>>(p, flag_words, assigned_words);
-        } else if (flag_bytes <= 48 * 1024) {
-            condensate_event_kernel<true, false><<<num_rows, kBlock, flag_bytes, s>>>(p, flag_words, 0);
-        } else {
-            condensate_event_kernel<false, false><<<num_rows, kBlock, 0, s>>>(p, 0, 0);
+        if (n_vert_h > 0) {
+            selection_keys_kernel<<<ceil_div(n_vert_h, 256), 256, 0, s>>>(p, w.keys, w.values);
+            int rc = check_launch("selection_keys");
+            if (rc) return rc;
+            HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, w.keys, w.keys_sorted, w.values, w.order,
+                                              (size_t)n_vert_h, 0, selection_key_bits(num_rows), s));
         }
-        int rc = check_launch("condensate_event_kernel");
+        const int rc = dimensions <= 4   ? run<4>(p, s, last_launch)
+                       : dimensions <= 8 ? run<8>(p, s, last_launch)
+                                         : run<kMaxDims>(p, s, last_launch);
         if (rc) return rc;
     }
-    cumulative_counts_kernel<<<1, 64, 0, s>>>(event_count, num_rows, d_n_condensates, d_error);
+    cumulative_counts_kernel<<<1, 64, 0, s>>>(w.n_alpha_at + (size_t)last_launch * num_rows, num_rows,
+                                              d_n_condensates, d_error);
     return check_launch("cumulative_counts");
 }
 

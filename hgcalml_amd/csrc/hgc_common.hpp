@@ -176,6 +176,14 @@ __device__ __forceinline__ uint32_t wave_inclusive_max(uint32_t v) {
     return v;
 }
 
+// LDS traffic of one wave stays in program order; this keeps the compiler from
+// moving the wave's own accesses across the point where lanes exchange data.
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 #endif  // __HIPCC__
 
 }  // namespace hgc

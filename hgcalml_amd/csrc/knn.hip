@@ -246,14 +246,6 @@ constexpr int kMarkCap = 2048;
 // against 0.78 ms with 4 and 0.95 ms with 8).
 constexpr int kQueriesPerBlock = 1;
 
-// LDS traffic of one wave stays in program order; this keeps the compiler from
-// moving the wave's own accesses across the point where lanes exchange data.
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 // q = x / w, r = x % w for 0 <= x < 2^23 and small w, without an integer divide:
 // the float quotient is off by at most one, the remainder says which way
 __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, int &r) {
