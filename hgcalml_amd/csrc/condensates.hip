@@ -82,6 +82,7 @@ struct CondParams {
     const float *bin_widths;
     const int *row_splits;
     int num_rows, by_max_beta, n_vert, n_vert_h;
+    int rows_aligned;  // ccoords and ccoords_h start on 16-byte boundaries
     // workspace
     const int *order_h;  // high-beta hits in selection order, grouped by event
     int *pos_h;          // [n_vert_h] position of a high-beta hit among all hits, -1 unknown
@@ -205,20 +206,30 @@ template <int CMAX>
 __global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams p) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= p.n_vert_h) return;
+    constexpr int cw = cand_words(CMAX);
     const int C = p.C, B = p.B;
     Grid g;
     g.load(p);
     const int q = p.order_h[i];
     const int at = p.pos_h[q];
-    uint32_t *rec = p.cand + (size_t)i * cand_words(CMAX);
+    uint32_t rec[cw];
     uint32_t *point = rec + CMAX + 8;
     float centre[CMAX];
+    if (CMAX == 4 && C == 4 && p.rows_aligned) {  // one 16-byte load per row
+        const float4 h = at >= 0 ? reinterpret_cast<const float4 *>(p.ccoords)[at] : float4{0.f, 0.f, 0.f, 0.f};
+        const float4 a = reinterpret_cast<const float4 *>(p.ccoords_h)[q];
+        rec[0] = __float_as_uint(h.x), rec[1] = __float_as_uint(h.y), rec[2] = __float_as_uint(h.z),
+        rec[3] = __float_as_uint(h.w);
+        centre[0] = a.x, centre[1] = a.y, centre[2] = a.z, centre[3] = a.w;
+    } else {
 #pragma unroll
-    for (int c = 0; c < CMAX; ++c) {
-        centre[c] = c < C ? p.ccoords_h[(size_t)q * C + c] : 0.f;
-        rec[c] = (c < C && at >= 0) ? __float_as_uint(p.ccoords[(size_t)at * C + c]) : 0u;
-        point[c] = __float_as_uint(centre[c]);
+        for (int c = 0; c < CMAX; ++c) {
+            centre[c] = c < C ? p.ccoords_h[(size_t)q * C + c] : 0.f;
+            rec[c] = (c < C && at >= 0) ? __float_as_uint(p.ccoords[(size_t)at * C + c]) : 0u;
+        }
     }
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) point[c] = __float_as_uint(centre[c]);
     int k[kMaxBinDims];
     g.split(at >= 0 ? p.hit_bin[at] : INT_MIN, B, k);
 #pragma unroll
@@ -246,7 +257,11 @@ __global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams
         }
         point[CMAX + 4 + d] = ((uint32_t)lo & 0xffffu) | ((uint32_t)hi << 16);
     }
+#pragma unroll
     for (int w = CMAX + 4 + kMaxBinDims; w < alpha_words(CMAX); ++w) point[w] = 0u;
+    uint4 *out = reinterpret_cast<uint4 *>(p.cand + (size_t)i * cw);
+#pragma unroll
+    for (int w = 0; w < cw; w += 4) out[w / 4] = uint4{rec[w], rec[w + 1], rec[w + 2], rec[w + 3]};
     const bool selectable = always_first(p.mask_h, p.n_vert_h, q) || p.beta_h[q] > -1.f;
     p.closed[i] = selectable ? 0 : 1;
 }
@@ -269,11 +284,11 @@ __device__ __forceinline__ bool in_sphere(const uint32_t (&a)[CMAX + 2], const f
 
 // ... and the hit's bin against the point's box of bins
 __device__ __forceinline__ bool in_box(const uint32_t (&box)[kMaxBinDims], const int (&k)[kMaxBinDims]) {
-    bool inside = true;
+    int inside = 1;  // no short cuts: twelve compares cost less than a chain of branches
 #pragma unroll
     for (int d = 0; d < kMaxBinDims; ++d)
-        inside = inside && k[d] >= (int)(int16_t)(box[d] & 0xffffu) && k[d] <= ((int)box[d] >> 16);
-    return inside;
+        inside &= (int)(k[d] >= (int)(int16_t)(box[d] & 0xffffu)) & (int)(k[d] <= ((int)box[d] >> 16));
+    return inside != 0;
 }
 
 // the whole test against a point in LDS (16-byte aligned); the box is only read for hits inside the sphere
@@ -442,28 +457,16 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
             if (!s_open[w]) continue;  // uniform
             if (wave == w) {
                 int cnt = 0;
+                bool chosen = false;
                 while (true) {
                     const uint64_t m = __ballot(open);
                     if (!m) break;
                     const int first = __builtin_ctzll(m);  // the next condensation point
                     if (lane == first) {
-                        // for the later waves (LDS) and the grid-wide kernels (global memory)
-                        uint32_t *slot = s_list + (size_t)(n_list + cnt) * aw;
-                        const int rank = n_alpha + cnt;
-                        uint32_t *out = p.points + (size_t)(first_h + rank) * aw;
-#pragma unroll
-                        for (int t = 0; t < aw; t += 4) {
-                            const uint4 v{point[t], point[t + 1], point[t + 2], point[t + 3]};
-                            *reinterpret_cast<uint4 *>(slot + t) = v;
-                            *reinterpret_cast<uint4 *>(out + t) = v;
-                        }
-                        const int q = (int)(point[CMAX + 1] & 0x7fffffffu);
-                        p.alpha_indices[first_h + rank] = (int)point[CMAX + 2];
-                        p.is_alpha_h[q] = 1;
-                        p.taken_h[q] = 1;
+                        chosen = true;
                         open = false;
                     }
-                    // its lanes get the point from the lane's registers
+                    // the other lanes get the point from that lane's registers
                     uint32_t head[CMAX + 2], box[kMaxBinDims];
 #pragma unroll
                     for (int t = 0; t < CMAX + 2; ++t) head[t] = (uint32_t)__builtin_amdgcn_readlane((int)point[t], first);
@@ -473,6 +476,24 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
                     float dsq;
                     if (open && !uncoverable && in_sphere<CMAX>(head, x, false, -1, dsq) && in_box(box, k)) open = false;
                     ++cnt;
+                }
+                const uint64_t chosen_mask = __ballot(chosen);
+                if (chosen) {
+                    // for the later waves (LDS) and the grid-wide kernels (global memory)
+                    const int nth = __popcll(chosen_mask & ((1ull << lane) - 1ull));
+                    uint32_t *slot = s_list + (size_t)(n_list + nth) * aw;
+                    const int rank = n_alpha + nth;
+                    uint32_t *out = p.points + (size_t)(first_h + rank) * aw;
+#pragma unroll
+                    for (int t = 0; t < aw; t += 4) {
+                        const uint4 v{point[t], point[t + 1], point[t + 2], point[t + 3]};
+                        *reinterpret_cast<uint4 *>(slot + t) = v;
+                        *reinterpret_cast<uint4 *>(out + t) = v;
+                    }
+                    const int q = (int)(point[CMAX + 1] & 0x7fffffffu);
+                    p.alpha_indices[first_h + rank] = (int)point[CMAX + 2];
+                    p.is_alpha_h[q] = 1;
+                    p.taken_h[q] = 1;
                 }
                 if (lane == 0) s_cnt[w] = cnt;
             }
@@ -517,6 +538,11 @@ template <int CMAX, int MODE>
 __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams p, int launch) {
     constexpr int aw = alpha_words(CMAX), cw = cand_words(CMAX);
     __shared__ __align__(16) uint32_t s_tile[kTile * aw];
+    // the same tile by component, for four sphere tests at a time: centres, radius^2 (-1 for
+    // a point that claims only itself), and q | 1 << 31 of such points (0 for the others)
+    __shared__ __align__(16) float s_centre[CMAX][kTile];
+    __shared__ __align__(16) float s_rsq[kTile];
+    __shared__ __align__(16) uint32_t s_self[kTile];
     const int tid = threadIdx.x;
     const int C = p.C, B = p.B;
     const int n_items = MODE == 0 ? p.n_vert_h : p.n_vert;
@@ -559,6 +585,13 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
         g.split(p.hit_bin[i], B, k);
     }
 
+    // sphere tests run on a copy whose first coordinate is NaN for a masked hit: no sphere claims it
+    float xs[CMAX];
+#pragma unroll
+    for (int c = 0; c < CMAX; ++c) xs[c] = x[c];
+    if (uncoverable) xs[0] = __uint_as_float(0x7fc00000u);
+    const uint32_t self_key = self_q >= 0 ? ((uint32_t)self_q | 0x80000000u) : 0xffffffffu;
+
     int shower = -1, asso = -1;
     float best = 10e20f;
 
@@ -573,22 +606,62 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
             const uint4 *src = reinterpret_cast<const uint4 *>(p.points + (size_t)(first_h + base) * aw);
             for (int e = tid; e < n_tile * (aw / 4); e += kScanBlock) reinterpret_cast<uint4 *>(s_tile)[e] = src[e];
             __syncthreads();
+            bool solitary_here = false;
+            if (tid < kTile) {
+                const uint32_t *a = s_tile + (size_t)tid * aw;
+                const bool real = tid < n_tile;
+                const uint32_t solq = real ? a[CMAX + 1] : 0u;
+                solitary_here = solq >> 31;
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c) s_centre[c][tid] = real ? __uint_as_float(a[c]) : 0.f;
+                s_rsq[tid] = (real && !solitary_here) ? __uint_as_float(a[CMAX]) : -1.f;
+                s_self[tid] = solitary_here ? solq : 0u;
+            }
+            const bool any_solitary = __syncthreads_or(solitary_here);
             if (mine) {
-                for (int t = 0; t < n_tile; ++t) {
-                    const uint32_t *a = s_tile + (size_t)t * aw;
-                    float dsq;
-                    if (!covers<CMAX>(a, x, uncoverable, self_q, k, dsq)) continue;
-                    if (MODE == 2) {
-                        const float lhs = best * __uint_as_float(a[CMAX]);
-                        if (!(lhs >= dsq)) continue;
-                        best = dsq;
+                for (int t4 = 0; t4 < n_tile; t4 += 4) {
+                    // four sphere tests, each the reference's serial sum over the coordinates
+                    float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+                    for (int c = 0; c < CMAX; ++c) {
+                        const float4 cc = *reinterpret_cast<const float4 *>(&s_centre[c][t4]);
+                        float t = cc.x - xs[c];
+                        d0 = d0 + t * t;
+                        t = cc.y - xs[c];
+                        d1 = d1 + t * t;
+                        t = cc.z - xs[c];
+                        d2 = d2 + t * t;
+                        t = cc.w - xs[c];
+                        d3 = d3 + t * t;
                     }
-                    shower = base + t;
-                    asso = (int)a[CMAX + 2];
-                    if (MODE != 2) {
-                        mine = alive = false;
-                        break;
+                    const float4 rr = *reinterpret_cast<const float4 *>(&s_rsq[t4]);
+                    uint32_t hits = (d0 <= rr.x ? 1u : 0u) | (d1 <= rr.y ? 2u : 0u) | (d2 <= rr.z ? 4u : 0u) |
+                                    (d3 <= rr.w ? 8u : 0u);
+                    if (any_solitary) {
+                        const uint4 sk = *reinterpret_cast<const uint4 *>(&s_self[t4]);
+                        hits |= (sk.x == self_key ? 1u : 0u) | (sk.y == self_key ? 2u : 0u) |
+                                (sk.z == self_key ? 4u : 0u) | (sk.w == self_key ? 8u : 0u);
                     }
+                    if (!hits) continue;
+                    // the complete test for those, in order
+                    for (int j = 0; j < 4; ++j) {
+                        if (!((hits >> j) & 1u)) continue;
+                        const uint32_t *a = s_tile + (size_t)(t4 + j) * aw;
+                        float dsq;
+                        if (!covers<CMAX>(a, x, uncoverable, self_q, k, dsq)) continue;
+                        if (MODE == 2) {
+                            const float lhs = best * __uint_as_float(a[CMAX]);
+                            if (!(lhs >= dsq)) continue;
+                            best = dsq;
+                        }
+                        shower = base + t4 + j;
+                        asso = (int)a[CMAX + 2];
+                        if (MODE != 2) {
+                            mine = alive = false;
+                            break;
+                        }
+                    }
+                    if (!mine) break;
                 }
             }
         }
@@ -775,6 +848,7 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int
     p.by_max_beta = assign_by_max_beta;
     p.n_vert = n_vert;
     p.n_vert_h = n_vert_h;
+    p.rows_aligned = ((reinterpret_cast<uintptr_t>(d_ccoords) | reinterpret_cast<uintptr_t>(d_ccoords_h)) & 15u) == 0;
     p.order_h = w.order;
     p.pos_h = w.pos_h;
     p.hit_bin = w.hit_bin;
