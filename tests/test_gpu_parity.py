@@ -876,10 +876,22 @@ def test_condensates_cfg5_full(oracle, by_max_beta):
     run_condensates(oracle, workloads.cfg5(), by_max_beta)
 
 
+@pytest.mark.parametrize("radius", [0.004, 0.03])
+@pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensates_thousands_of_points_per_event(oracle, by_max_beta, radius):
+    """small radii: most high-beta hits become condensation points, more per launch of
+    the event kernel than its LDS list holds (the launch ends early, the last one
+    closes the rest of its candidates itself and starts a new list)"""
+    cfg = workloads.cfg5(scale=0.5, n_events=2)
+    cfg["dist"] = np.full_like(cfg["dist"], radius)
+    got = run_condensates(oracle, cfg, by_max_beta)
+    per_event = np.diff(got[4].cpu().numpy())
+    assert per_event.min() > 15000
+
+
 @pytest.mark.parametrize("by_max_beta", [True, False])
 def test_condensates_more_hits_than_the_lds_flags_hold(oracle, by_max_beta):
-    """1.3 M hits with ~0.9 M above the beta threshold: neither the assigned bits nor
-    the claimed flags fit into LDS, the kernel keeps its flags in global memory"""
+    """1.3 M hits with ~0.9 M above the beta threshold in 4 events"""
     cfg = workloads.cfg5(scale=5.2, n_events=4)
     cfg["beta_threshold"] = 0.02
     assert (cfg["betas"] > 0.02).sum() > 48 * 1024 * 8
