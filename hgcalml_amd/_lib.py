@@ -46,6 +46,8 @@ _SIGNATURES = {
     "hgc_probe_row_gather": (_c_int, [_ptr] * 3 + [_c_int] * 3 + [_ptr]),
     "hgc_binned_assign_to_condensates_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),
     "hgc_binned_assign_to_condensates": (_c_int, [_c_int, _c_int] + [_ptr] * 21 + [_c_int] * 4 + [_ptr, _ptr, _c_size, _ptr]),
+    "hgc_build_and_assign_condensates_workspace_bytes": (_c_size, [_c_int] * 5),
+    "hgc_build_and_assign_condensates": (_c_int, [_ptr] * 5 + [_c_int] * 3 + [_c_float, _c_float] + [_c_int] * 3 + [_ptr] * 6 + [_c_size, _ptr]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

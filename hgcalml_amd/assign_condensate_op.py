@@ -6,7 +6,6 @@ import math
 import torch
 
 from . import ops
-from .bin_by_coordinates_op import BinByCoordinates
 
 
 def merge_noise_as_indiv_cp(assignment, asso_idx, alpha_idx, is_cond, n_condensates, row_splits):
@@ -63,60 +62,13 @@ def BuildAndAssignCondensatesBinned(ccoords, betas, dist, row_splits, beta_thres
     assert 0. <= beta_threshold <= 1.
     assert distance_threshold > 0.
     ccoords = ccoords.to(torch.float32)
-    dev = ccoords.device
     n = ccoords.shape[0]
-    row_splits = row_splits.to(device=dev, dtype=torch.int32).contiguous()
-    num_rows = row_splits.numel() - 1
-
-    dist = (dist.to(torch.float32) / distance_threshold).reshape(-1)
-    betas = betas.to(torch.float32).reshape(-1)
-    if no_condensation_mask is None:
-        mask = torch.zeros((n,), dtype=torch.int32, device=dev)
-    else:
-        mask = no_condensation_mask.to(device=dev, dtype=torch.int32).reshape(-1)
-
+    # the whole chain (shift to the minimum, binning, bin order, high-beta subset, assignment,
+    # back to the caller's order) runs inside the library
     n_bins_sc = max(4, min(int(math.ceil(math.pow(n / 5, 1 / 3))), 25))
-    ccoords = (ccoords - ccoords.min(dim=0, keepdim=True).values).contiguous()
-    n_bin_dims = min(ccoords.shape[1], nbin_dims)
-
-    # binning of the first n_bin_dims columns (pre-normalised), stable sort into bin order
-    _shift, bin_width, n_bins = ops.bin_setup(ccoords, n_bin_dims, True, n_bins=n_bins_sc)
-    cells_bound = (n_bins_sc + 1) ** n_bin_dims * num_rows
-    _, bins_flat, _ = ops.bin_points(ccoords, n_bin_dims, None, row_splits, bin_width, n_bins, cells_bound, False)
-    sorting, bin_splits = ops.sort_by_bin(bins_flat, cells_bound)
-
-    ccoords_s = ops.gather_rows(ccoords, sorting)
-    betas_s = ops.gather_rows(betas.contiguous(), sorting)
-    dist_s = ops.gather_rows(dist.contiguous(), sorting)
-    mask_s = ops.gather_rows(mask.contiguous(), sorting)
-    bins_s = ops.gather_rows(bins_flat, sorting)
-
-    # high-beta subset, same order
-    high = (betas_s > beta_threshold) | (mask_s > 0)
-    csum = torch.cumsum(high.to(torch.int32), 0, dtype=torch.int32)
-    to_filtered = torch.where(high, csum - 1, torch.full_like(csum, -1))
-    csum0 = torch.cat([torch.zeros(1, dtype=torch.int32, device=dev), csum])
-    row_splits_h = csum0[row_splits.to(torch.int64)].contiguous()
-    sel = torch.nonzero(high).reshape(-1)
-    ccoords_h = ccoords_s[sel]
-    betas_h = betas_s[sel]
-    dist_h = dist_s[sel]
-    mask_h = mask_s[sel]
-    orig_h = sorting[sel]
-
-    _, assignment_s, alpha, asso_s, n_condensates = torch.ops.hgcalml.binned_assign_to_condensates(
-        ccoords_s, dist_s, betas_s, mask_s, bins_s, bin_splits, to_filtered, orig_h, row_splits, n_bins, bin_width,
-        ccoords_h, dist_h, betas_h, mask_h, row_splits_h, float(beta_threshold), bool(assign_by_max_beta))
-
-    perm = sorting.to(torch.int64)
-    assignment = torch.empty_like(assignment_s)
-    asso = torch.empty_like(asso_s)
-    assignment[perm] = assignment_s
-    asso[perm] = asso_s
-
-    alpha_idx = alpha[alpha != -1]
-    is_cond = torch.zeros((n,), dtype=torch.bool, device=dev)
-    is_cond[alpha_idx.to(torch.int64)] = True
+    assignment, asso, alpha_idx, is_cond, n_condensates = ops.build_and_assign_condensates(
+        ccoords, betas, dist, no_condensation_mask, row_splits, beta_threshold, distance_threshold,
+        assign_by_max_beta, nbin_dims, n_bins_sc)
     out = (assignment[:, None], asso, alpha_idx, is_cond[:, None], n_condensates)
     if keep_noise:
         out = merge_noise_as_indiv_cp(*out, row_splits)

@@ -83,6 +83,12 @@ struct CondParams {
     const int *row_splits;
     int num_rows, by_max_beta, n_vert, n_vert_h;
     int rows_aligned;  // ccoords and ccoords_h start on 16-byte boundaries
+    // The *_h arrays may be the arrays of all hits themselves (n_vert_h == n_vert, identity
+    // indices) instead of a filtered copy: then `high` [n_vert] says which hits belong to the
+    // high-beta subset, and `quirk` = {index of the first of them, its no_condensation_mask,
+    // that of the second one} stands for the first two entries of the filtered mask.
+    const int *high;
+    const int *quirk;
     // workspace
     const int *order_h;  // high-beta hits in selection order, grouped by event
     int *pos_h;          // [n_vert_h] position of a high-beta hit among all hits, -1 unknown
@@ -114,9 +120,18 @@ __host__ __device__ constexpr int cand_words(int cmax) { return cmax + 8 + alpha
 __device__ __forceinline__ int saturate16(int v) { return max(-32768, min(32767, v)); }
 
 // the reference indexes the high-beta mask with the truth value of (q > 0)
-__device__ __forceinline__ bool always_first(const int *mask_h, int n_vert_h, int q) {
+__device__ __forceinline__ bool always_first(const CondParams &p, int q) {
+    if (p.high) return (q == p.quirk[0] ? p.quirk[1] : p.quirk[2]) != 0;
     const int slot = q > 0 ? 1 : 0;
-    return slot < n_vert_h && mask_h[slot] != 0;
+    return slot < p.n_vert_h && p.mask_h[slot] != 0;
+}
+
+// 0: picked as soon as it is the first unclaimed one, in position order; 1: picked by beta;
+// 2: never picked
+__device__ __forceinline__ int selection_class(const CondParams &p, int q) {
+    if (p.high && !p.high[q]) return 2;
+    if (always_first(p, q)) return 0;
+    return p.beta_h[q] > -1.f ? 1 : 2;  // beta <= -1 (or NaN) is never picked
 }
 
 // r with splits[r] <= i < splits[r+1]
@@ -138,16 +153,12 @@ __global__ __launch_bounds__(256) void selection_keys_kernel(const CondParams p,
     const int q = blockIdx.x * blockDim.x + threadIdx.x;
     if (q >= p.n_vert_h) return;
     const uint64_t ev = (uint64_t)event_of(p.row_splits_h, p.num_rows, q);
-    uint64_t cls, low;
-    if (always_first(p.mask_h, p.n_vert_h, q)) {
-        cls = 0;  // chosen as soon as it is the first unclaimed one, in position order
-        low = 0;
-    } else {
-        const float b = p.beta_h[q];
-        uint32_t u = __float_as_uint(b);
+    const uint64_t cls = (uint64_t)selection_class(p, q);
+    uint64_t low = 0;
+    if (cls == 1) {
+        uint32_t u = __float_as_uint(p.beta_h[q]);
         u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // monotone map float -> uint
         low = (uint32_t)~u;                               // larger beta first
-        cls = (b > -1.f) ? 1 : 2;                         // beta <= -1 (or NaN) is never picked
     }
     keys[q] = (ev << 34) | (cls << 32) | low;
     values[q] = q;
@@ -211,6 +222,9 @@ __global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams
     Grid g;
     g.load(p);
     const int q = p.order_h[i];
+    const bool selectable = selection_class(p, q) < 2;
+    p.closed[i] = selectable ? 0 : 1;
+    if (!selectable) return;  // nobody reads its record
     const int at = p.pos_h[q];
     uint32_t rec[cw];
     uint32_t *point = rec + CMAX + 8;
@@ -262,8 +276,6 @@ __global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams
     uint4 *out = reinterpret_cast<uint4 *>(p.cand + (size_t)i * cw);
 #pragma unroll
     for (int w = 0; w < cw; w += 4) out[w / 4] = uint4{rec[w], rec[w + 1], rec[w + 2], rec[w + 3]};
-    const bool selectable = always_first(p.mask_h, p.n_vert_h, q) || p.beta_h[q] > -1.f;
-    p.closed[i] = selectable ? 0 : 1;
 }
 
 // The reference's claim test of one hit against one condensation point, in two
@@ -773,13 +785,8 @@ int run(const CondParams &p, hipStream_t s, int &last_launch) {
 }
 
 }  // namespace
-}  // namespace hgc
 
-using namespace hgc;
-
-extern "C" {
-
-size_t hgc_binned_assign_to_condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows) {
+size_t condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows) {
     const size_t nh = std::max(n_vert_h, 1);
     size_t temp = 0;
     (void)rocprim::radix_sort_pairs(nullptr, temp, (const uint64_t *)nullptr, (uint64_t *)nullptr,
@@ -788,26 +795,24 @@ size_t hgc_binned_assign_to_condensates_workspace_bytes(int n_vert, int n_vert_h
     return align_up(temp) + carve_workspace(nullptr, n_vert, n_vert_h, num_rows).used;
 }
 
-int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,
-                                     const float *d_ccoords_h, const float *d_dist_h, const float *d_beta_h,
-                                     const int *d_no_condensation_mask_h, int *d_high_assigned_status_h,
-                                     const int *d_original_indices_h, const int *d_row_splits_h,
-                                     const float *d_ccoords, const float *d_dist,
-                                     const int *d_no_condensation_mask, const int *d_indices_to_filtered,
-                                     float *d_assignment_min_distance, int *d_assignment, int *d_association,
-                                     int *d_n_condensates, int *d_alpha_indices, const int *d_bin_splits,
-                                     const int *d_n_bins, const float *d_bin_widths, const int *d_row_splits,
-                                     int num_rows, int assign_by_max_beta, int n_vert, int n_vert_h, int *d_error,
-                                     void *workspace, size_t workspace_bytes, hgc_stream_t stream) {
-    (void)d_dist;  // carried by the reference functor, never read by its kernel
+int condensates_assign(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,
+                       const float *d_ccoords_h, const float *d_dist_h, const float *d_beta_h,
+                       const int *d_no_condensation_mask_h, int *d_high_assigned_status_h,
+                       const int *d_original_indices_h, const int *d_row_splits_h, const float *d_ccoords,
+                       const int *d_no_condensation_mask, const int *d_indices_to_filtered,
+                       float *d_assignment_min_distance, int *d_assignment, int *d_association,
+                       int *d_n_condensates, int *d_alpha_indices, const int *d_bin_splits, const int *d_n_bins,
+                       const float *d_bin_widths, const int *d_row_splits, int num_rows, int assign_by_max_beta,
+                       int n_vert, int n_vert_h, int *d_error, const int *d_high, const int *d_quirk,
+                       void *workspace, size_t workspace_bytes, hipStream_t s) {
     HGC_REQUIRE(dimensions >= 1 && dimensions <= kMaxDims, "1 <= coordinate dimensions <= %d", kMaxDims);
     HGC_REQUIRE(dimensions_binning >= 1 && dimensions_binning <= kMaxBinDims && dimensions_binning <= dimensions,
                 "1 <= binning dimensions <= min(%d, coordinate dimensions)", kMaxBinDims);
     HGC_REQUIRE(num_rows >= 0 && n_vert >= 0 && n_vert_h >= 0 && n_vert_h <= n_vert, "bad sizes");
     HGC_REQUIRE(d_n_condensates && d_row_splits && d_row_splits_h, "null pointer");
-    hipStream_t s = as_stream(stream);
+    HGC_REQUIRE(!d_high || (d_quirk && n_vert_h == n_vert), "hits as their own high-beta subset: sizes differ");
     if (!workspace || !aligned256(workspace) ||
-        workspace_bytes < hgc_binned_assign_to_condensates_workspace_bytes(n_vert, n_vert_h, num_rows))
+        workspace_bytes < condensates_workspace_bytes(n_vert, n_vert_h, num_rows))
         return fail(HGC_ERR_WORKSPACE, "condensates workspace missing, misaligned or too small");
     if (n_vert > 0)
         HGC_REQUIRE(d_ccoords && d_no_condensation_mask && d_indices_to_filtered && d_assignment && d_association &&
@@ -849,6 +854,8 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int
     p.n_vert = n_vert;
     p.n_vert_h = n_vert_h;
     p.rows_aligned = ((reinterpret_cast<uintptr_t>(d_ccoords) | reinterpret_cast<uintptr_t>(d_ccoords_h)) & 15u) == 0;
+    p.high = d_high;
+    p.quirk = d_quirk;
     p.order_h = w.order;
     p.pos_h = w.pos_h;
     p.hit_bin = w.hit_bin;
@@ -875,6 +882,37 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int
     cumulative_counts_kernel<<<1, 64, 0, s>>>(w.n_alpha_at + (size_t)last_launch * num_rows, num_rows,
                                               d_n_condensates, d_error);
     return check_launch("cumulative_counts");
+}
+
+}  // namespace hgc
+
+using namespace hgc;
+
+extern "C" {
+
+size_t hgc_binned_assign_to_condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows) {
+    return condensates_workspace_bytes(n_vert, n_vert_h, num_rows);
+}
+
+int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,
+                                     const float *d_ccoords_h, const float *d_dist_h, const float *d_beta_h,
+                                     const int *d_no_condensation_mask_h, int *d_high_assigned_status_h,
+                                     const int *d_original_indices_h, const int *d_row_splits_h,
+                                     const float *d_ccoords, const float *d_dist,
+                                     const int *d_no_condensation_mask, const int *d_indices_to_filtered,
+                                     float *d_assignment_min_distance, int *d_assignment, int *d_association,
+                                     int *d_n_condensates, int *d_alpha_indices, const int *d_bin_splits,
+                                     const int *d_n_bins, const float *d_bin_widths, const int *d_row_splits,
+                                     int num_rows, int assign_by_max_beta, int n_vert, int n_vert_h, int *d_error,
+                                     void *workspace, size_t workspace_bytes, hgc_stream_t stream) {
+    (void)d_dist;  // carried by the reference functor, never read by its kernel
+    return condensates_assign(dimensions, dimensions_binning, d_condensates_assigned_h, d_ccoords_h, d_dist_h,
+                              d_beta_h, d_no_condensation_mask_h, d_high_assigned_status_h, d_original_indices_h,
+                              d_row_splits_h, d_ccoords, d_no_condensation_mask, d_indices_to_filtered,
+                              d_assignment_min_distance, d_assignment, d_association, d_n_condensates,
+                              d_alpha_indices, d_bin_splits, d_n_bins, d_bin_widths, d_row_splits, num_rows,
+                              assign_by_max_beta, n_vert, n_vert_h, d_error, nullptr, nullptr, workspace,
+                              workspace_bytes, as_stream(stream));
 }
 
 }  // extern "C"

@@ -89,6 +89,23 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
                               int n_neigh, int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
                               int use_direction, hipStream_t s);
 
+// hgc_binned_assign_to_condensates with two more arguments: with d_high set, the *_h
+// arrays are the arrays of all hits themselves (n_vert_h == n_vert, d_indices_to_filtered[i]
+// = i or -1, d_row_splits_h = d_row_splits) and d_high [n_vert] says which hits form the
+// high-beta subset; d_quirk = {index of the first of them, its no_condensation_mask, the
+// second one's} then stands for the first two entries of the filtered mask.
+size_t condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows);
+int condensates_assign(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,
+                       const float *d_ccoords_h, const float *d_dist_h, const float *d_beta_h,
+                       const int *d_no_condensation_mask_h, int *d_high_assigned_status_h,
+                       const int *d_original_indices_h, const int *d_row_splits_h, const float *d_ccoords,
+                       const int *d_no_condensation_mask, const int *d_indices_to_filtered,
+                       float *d_assignment_min_distance, int *d_assignment, int *d_association,
+                       int *d_n_condensates, int *d_alpha_indices, const int *d_bin_splits, const int *d_n_bins,
+                       const float *d_bin_widths, const int *d_row_splits, int num_rows, int assign_by_max_beta,
+                       int n_vert, int n_vert_h, int *d_error, const int *d_high, const int *d_quirk,
+                       void *workspace, size_t workspace_bytes, hipStream_t s);
+
 // ---- device helpers -------------------------------------------------------
 
 #ifdef __HIPCC__

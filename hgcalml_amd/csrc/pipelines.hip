@@ -5,9 +5,16 @@
 //   hgc_binned_select_knn_pipeline  modules/binned_select_knn_op.py:33-104
 //     (bounding box and grid, bin assignment, grouping by bin with the inputs
 //      moved along, search, un-sort)
+//   hgc_build_and_assign_condensates  modules/assign_condensate_op.py:210-373
+//     (coordinates shifted to their minimum, grid, bin assignment, stable sort
+//      into bin order, high-beta subset, assignment, back to the caller's order)
 #include "hgc_common.hpp"
 
 #include <algorithm>
+
+namespace hgc {
+int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
+}
 
 using namespace hgc;
 
@@ -45,9 +52,277 @@ KnnPipelineLayout knn_layout(int n_vert, int n_coords, int n_bin_dims, int n_rs,
     return L;
 }
 
+// ---- condensates ------------------------------------------------------------
+
+constexpr int kMaxCoordDims = 16;
+
+__device__ __forceinline__ uint32_t ordered_bits(float x) {
+    const uint32_t u = __float_as_uint(x);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float from_ordered_bits(uint32_t u) {
+    return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
+}
+
+// column minima (NaN ignored) as order-preserving bit patterns, combined with atomicMin
+__global__ __launch_bounds__(256) void column_min_kernel(const float *__restrict__ x, int n, int C,
+                                                         uint32_t *__restrict__ mins) {
+    __shared__ uint32_t s_min[kMaxCoordDims];
+    if (threadIdx.x < kMaxCoordDims) s_min[threadIdx.x] = 0xffffffffu;
+    __syncthreads();
+    uint32_t lo[kMaxCoordDims];
+#pragma unroll
+    for (int c = 0; c < kMaxCoordDims; ++c) lo[c] = 0xffffffffu;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
+#pragma unroll
+        for (int c = 0; c < kMaxCoordDims; ++c)
+            if (c < C) {
+                const float v = x[(size_t)i * C + c];
+                if (v == v) lo[c] = min(lo[c], ordered_bits(v));
+            }
+#pragma unroll
+    for (int c = 0; c < kMaxCoordDims; ++c) {
+        if (c < C) {
+            uint32_t v = lo[c];
+            for (int off = 32; off > 0; off >>= 1) v = min(v, (uint32_t)__shfl_xor((int)v, off, kWave));
+            if (lane_id() == 0) atomicMin(&s_min[c], v);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < C) atomicMin(&mins[threadIdx.x], s_min[threadIdx.x]);
+}
+
+// coordinates minus their column minimum: the wrapper's ccoords - min(ccoords)
+__global__ __launch_bounds__(256) void shift_to_minimum_kernel(const float *__restrict__ x, long long n_values, int C,
+                                                               const uint32_t *__restrict__ mins,
+                                                               float *__restrict__ out) {
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n_values) return;
+    out[e] = x[e] - from_ordered_bits(mins[e % C]);
+}
+
+// inputs moved into bin order, local radii scaled, the high-beta subset marked
+__global__ __launch_bounds__(256) void condensate_inputs_kernel(const float *__restrict__ shifted,
+                                                                const float *__restrict__ betas,
+                                                                const float *__restrict__ dist,
+                                                                const int *__restrict__ mask,
+                                                                const int *__restrict__ sorting, int n, int C,
+                                                                float beta_threshold, float distance_threshold,
+                                                                float *__restrict__ coords_s,
+                                                                float *__restrict__ betas_s,
+                                                                float *__restrict__ dist_s, int *__restrict__ mask_s,
+                                                                int *__restrict__ high, int *__restrict__ to_filtered) {
+    const int at = blockIdx.x * blockDim.x + threadIdx.x;
+    if (at >= n) return;
+    const int i = sorting[at];
+    for (int c = 0; c < C; ++c) coords_s[(size_t)at * C + c] = shifted[(size_t)i * C + c];
+    const float b = betas[i];
+    const int m = mask ? mask[i] : 0;
+    betas_s[at] = b;
+    dist_s[at] = dist[i] / distance_threshold;
+    mask_s[at] = m;
+    const bool is_high = b > beta_threshold || m > 0;
+    high[at] = is_high;
+    to_filtered[at] = is_high ? at : -1;
+}
+
+// {first hit of the high-beta subset, its mask, the second one's mask}
+__global__ __launch_bounds__(1024) void first_two_high_kernel(const int *__restrict__ high,
+                                                              const int *__restrict__ mask_s, int n,
+                                                              int *__restrict__ quirk) {
+    __shared__ int s_count[16], s_found[2];
+    if (threadIdx.x < 2) s_found[threadIdx.x] = -1;
+    __syncthreads();
+    int found = 0;
+    for (int base = 0; base < n && found < 2; base += 1024) {
+        const int i = base + threadIdx.x;
+        const bool h = i < n && high[i] != 0;
+        const uint64_t m = __ballot(h);
+        if (lane_id() == 0) s_count[threadIdx.x >> 6] = __popcll(m);
+        __syncthreads();
+        int before = 0, total = 0;
+        for (int w = 0; w < 16; ++w) {
+            if (w < (int)(threadIdx.x >> 6)) before += s_count[w];
+            total += s_count[w];
+        }
+        const int nth = found + before + __popcll(m & ((1ull << lane_id()) - 1ull));
+        if (h && nth < 2) s_found[nth] = i;
+        found += total;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        quirk[0] = s_found[0];
+        quirk[1] = s_found[0] >= 0 ? mask_s[s_found[0]] : 0;
+        quirk[2] = s_found[1] >= 0 ? mask_s[s_found[1]] : 0;
+    }
+}
+
+// results back in the caller's order; the condensation points of all events as one list
+__global__ __launch_bounds__(256) void condensate_outputs_kernel(const int *__restrict__ sorting,
+                                                                 const int *__restrict__ assignment_s,
+                                                                 const int *__restrict__ association_s,
+                                                                 const int *__restrict__ is_alpha,
+                                                                 const int *__restrict__ alpha_indices,
+                                                                 const int *__restrict__ row_splits,
+                                                                 const int *__restrict__ n_condensates, int n,
+                                                                 int num_rows, int *__restrict__ assignment,
+                                                                 int *__restrict__ association,
+                                                                 unsigned char *__restrict__ is_cond,
+                                                                 int *__restrict__ alpha_idx) {
+    const int at = blockIdx.x * blockDim.x + threadIdx.x;
+    if (at >= n) return;
+    const int i = sorting[at];
+    assignment[i] = assignment_s[at];
+    association[i] = association_s[at];
+    is_cond[i] = is_alpha[at] != 0;
+    int lo = 1, hi = num_rows + 1;  // event = last r with row_splits[r] <= at
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (row_splits[mid] > at)
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    const int r = min(lo - 1, num_rows - 1);
+    const int nth = at - row_splits[r];
+    if (nth < n_condensates[r + 1] - n_condensates[r]) alpha_idx[n_condensates[r] + nth] = alpha_indices[at];
+}
+
+struct CondPipelineLayout {
+    size_t mins, shifted, shift, bin_width, n_bins, binass, flat, sorting, bin_splits, coords_s, betas_s, dist_s,
+        mask_s, high, to_filtered, quirk, taken, is_alpha, best, assignment_s, association_s, alpha_indices, setup_ws,
+        sort_ws, core_ws, total;
+    size_t setup_bytes, sort_bytes, core_bytes;
+    int cells_bound, n_bin_dims;
+};
+
+bool cond_layout(int n_vert, int n_coords, int num_rows, int n_bins_scalar, int nbin_dims, CondPipelineLayout &L) {
+    L = CondPipelineLayout{};
+    L.n_bin_dims = std::min(n_coords, nbin_dims);
+    long long cells = std::max(num_rows, 1);
+    for (int d = 0; d < L.n_bin_dims; ++d) cells = std::min<long long>(cells * (n_bins_scalar + 1), 1ll << 40);
+    if (cells >= (1ll << 31) - 2) return false;
+    L.cells_bound = (int)cells;
+    const size_t n = std::max(n_vert, 1);
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        size_t at = off;
+        off += align_up(bytes);
+        return at;
+    };
+    L.mins = take(kMaxCoordDims * sizeof(uint32_t));
+    L.shifted = take(n * n_coords * sizeof(float));
+    L.shift = take(8 * sizeof(float));
+    L.bin_width = take(sizeof(float));
+    L.n_bins = take(8 * sizeof(int));
+    L.binass = take(n * (L.n_bin_dims + 1) * sizeof(int));
+    L.flat = take(n * sizeof(int));
+    L.sorting = take(n * sizeof(int));
+    L.bin_splits = take(((size_t)L.cells_bound + 1) * sizeof(int));
+    L.coords_s = take(n * n_coords * sizeof(float));
+    L.betas_s = take(n * sizeof(float));
+    L.dist_s = take(n * sizeof(float));
+    L.mask_s = take(n * sizeof(int));
+    L.high = take(n * sizeof(int));
+    L.to_filtered = take(n * sizeof(int));
+    L.quirk = take(4 * sizeof(int));
+    L.taken = take(n * sizeof(int));
+    L.is_alpha = take(n * sizeof(int));
+    L.best = take(n * sizeof(float));
+    L.assignment_s = take(n * sizeof(int));
+    L.association_s = take(n * sizeof(int));
+    L.alpha_indices = take(n * sizeof(int));
+    L.setup_bytes = hgc_bin_setup_workspace_bytes(n_vert, L.n_bin_dims);
+    L.sort_bytes = hgc_sort_by_bin_workspace_bytes(n_vert, L.cells_bound);
+    L.core_bytes = condensates_workspace_bytes(n_vert, n_vert, num_rows);
+    L.setup_ws = take(L.setup_bytes);
+    L.sort_ws = take(L.sort_bytes);
+    L.core_ws = take(L.core_bytes);
+    L.total = off;
+    return true;
+}
+
 }  // namespace
 
 extern "C" {
+
+size_t hgc_build_and_assign_condensates_workspace_bytes(int n_vert, int n_coords, int num_rows, int n_bins_scalar,
+                                                        int nbin_dims) {
+    CondPipelineLayout L;
+    if (n_vert < 0 || n_coords < 1 || n_coords > kMaxCoordDims || num_rows < 0 || n_bins_scalar < 1 || nbin_dims < 1 ||
+        nbin_dims > 6 || !cond_layout(n_vert, n_coords, num_rows, n_bins_scalar, nbin_dims, L))
+        return 0;
+    return L.total;
+}
+
+int hgc_build_and_assign_condensates(const float *d_ccoords, const float *d_betas, const float *d_dist,
+                                     const int *d_no_condensation_mask, const int *d_row_splits, int n_vert,
+                                     int n_coords, int num_rows, float beta_threshold, float distance_threshold,
+                                     int assign_by_max_beta, int nbin_dims, int n_bins_scalar, int *d_assignment,
+                                     int *d_association, int *d_alpha_idx, unsigned char *d_is_cond,
+                                     int *d_n_condensates, void *workspace, size_t workspace_bytes,
+                                     hgc_stream_t stream) {
+    HGC_REQUIRE(n_vert >= 0 && num_rows >= 0, "bad sizes");
+    HGC_REQUIRE(n_coords >= 1 && n_coords <= kMaxCoordDims, "1 <= coordinate dimensions <= %d", kMaxCoordDims);
+    HGC_REQUIRE(nbin_dims >= 1 && nbin_dims <= 6, "1 <= nbin_dims <= 6");
+    HGC_REQUIRE(n_bins_scalar >= 1, "n_bins must be positive");
+    HGC_REQUIRE(distance_threshold > 0.f, "distance_threshold must be positive");
+    HGC_REQUIRE(d_row_splits && d_n_condensates, "null pointer");
+    hipStream_t s = as_stream(stream);
+    if (n_vert == 0) return launch_fill_i32(d_n_condensates, 0, (long long)num_rows + 1, s);
+    HGC_REQUIRE(num_rows >= 1, "hits without an event");
+    HGC_REQUIRE(d_ccoords && d_betas && d_dist && d_assignment && d_association && d_alpha_idx && d_is_cond,
+                "null pointer");
+    CondPipelineLayout L;
+    HGC_REQUIRE(cond_layout(n_vert, n_coords, num_rows, n_bins_scalar, nbin_dims, L),
+                "bin table overflows int32: fewer bins or events per call");
+    if (!workspace || !aligned256(workspace) || workspace_bytes < L.total)
+        return fail(HGC_ERR_WORKSPACE, "condensates workspace missing, misaligned or too small");
+    char *ws = static_cast<char *>(workspace);
+    auto F = [&](size_t off) { return reinterpret_cast<float *>(ws + off); };
+    auto I = [&](size_t off) { return reinterpret_cast<int *>(ws + off); };
+    uint32_t *mins = reinterpret_cast<uint32_t *>(ws + L.mins);
+    const int B = L.n_bin_dims;
+    int rc;
+
+    if ((rc = launch_fill_i32(reinterpret_cast<int *>(mins), -1, kMaxCoordDims, s))) return rc;
+    column_min_kernel<<<std::max(1, std::min(512, ceil_div(n_vert, 1024))), 256, 0, s>>>(d_ccoords, n_vert, n_coords,
+                                                                                          mins);
+    if ((rc = check_launch("column_min"))) return rc;
+    const long long n_values = (long long)n_vert * n_coords;
+    shift_to_minimum_kernel<<<ceil_div(n_values, 256), 256, 0, s>>>(d_ccoords, n_values, n_coords, mins,
+                                                                    F(L.shifted));
+    if ((rc = check_launch("shift_to_minimum"))) return rc;
+    // grid over the already shifted coordinates, hits into stable bin order
+    if ((rc = hgc_bin_setup(F(L.shifted), n_coords, n_vert, B, 1, n_bins_scalar, nullptr, F(L.shift), F(L.bin_width),
+                            I(L.n_bins), ws + L.setup_ws, L.setup_bytes, stream)))
+        return rc;
+    if ((rc = hgc_bin_by_coordinates_strided(F(L.shifted), n_coords, nullptr, d_row_splits, F(L.bin_width),
+                                             I(L.n_bins), I(L.binass), I(L.flat), nullptr, nullptr, n_vert, B,
+                                             num_rows + 1, L.cells_bound, 0, stream)))
+        return rc;
+    if ((rc = hgc_sort_by_bin(I(L.flat), n_vert, L.cells_bound, I(L.sorting), I(L.bin_splits), ws + L.sort_ws,
+                              L.sort_bytes, stream)))
+        return rc;
+    condensate_inputs_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(
+        F(L.shifted), d_betas, d_dist, d_no_condensation_mask, I(L.sorting), n_vert, n_coords, beta_threshold,
+        distance_threshold, F(L.coords_s), F(L.betas_s), F(L.dist_s), I(L.mask_s), I(L.high), I(L.to_filtered));
+    if ((rc = check_launch("condensate_inputs"))) return rc;
+    first_two_high_kernel<<<1, 1024, 0, s>>>(I(L.high), I(L.mask_s), n_vert, I(L.quirk));
+    if ((rc = check_launch("first_two_high"))) return rc;
+    // every hit is its own entry of the "high-beta" arrays; `high` says which ones count
+    if ((rc = condensates_assign(n_coords, B, I(L.taken), F(L.coords_s), F(L.dist_s), F(L.betas_s), I(L.mask_s),
+                                 I(L.is_alpha), I(L.sorting), d_row_splits, F(L.coords_s), I(L.mask_s),
+                                 I(L.to_filtered), F(L.best), I(L.assignment_s), I(L.association_s), d_n_condensates,
+                                 I(L.alpha_indices), I(L.bin_splits), I(L.n_bins), F(L.bin_width), d_row_splits,
+                                 num_rows, assign_by_max_beta, n_vert, n_vert, nullptr, I(L.high), I(L.quirk),
+                                 ws + L.core_ws, L.core_bytes, s)))
+        return rc;
+    condensate_outputs_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(
+        I(L.sorting), I(L.assignment_s), I(L.association_s), I(L.is_alpha), I(L.alpha_indices), d_row_splits,
+        d_n_condensates, n_vert, num_rows, d_assignment, d_association, d_is_cond, d_alpha_idx);
+    return check_launch("condensate_outputs");
+}
 
 size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, int n_rs, int n_bins_scalar,
                                                       int max_bin_dims, int use_direction) {

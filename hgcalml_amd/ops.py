@@ -428,3 +428,30 @@ def binned_assign_to_condensates(ccoords: torch.Tensor, dist: torch.Tensor, beta
                                                p(row_splits), num_rows, int(assign_by_max_beta), n, nh, None, p(ws),
                                                ws.numel(), stream()))
     return assigned_h, assigned, alpha, asso, ncond
+
+
+def build_and_assign_condensates(ccoords, betas, dist, mask, row_splits, beta_threshold, distance_threshold,
+                                 assign_by_max_beta, nbin_dims, n_bins_scalar):
+    """modules/assign_condensate_op.py:210-373 (without keep_noise) as one call into the library;
+    returns (assignment [n], association [n], alpha_idx [n_condensates], is_cond [n] bool,
+    n_condensates [events + 1]). One host synchronisation, for the length of alpha_idx."""
+    dev = require_device(ccoords, betas, dist)
+    ccoords, betas, dist = f32(ccoords), f32(betas).reshape(-1), f32(dist).reshape(-1)
+    row_splits = i32(row_splits.to(dev))
+    if mask is not None:
+        mask = i32(mask.to(dev)).reshape(-1)
+    n, c = ccoords.shape
+    num_rows = row_splits.numel() - 1
+    assignment = torch.empty((n,), dtype=torch.int32, device=dev)
+    asso = torch.empty((n,), dtype=torch.int32, device=dev)
+    alpha = torch.empty((max(n, 1),), dtype=torch.int32, device=dev)
+    is_cond = torch.empty((n,), dtype=torch.bool, device=dev)
+    ncond = torch.empty((num_rows + 1,), dtype=torch.int32, device=dev)
+    ws = workspace(lib.hgc_build_and_assign_condensates_workspace_bytes(n, c, num_rows, n_bins_scalar, nbin_dims), dev)
+    check(lib.hgc_build_and_assign_condensates(p(ccoords), p(betas), p(dist), p(mask), p(row_splits), n, c, num_rows,
+                                               float(beta_threshold), float(distance_threshold),
+                                               int(assign_by_max_beta), nbin_dims, n_bins_scalar, p(assignment),
+                                               p(asso), p(alpha), p(is_cond), p(ncond), p(ws), ws.numel(), stream()))
+    total = int(ncond[-1]) if n > 0 else 0
+    return assignment, asso, alpha[:total], is_cond, ncond
+

@@ -360,6 +360,30 @@ int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning,
                                      void *workspace, size_t workspace_bytes,
                                      hgc_stream_t stream);
 
+/* The whole wrapper modules/assign_condensate_op.py:210-373
+ * (BuildAndAssignCondensatesBinned without keep_noise) in one call: coordinates
+ * shifted to their column minima, grid of n_bins_scalar bins along the widest of
+ * the first min(nbin_dims, n_coords) coordinates, bin assignment, stable sort
+ * into bin order, local radii divided by distance_threshold, high-beta subset
+ * (beta > beta_threshold or masked), assignment, results back in the caller's
+ * order. Inputs in the caller's order: d_ccoords [n_vert, n_coords], d_betas,
+ * d_dist [n_vert], d_no_condensation_mask [n_vert] or NULL, d_row_splits
+ * [num_rows + 1]. Outputs: d_assignment, d_association [n_vert], d_is_cond
+ * [n_vert] (one byte each), d_n_condensates [num_rows + 1] (cumulative) and
+ * d_alpha_idx, which must have room for n_vert entries; its first
+ * d_n_condensates[num_rows] ones are the condensation points of all events in
+ * selection order. No host synchronisation (the caller reads
+ * d_n_condensates[num_rows] to learn how many entries of d_alpha_idx count). */
+size_t hgc_build_and_assign_condensates_workspace_bytes(int n_vert, int n_coords, int num_rows,
+                                                        int n_bins_scalar, int nbin_dims);
+int hgc_build_and_assign_condensates(const float *d_ccoords, const float *d_betas, const float *d_dist,
+                                     const int *d_no_condensation_mask, const int *d_row_splits,
+                                     int n_vert, int n_coords, int num_rows, float beta_threshold,
+                                     float distance_threshold, int assign_by_max_beta, int nbin_dims,
+                                     int n_bins_scalar, int *d_assignment, int *d_association,
+                                     int *d_alpha_idx, unsigned char *d_is_cond, int *d_n_condensates,
+                                     void *workspace, size_t workspace_bytes, hgc_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
