@@ -98,6 +98,7 @@ struct CondParams {
                          // picked at all, or a point of an earlier launch covers it)
     uint32_t *points;    // [n_vert_h] an event's condensation points in selection order, from
                          // row_splits_h[event] on
+    int *walk_end;       // [num_rows] end of the event's candidates that can be picked at all
     int *cursor_at;      // [kMaxLaunches][num_rows] selection position an event's walk stopped at
     int *n_alpha_at;     // [kMaxLaunches][num_rows] points of the event after that launch
 };
@@ -172,6 +173,7 @@ __global__ __launch_bounds__(256) void selection_keys_kernel(const CondParams p,
 // position of every high-beta hit among all hits
 __global__ __launch_bounds__(256) void hit_prepare_kernel(const CondParams p) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < p.num_rows) p.walk_end[i] = p.row_splits_h[i + 1];  // unless candidate_records_kernel finds less
     if (i >= p.n_vert) return;
     const int r = event_of(p.row_splits, p.num_rows, i);
     int cells = 1;
@@ -224,7 +226,12 @@ __global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams
     const int q = p.order_h[i];
     const bool selectable = selection_class(p, q) < 2;
     p.closed[i] = selectable ? 0 : 1;
-    if (!selectable) return;  // nobody reads its record
+    if (!selectable) {
+        // those that are never picked come last in an event's order: the walk ends at the first one
+        const int ev = event_of(p.row_splits_h, p.num_rows, i);
+        if (i == p.row_splits_h[ev] || selection_class(p, p.order_h[i - 1]) < 2) p.walk_end[ev] = i;
+        return;  // nobody reads its record
+    }
     const int at = p.pos_h[q];
     uint32_t rec[cw];
     uint32_t *point = rec + CMAX + 8;
@@ -344,7 +351,7 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
-    const int first_h = p.row_splits_h[r], last_h = p.row_splits_h[r + 1];
+    const int first_h = p.row_splits_h[r], last_h = p.walk_end[r];
 
     int cur = launch == 0 ? first_h : p.cursor_at[(launch - 1) * p.num_rows + r];
     int n_alpha = launch == 0 ? 0 : p.n_alpha_at[(launch - 1) * p.num_rows + r];
@@ -709,12 +716,15 @@ int selection_key_bits(int num_rows) {
 
 struct Workspace {
     uint64_t *keys, *keys_sorted;
-    int *values, *order, *pos_h, *hit_bin, *closed, *cursor_at, *n_alpha_at;
+    int *values, *order, *pos_h, *hit_bin, *closed, *walk_end, *cursor_at, *n_alpha_at;
     uint32_t *cand, *points;
     size_t used;
 };
 
-Workspace carve_workspace(void *base, int n_vert, int n_vert_h, int num_rows) {
+int coordinate_slots(int dimensions) { return dimensions <= 4 ? 4 : dimensions <= 8 ? 8 : kMaxDims; }
+
+Workspace carve_workspace(void *base, int n_vert, int n_vert_h, int num_rows, int dimensions) {
+    const int cmax = coordinate_slots(dimensions);
     const size_t nh = std::max(n_vert_h, 1), n = std::max(n_vert, 1), rows = std::max(num_rows, 1);
     Carver carve(base);
     Workspace w;
@@ -725,10 +735,11 @@ Workspace carve_workspace(void *base, int n_vert, int n_vert_h, int num_rows) {
     w.pos_h = carve.take<int>(nh);
     w.hit_bin = carve.take<int>(n);
     w.closed = carve.take<int>(nh);
-    w.points = carve.take<uint32_t>(nh * (size_t)alpha_words(kMaxDims));
+    w.points = carve.take<uint32_t>(nh * (size_t)alpha_words(cmax));
+    w.walk_end = carve.take<int>(rows);
     w.cursor_at = carve.take<int>(kMaxLaunches * rows);
     w.n_alpha_at = carve.take<int>(kMaxLaunches * rows);
-    w.cand = carve.take<uint32_t>(nh * (size_t)cand_words(kMaxDims));
+    w.cand = carve.take<uint32_t>(nh * (size_t)cand_words(cmax));
     w.used = carve.used;
     return w;
 }
@@ -737,10 +748,8 @@ Workspace carve_workspace(void *base, int n_vert, int n_vert_h, int num_rows) {
 template <int CMAX>
 int run(const CondParams &p, hipStream_t s, int &last_launch) {
     int rc;
-    if (p.n_vert > 0) {
-        hit_prepare_kernel<<<ceil_div(p.n_vert, 256), 256, 0, s>>>(p);
-        if ((rc = check_launch("hit_prepare"))) return rc;
-    }
+    hit_prepare_kernel<<<ceil_div(std::max(p.n_vert, p.num_rows), 256), 256, 0, s>>>(p);
+    if ((rc = check_launch("hit_prepare"))) return rc;
     if (p.n_vert_h > 0) {
         candidate_records_kernel<CMAX><<<ceil_div(p.n_vert_h, 256), 256, 0, s>>>(p);
         if ((rc = check_launch("candidate_records"))) return rc;
@@ -786,13 +795,13 @@ int run(const CondParams &p, hipStream_t s, int &last_launch) {
 
 }  // namespace
 
-size_t condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows) {
+size_t condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows, int dimensions) {
     const size_t nh = std::max(n_vert_h, 1);
     size_t temp = 0;
     (void)rocprim::radix_sort_pairs(nullptr, temp, (const uint64_t *)nullptr, (uint64_t *)nullptr,
                                     (const int *)nullptr, (int *)nullptr, nh, 0,
                                     selection_key_bits(std::max(num_rows, 1)), (hipStream_t) nullptr);
-    return align_up(temp) + carve_workspace(nullptr, n_vert, n_vert_h, num_rows).used;
+    return align_up(temp) + carve_workspace(nullptr, n_vert, n_vert_h, num_rows, dimensions).used;
 }
 
 int condensates_assign(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,
@@ -812,7 +821,7 @@ int condensates_assign(int dimensions, int dimensions_binning, int *d_condensate
     HGC_REQUIRE(d_n_condensates && d_row_splits && d_row_splits_h, "null pointer");
     HGC_REQUIRE(!d_high || (d_quirk && n_vert_h == n_vert), "hits as their own high-beta subset: sizes differ");
     if (!workspace || !aligned256(workspace) ||
-        workspace_bytes < condensates_workspace_bytes(n_vert, n_vert_h, num_rows))
+        workspace_bytes < condensates_workspace_bytes(n_vert, n_vert_h, num_rows, dimensions))
         return fail(HGC_ERR_WORKSPACE, "condensates workspace missing, misaligned or too small");
     if (n_vert > 0)
         HGC_REQUIRE(d_ccoords && d_no_condensation_mask && d_indices_to_filtered && d_assignment && d_association &&
@@ -823,7 +832,7 @@ int condensates_assign(int dimensions, int dimensions_binning, int *d_condensate
                         d_high_assigned_status_h && d_original_indices_h && d_alpha_indices,
                     "null pointer");
 
-    const Workspace w = carve_workspace(workspace, n_vert, n_vert_h, num_rows);
+    const Workspace w = carve_workspace(workspace, n_vert, n_vert_h, num_rows, dimensions);
     void *temp = static_cast<char *>(workspace) + w.used;
     size_t temp_bytes = workspace_bytes - w.used;
 
@@ -862,6 +871,7 @@ int condensates_assign(int dimensions, int dimensions_binning, int *d_condensate
     p.cand = w.cand;
     p.closed = w.closed;
     p.points = w.points;
+    p.walk_end = w.walk_end;
     p.cursor_at = w.cursor_at;
     p.n_alpha_at = w.n_alpha_at;
 
@@ -874,9 +884,10 @@ int condensates_assign(int dimensions, int dimensions_binning, int *d_condensate
             HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, w.keys, w.keys_sorted, w.values, w.order,
                                               (size_t)n_vert_h, 0, selection_key_bits(num_rows), s));
         }
-        const int rc = dimensions <= 4   ? run<4>(p, s, last_launch)
-                       : dimensions <= 8 ? run<8>(p, s, last_launch)
-                                         : run<kMaxDims>(p, s, last_launch);
+        const int slots = coordinate_slots(dimensions);
+        const int rc = slots == 4   ? run<4>(p, s, last_launch)
+                       : slots == 8 ? run<8>(p, s, last_launch)
+                                    : run<kMaxDims>(p, s, last_launch);
         if (rc) return rc;
     }
     cumulative_counts_kernel<<<1, 64, 0, s>>>(w.n_alpha_at + (size_t)last_launch * num_rows, num_rows,
@@ -891,7 +902,7 @@ using namespace hgc;
 extern "C" {
 
 size_t hgc_binned_assign_to_condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows) {
-    return condensates_workspace_bytes(n_vert, n_vert_h, num_rows);
+    return condensates_workspace_bytes(n_vert, n_vert_h, num_rows, kMaxDims);  // the dimensions come with the call
 }
 
 int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,

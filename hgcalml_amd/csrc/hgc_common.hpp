@@ -94,7 +94,7 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
 // = i or -1, d_row_splits_h = d_row_splits) and d_high [n_vert] says which hits form the
 // high-beta subset; d_quirk = {index of the first of them, its no_condensation_mask, the
 // second one's} then stands for the first two entries of the filtered mask.
-size_t condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows);
+size_t condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows, int dimensions);
 int condensates_assign(int dimensions, int dimensions_binning, int *d_condensates_assigned_h,
                        const float *d_ccoords_h, const float *d_dist_h, const float *d_beta_h,
                        const int *d_no_condensation_mask_h, int *d_high_assigned_status_h,

@@ -234,7 +234,7 @@ bool cond_layout(int n_vert, int n_coords, int num_rows, int n_bins_scalar, int 
     L.alpha_indices = take(n * sizeof(int));
     L.setup_bytes = hgc_bin_setup_workspace_bytes(n_vert, L.n_bin_dims);
     L.sort_bytes = hgc_sort_by_bin_workspace_bytes(n_vert, L.cells_bound);
-    L.core_bytes = condensates_workspace_bytes(n_vert, n_vert, num_rows);
+    L.core_bytes = condensates_workspace_bytes(n_vert, n_vert, num_rows, n_coords);
     L.setup_ws = take(L.setup_bytes);
     L.sort_ws = take(L.sort_bytes);
     L.core_ws = take(L.core_bytes);
