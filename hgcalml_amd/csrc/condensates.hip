@@ -638,49 +638,66 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
             }
             const bool any_solitary = __syncthreads_or(solitary_here);
             if (mine) {
-                for (int t4 = 0; t4 < n_tile; t4 += 4) {
-                    // four sphere tests, each the reference's serial sum over the coordinates
-                    float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+                int next_t = 0;
+                while (next_t < n_tile) {
+                    // the first point from next_t on whose sphere (or self test) takes the hit: four
+                    // tests per step, each the reference's serial sum over the coordinates. The lanes
+                    // of a wave leave this loop one by one; the complete test below then runs once
+                    // for all of them.
+                    int found = n_tile;
+                    for (int t4 = next_t & ~3; t4 < n_tile; t4 += 4) {
+                        float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
-                    for (int c = 0; c < CMAX; ++c) {
-                        const float4 cc = *reinterpret_cast<const float4 *>(&s_centre[c][t4]);
-                        float t = cc.x - xs[c];
-                        d0 = d0 + t * t;
-                        t = cc.y - xs[c];
-                        d1 = d1 + t * t;
-                        t = cc.z - xs[c];
-                        d2 = d2 + t * t;
-                        t = cc.w - xs[c];
-                        d3 = d3 + t * t;
-                    }
-                    const float4 rr = *reinterpret_cast<const float4 *>(&s_rsq[t4]);
-                    uint32_t hits = (d0 <= rr.x ? 1u : 0u) | (d1 <= rr.y ? 2u : 0u) | (d2 <= rr.z ? 4u : 0u) |
-                                    (d3 <= rr.w ? 8u : 0u);
-                    if (any_solitary) {
-                        const uint4 sk = *reinterpret_cast<const uint4 *>(&s_self[t4]);
-                        hits |= (sk.x == self_key ? 1u : 0u) | (sk.y == self_key ? 2u : 0u) |
-                                (sk.z == self_key ? 4u : 0u) | (sk.w == self_key ? 8u : 0u);
-                    }
-                    if (!hits) continue;
-                    // the complete test for those, in order
-                    for (int j = 0; j < 4; ++j) {
-                        if (!((hits >> j) & 1u)) continue;
-                        const uint32_t *a = s_tile + (size_t)(t4 + j) * aw;
-                        float dsq;
-                        if (!covers<CMAX>(a, x, uncoverable, self_q, k, dsq)) continue;
-                        if (MODE == 2) {
-                            const float lhs = best * __uint_as_float(a[CMAX]);
-                            if (!(lhs >= dsq)) continue;
-                            best = dsq;
+                        for (int c = 0; c < CMAX; ++c) {
+                            const float4 cc = *reinterpret_cast<const float4 *>(&s_centre[c][t4]);
+                            float t = cc.x - xs[c];
+                            d0 = d0 + t * t;
+                            t = cc.y - xs[c];
+                            d1 = d1 + t * t;
+                            t = cc.z - xs[c];
+                            d2 = d2 + t * t;
+                            t = cc.w - xs[c];
+                            d3 = d3 + t * t;
                         }
-                        shower = base + t4 + j;
-                        asso = (int)a[CMAX + 2];
-                        if (MODE != 2) {
-                            mine = alive = false;
+                        const float4 rr = *reinterpret_cast<const float4 *>(&s_rsq[t4]);
+                        uint32_t hits = (d0 <= rr.x ? 1u : 0u) | (d1 <= rr.y ? 2u : 0u) | (d2 <= rr.z ? 4u : 0u) |
+                                        (d3 <= rr.w ? 8u : 0u);
+                        if (any_solitary) {
+                            const uint4 sk = *reinterpret_cast<const uint4 *>(&s_self[t4]);
+                            hits |= (sk.x == self_key ? 1u : 0u) | (sk.y == self_key ? 2u : 0u) |
+                                    (sk.z == self_key ? 4u : 0u) | (sk.w == self_key ? 8u : 0u);
+                        }
+                        if (MODE == 2) {
+                            // every point that covers the hit takes part in the running comparison
+                            for (int j = 0; j < 4; ++j) {
+                                if (!((hits >> j) & 1u)) continue;
+                                const uint32_t *a = s_tile + (size_t)(t4 + j) * aw;
+                                float dsq;
+                                if (!covers<CMAX>(a, x, uncoverable, self_q, k, dsq)) continue;
+                                const float lhs = best * __uint_as_float(a[CMAX]);
+                                if (!(lhs >= dsq)) continue;
+                                best = dsq;
+                                shower = base + t4 + j;
+                                asso = (int)a[CMAX + 2];
+                            }
+                            continue;
+                        }
+                        if (t4 < next_t) hits &= ~((1u << (next_t - t4)) - 1u);
+                        if (hits) {
+                            found = t4 + __builtin_ctz(hits);
                             break;
                         }
                     }
-                    if (!mine) break;
+                    if (found >= n_tile) break;
+                    next_t = found + 1;
+                    // the complete test for that one
+                    const uint32_t *a = s_tile + (size_t)found * aw;
+                    float dsq;
+                    if (!covers<CMAX>(a, x, uncoverable, self_q, k, dsq)) continue;
+                    shower = base + found;
+                    asso = (int)a[CMAX + 2];
+                    mine = alive = false;
+                    break;
                 }
             }
         }
