@@ -1,7 +1,8 @@
 """Seeded sweep over random shapes and option combinations: every op of the path
 on the GPU against the oracle (kNN options incl. radius x tf_compatible x
 direction, ragged events, lattice ties; accumulate forward / gradient / PushKnn /
-distance gradient over the resulting tables; condensates with per-hit radii)."""
+distance gradient over the resulting tables; condensates with per-hit radii, masks,
+ties and 1-9 coordinates)."""
 import numpy as np
 import pytest
 
@@ -113,3 +114,54 @@ def test_random_knn_long_lists_and_dense_blobs(oracle, seed):
     kw = {} if radius is None else {"radius": radius}
     assert check_knn_rows(oracle, gi, gd, coords, rs, K, differ, **kw) == len(differ)
     assert len(differ) <= n // 100
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_condensates(oracle, seed):
+    """condensate assignment over random sizes, 1-9 coordinates, 1-4 binned dimensions, uniform /
+    normal / lattice / clustered hits, beta with ties, radii from tiny to half the extent (per hit
+    or common), distance thresholds, sparse to full no_condensation_mask, both assignment modes"""
+    from hgcalml_amd import BuildAndAssignCondensatesBinned
+    rng = np.random.default_rng(5000 + seed)
+    n = int(rng.choice([rng.integers(1, 60), rng.integers(60, 3000), rng.integers(3000, 40000)]))
+    C = int(rng.integers(1, 10))
+    nbin_dims = int(rng.integers(1, 5))
+    n_ev = int(rng.integers(1, 6))
+    rs = np.concatenate([[0], np.sort(rng.integers(0, n + 1, n_ev - 1)), [n]]).astype(np.int32)
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        x = rng.random((n, C), dtype=np.float32)
+    elif kind == 1:
+        x = rng.standard_normal((n, C)).astype(np.float32)
+    elif kind == 2:
+        x = rng.integers(0, 4, (n, C)).astype(np.float32)  # distance ties, coincident hits
+    else:
+        k = max(1, n // 50)
+        centres = rng.random((k, C)) * 2 - 1
+        x = (centres[rng.integers(0, k, n)] + 0.03 * rng.standard_normal((n, C))).astype(np.float32)
+    beta_kind = int(rng.integers(0, 3))
+    if beta_kind == 0:
+        beta = rng.random((n, 1), dtype=np.float32)
+    elif beta_kind == 1:
+        beta = (rng.integers(0, 8, (n, 1)) / 8).astype(np.float32)
+    else:
+        beta = np.clip(rng.beta(0.5, 2, (n, 1)) + 0.5 * (rng.random((n, 1)) < 0.3), 0, 0.999).astype(np.float32)
+    # radii relative to the extent: the reference's box walk counts its cells in an int
+    extent = max(1e-3, float((x.max(0) - x.min(0)).max()))
+    scale = float(rng.choice([0.001, 0.02, 0.1, 0.2, 0.3, 0.5])) * extent
+    dist = (scale * (0.5 + rng.random((n, 1)))).astype(np.float32)
+    if rng.random() < 0.3:
+        dist[:] = scale
+    threshold = float(rng.choice([0.5, 1.0, 0.7, 2.0]))
+    t_b = float(rng.choice([0.0, 1e-5, 0.1, 0.5, 0.95]))
+    mask = None
+    if rng.random() < 0.5:
+        mask = (rng.random((n, 1)) < float(rng.choice([0.001, 0.02, 0.3, 1.0]))).astype(np.int32)
+    kw = dict(distance_threshold=threshold, assign_by_max_beta=bool(rng.integers(0, 2)), nbin_dims=nbin_dims)
+    ref = oracle.BuildAndAssignCondensatesBinned(x, beta, dist, rs, t_b, no_condensation_mask=mask, **kw)
+    got = BuildAndAssignCondensatesBinned(t(x), t(beta), t(dist), t(rs), t_b,
+                                          no_condensation_mask=None if mask is None else t(mask), **kw)
+    for name, a, b in zip(("assignment", "association", "alpha_idx", "is_cond", "n_condensates"), got, ref):
+        a = a.cpu().numpy()
+        assert a.shape == b.shape, name
+        assert (a == b).all(), name
