@@ -77,11 +77,24 @@ def test_host_side_argument_checks(capi):
     assert capi.hgc_sort_by_bin_workspace_bytes(150000, 27000) >= 2 * 150000 * 4
     # the sorted keys, plus whatever rocPRIM asks for itself
     assert capi.hgc_inverse_neighbour_index_workspace_bytes(1000, 64) >= 64000 * 4
+    # the one-call condensate wrapper: sizes checked on the host, the empty input needs no workspace
+    capi.hgc_build_and_assign_condensates_workspace_bytes.restype = ctypes.c_size_t
+    assert capi.hgc_build_and_assign_condensates_workspace_bytes(1000, 4, 2, 6, 3) > 1000 * 4 * 4
+    assert capi.hgc_build_and_assign_condensates_workspace_bytes(1000, 17, 2, 6, 3) == 0
+    c = capi.hgc_build_and_assign_condensates
+    c.argtypes = ([ctypes.c_void_p] * 5 + [ctypes.c_int] * 3 + [ctypes.c_float] * 2 + [ctypes.c_int] * 3 +
+                  [ctypes.c_void_p] * 6 + [ctypes.c_size_t, ctypes.c_void_p])
+    one = ctypes.c_void_p(256)
+    assert c(one, one, one, null, one, 10, 17, 1, 0.1, 1.0, 1, 3, 5, one, one, one, one, one, null, 0, null) == -1
+    assert b"coordinate dimensions" in capi.hgc_last_error()
+    assert c(one, one, one, null, one, 10, 4, 1, 0.1, 1.0, 1, 0, 5, one, one, one, one, one, null, 0, null) == -1
+    assert c(one, one, one, null, one, 10, 4, 1, 0.1, 0.0, 1, 3, 5, one, one, one, one, one, null, 0, null) == -1
+    assert b"distance_threshold" in capi.hgc_last_error()
+    assert c(one, one, one, null, one, 10, 4, 1, 0.1, 1.0, 1, 3, 5, one, one, one, one, one, null, 0, null) == -2
     # missing workspace is reported, not dereferenced
     h = capi.hgc_sort_by_bin
     h.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                   ctypes.c_size_t, ctypes.c_void_p]
-    one = ctypes.c_void_p(256)
     assert h(one, 10, 10, one, one, null, 0, null) == -2
 
 
