@@ -338,8 +338,11 @@ int hgc_probe_row_gather(const float *d_feat, const int *d_idxs, float *d_out,
  *   (original indices of the condensate points per event, -1 padded).
  *   d_condensates_assigned_h [n_vert_h] and d_assignment_min_distance [n_vert]
  *   (the latter only if !assign_by_max_beta) are caller scratch like in the
- *   reference. d_error (may be NULL) receives 1 if an event made no progress
- *   (the reference throws std::runtime_error there). */
+ *   reference. d_error (may be NULL) is set to 0: the loop that could stall in
+ *   the reference (it throws std::runtime_error there) does not exist here.
+ *   The two views of the hits must agree as the reference wrapper builds them:
+ *   d_indices_to_filtered[i] = q exactly for the hit i that entry q of the *_h
+ *   arrays was taken from (same coordinates and mask), -1 for the others. */
 size_t hgc_binned_assign_to_condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows);
 int hgc_binned_assign_to_condensates(int dimensions, int dimensions_binning,
                                      int *d_condensates_assigned_h,
