@@ -38,9 +38,13 @@
  *   hgo_push_knn             pinned: ordered unbuffered scatter-add (bitwise).
  *   hgo_push_knn_grad        pinned: float64 autograd of that scatter-add.
  *   hgo_local_distance       pinned: the brute-force serial fp32 distance.
- *   hgo_assign_to_condensates pinned for an all-zero no_condensation_mask by a
- *                            bin-free sequential greedy; behaviour with a
- *                            non-zero mask is "parity unpinned".
+ *   hgo_assign_to_condensates pinned by a bin-free sequential greedy written from
+ *                            the reference text, without and with a
+ *                            no_condensation_mask (incl. masks on the first two
+ *                            high-beta entries, which switch the pick order).
+ *                            That both restate the reference's mask indexing
+ *                            the same way is all that pins it: "parity
+ *                            unpinned" against the compiled reference there.
  *
  * Build: gcc -O2 -ffp-contract=off -shared -fPIC (see oracle/Makefile).
  * All fp32 arithmetic is written as separate multiplies and adds, in the

@@ -307,40 +307,73 @@ def test_accumulate_grad_summation_order_and_self_rule(oracle):
 
 # ------------------------------------------------------------------ condensates
 
-def bin_free_greedy(oracle, cfg, by_max_beta):
+def stable_bin_positions(oracle, cfg):
+    """position of every hit in the wrapper's stable bin order (what breaks ties between equal betas)"""
+    cc = cfg["ccoords"].astype(np.float32)
+    n = len(cc)
+    cc = cc - cc.min(0, keepdims=True)
+    n_bins_sc = max(4, min(int(np.ceil((n / 5) ** (1 / 3))), 25))
+    _, flat, _, _ = oracle.BinByCoordinates(cc[:, :3], cfg["row_splits"], n_bins=n_bins_sc, calc_n_per_bin=False,
+                                            pre_normalized=True)
+    pos = np.empty(n, np.int64)
+    pos[np.argsort(flat, kind="stable")] = np.arange(n)
+    return pos
+
+
+def bin_free_greedy(oracle, cfg, by_max_beta, mask=None):
+    """The reference's loop without bins, written from its text
+    (binned_assign_to_condensates_kernel.cc:23-125 claim, :180-226 pick): every pick scans the
+    unclaimed high-beta hits in position order; the no_condensation_mask of the high-beta subset
+    is indexed with the truth value of (index > 0), and an entry that is set there ends the scan at
+    the first unclaimed hit. A masked pick claims only itself; a masked hit is claimed by nobody else."""
     cc = cfg["ccoords"].astype(np.float32)
     beta = cfg["betas"].reshape(-1)
     rad = (cfg["dist"].reshape(-1) / np.float32(cfg["distance_threshold"])).astype(np.float32)
     rs = cfg["row_splits"]
     n = len(beta)
+    mask = np.zeros(n, np.int32) if mask is None else np.asarray(mask).reshape(-1).astype(np.int32)
     cc = cc - cc.min(0, keepdims=True)
-    # the position tie-break needs the stable bin order; take it from the binning oracle
-    n_bins_sc = max(4, min(int(np.ceil((n / 5) ** (1 / 3))), 25))
-    _, flat, _, _ = oracle.BinByCoordinates(cc[:, :3], rs, n_bins=n_bins_sc, calc_n_per_bin=False,
-                                            pre_normalized=True)
-    pos = np.empty(n, np.int64)
-    pos[np.argsort(flat, kind="stable")] = np.arange(n)
+    pos = stable_bin_positions(oracle, cfg)
+    is_high = (beta > np.float32(cfg["beta_threshold"])) | (mask > 0)
+    # the filtered arrays: high-beta hits in position order, events one after the other
+    filtered = np.concatenate([
+        (np.arange(rs[e], rs[e + 1])[is_high[rs[e]:rs[e + 1]]])[np.argsort(pos[rs[e]:rs[e + 1]][is_high[rs[e]:rs[e + 1]]],
+                                                                              kind="stable")]
+        for e in range(len(rs) - 1)]).astype(np.int64)
+    mask_h = mask[filtered]
     assignment = np.full(n, -1, np.int32)
     asso = np.full(n, -1, np.int32)
     alphas, ncond = [], [0]
+    q0 = 0
     for e in range(len(rs) - 1):
         lo, hi = rs[e], rs[e + 1]
-        members = np.arange(lo, hi)
-        high = members[beta[lo:hi] > np.float32(cfg["beta_threshold"])]
-        order = high[np.lexsort((pos[high], -beta[high].astype(np.float64)))]
-        taken = np.zeros(n, bool)
+        mine = filtered[(filtered >= lo) & (filtered < hi)]    # this event's entries, global index q0 + i
+        taken = np.zeros(len(mine), bool)
+        claimed = np.zeros(n, bool)
         best = np.full(n, np.float32(10e20), np.float32)
         shower = 0
-        for a in order:
-            if taken[a]:
-                continue
-            taken[a] = True
+        while True:
+            biggest, pick = np.float32(-1), -1
+            for i in np.nonzero(~taken)[0]:
+                q = q0 + i
+                if q < len(mask_h) and (1 if q > 0 else 0) < len(mask_h) and mask_h[1 if q > 0 else 0]:
+                    pick, biggest = i, np.float32(0)
+                    break
+                if beta[mine[i]] > biggest:
+                    biggest, pick = beta[mine[i]], i
+            if biggest == np.float32(-1):
+                break
+            a = mine[pick]
+            taken[pick] = True
             d = np.zeros(hi - lo, np.float32)
             for c in range(cc.shape[1]):
                 t = (cc[a, c] - cc[lo:hi, c]).astype(np.float32)
                 d = (d + (t * t).astype(np.float32)).astype(np.float32)
             rsq = np.float32(rad[a] * rad[a])
-            inside = d <= rsq
+            if mask[a] > 0:
+                inside = np.arange(lo, hi) == a
+            else:
+                inside = (d <= rsq) & (mask[lo:hi] == 0)
             if by_max_beta:
                 claim = inside & (assignment[lo:hi] == -1)
             else:
@@ -348,10 +381,12 @@ def bin_free_greedy(oracle, cfg, by_max_beta):
                 best[lo:hi] = np.where(claim, d, best[lo:hi])
             assignment[lo:hi] = np.where(claim, shower, assignment[lo:hi])
             asso[lo:hi] = np.where(claim, a, asso[lo:hi])
-            taken[lo:hi] |= claim
+            claimed[lo:hi] |= claim
+            taken |= claimed[mine]
             alphas.append(a)
             shower += 1
         ncond.append(ncond[-1] + shower)
+        q0 += len(mine)
     return assignment, asso, np.array(alphas, np.int32), np.array(ncond, np.int32)
 
 
@@ -511,6 +546,44 @@ def test_condensates_vs_bin_free_greedy(oracle, by_max_beta, t_d):
     assert (ncond == np.concatenate([[0], np.cumsum(per_event_max)])).all()
     for e in range(len(rs) - 1):
         assert (assignment[alpha[ncond[e]:ncond[e + 1]], 0] == np.arange(ncond[e + 1] - ncond[e])).all()
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
+@pytest.mark.parametrize("case", ["sparse", "first", "second", "first two", "dense"])
+def test_condensates_with_mask_vs_bin_free_greedy(oracle, by_max_beta, case):
+    """no_condensation_mask: sparse and dense random masks, and masks on the first / second entry of
+    the high-beta subset, which switch the reference's pick loop to position order (its index
+    expression `mask_h[offset + i > 0]`)"""
+    cfg = workloads.cfg5(scale=0.016, n_events=3)   # 3 x 1000 hits
+    rng = np.random.default_rng(12)
+    cfg["dist"] = (0.3 * rng.uniform(0.6, 1.4, size=cfg["dist"].shape)).astype(np.float32)
+    n = len(cfg["betas"])
+    pos = stable_bin_positions(oracle, cfg)
+    high = cfg["betas"].reshape(-1) > np.float32(cfg["beta_threshold"])
+    first_two = np.argsort(np.where(high[:cfg["row_splits"][1]], pos[:cfg["row_splits"][1]], n))[:2]
+    mask = np.zeros(n, np.int32)
+    if case == "sparse":
+        mask[rng.random(n) < 0.02] = 1
+        mask[first_two] = 0
+    elif case == "dense":
+        mask[rng.random(n) < 0.4] = 1
+    elif case == "first":
+        mask[first_two[0]] = 1
+    elif case == "second":
+        mask[first_two[1]] = 1
+    else:
+        mask[first_two] = 1
+    assignment, asso, alpha, is_cond, ncond = oracle.BuildAndAssignCondensatesBinned(
+        cfg["ccoords"], cfg["betas"], cfg["dist"], cfg["row_splits"], cfg["beta_threshold"],
+        no_condensation_mask=mask[:, None], assign_by_max_beta=by_max_beta)
+    r_assignment, r_asso, r_alpha, r_ncond = bin_free_greedy(oracle, cfg, by_max_beta, mask=mask)
+    assert (ncond == r_ncond).all()
+    assert (alpha == r_alpha).all()
+    assert (assignment[:, 0] == r_assignment).all()
+    assert (asso == r_asso).all()
+    # a masked hit is its own condensation point
+    masked = np.nonzero(mask)[0]
+    assert (asso[masked] == masked).all() and is_cond[masked, 0].all()
 
 
 @pytest.mark.parametrize("t_b", [1e-5, 0.1, 0.9999])
