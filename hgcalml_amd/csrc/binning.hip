@@ -305,26 +305,24 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
     }
 }
 
-// position of every point in bin order
-__global__ __launch_bounds__(256) void place_in_bin_order_kernel(const int *__restrict__ flat,
-                                                                 const int *__restrict__ rank,
-                                                                 const int *__restrict__ boundaries, int n_vert,
-                                                                 int sub_shift, int *__restrict__ sorting) {
-    const int p = blockIdx.x * blockDim.x + threadIdx.x;
-    if (p < n_vert)
-        sorting[boundaries[((size_t)flat[p] << sub_shift) | (p & ((1 << sub_shift) - 1))] + rank[p]] = p;
-}
-
-// the inputs in bin order: row `at` of every output is row sorting[at] of its input
-__global__ __launch_bounds__(256) void gather_bin_order_kernel(
+// position of every point in bin order, and its inputs moved there: row `at` of every
+// output is row sorting[at] of its input
+__global__ __launch_bounds__(256) void move_to_bin_order_kernel(
     const float *__restrict__ coords, const int *__restrict__ binass, const int *__restrict__ flat,
-    const int *__restrict__ direction, const int *__restrict__ sorting, int n_vert, int n_coords, int n_dims,
+    const int *__restrict__ rank, const int *__restrict__ direction, const int *__restrict__ boundaries, int n_vert,
+    int n_coords, int n_dims, int sub_shift, int rows_aligned, int *__restrict__ sorting,
     float *__restrict__ scoords, int *__restrict__ sflat, int *__restrict__ sbinass, int *__restrict__ sdir) {
-    const int at = blockIdx.x * blockDim.x + threadIdx.x;
-    if (at >= n_vert) return;
-    const int p = sorting[at];
-    sflat[at] = flat[p];
-    for (int c = 0; c < n_coords; ++c) scoords[(size_t)at * n_coords + c] = coords[(size_t)p * n_coords + c];
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_vert) return;
+    const int cell = flat[p];
+    const int at = boundaries[((size_t)cell << sub_shift) | (p & ((1 << sub_shift) - 1))] + rank[p];
+    sorting[at] = p;
+    sflat[at] = cell;
+    if (n_coords == 4 && rows_aligned) {
+        reinterpret_cast<float4 *>(scoords)[at] = reinterpret_cast<const float4 *>(coords)[p];
+    } else {
+        for (int c = 0; c < n_coords; ++c) scoords[(size_t)at * n_coords + c] = coords[(size_t)p * n_coords + c];
+    }
     for (int c = 0; c <= n_dims; ++c) sbinass[(size_t)at * (n_dims + 1) + c] = binass[(size_t)p * (n_dims + 1) + c];
     if (direction) sdir[at] = direction[p];
 }
@@ -397,14 +395,13 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
     if (rc) return rc;
     // boundaries[b << sub_shift] = number of points in bins below b
     HGC_HIP(rocprim::exclusive_scan(temp, temp_bytes, counts, d_boundaries, 0, n_counters, rocprim::plus<int>(), s));
-    place_in_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(flat, rank, d_boundaries, n_vert, sub_shift,
-                                                                    d_sorting);
-    rc = check_launch("place_in_bin_order");
-    if (rc) return rc;
-    gather_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, binass, flat, d_direction, d_sorting, n_vert,
-                                                                  n_coords, n_bin_dims, d_scoords, d_sflat, d_sbinass,
-                                                                  d_sdir);
-    return check_launch("gather_bin_order");
+    const int rows_aligned =
+        ((reinterpret_cast<uintptr_t>(d_coords) | reinterpret_cast<uintptr_t>(d_scoords)) & 15u) == 0;
+    move_to_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, binass, flat, rank, d_direction,
+                                                                   d_boundaries, n_vert, n_coords, n_bin_dims,
+                                                                   sub_shift, rows_aligned, d_sorting, d_scoords,
+                                                                   d_sflat, d_sbinass, d_sdir);
+    return check_launch("move_to_bin_order");
 }
 
 }  // namespace hgc
