@@ -31,6 +31,21 @@ class _AccumulateFn(torch.autograd.Function):
         return gw, gx, None, None
 
 
+class _ExpNegFn(torch.autograd.Function):
+    """weights = exp(-distances) (modules/accknn_op.py:86) and its chain rule, one kernel each"""
+
+    @staticmethod
+    def forward(ctx, distances):
+        weights = ops.exp_neg(distances)
+        ctx.save_for_backward(weights)
+        return weights
+
+    @staticmethod
+    def backward(ctx, grad_weights):
+        weights, = ctx.saved_tensors
+        return ops.exp_neg_grad(grad_weights.contiguous(), weights)
+
+
 def _torch_composition(weights, features, indices, mean_and_max):
     # the reference's pure-TF path (modules/accknn_op.py:27-36): padded slots
     # contribute 0 to the mean and to the max
@@ -57,10 +72,10 @@ def AccumulateKnn(distances, features, indices, mean_and_max=True, force_tf=Fals
 
     Returns (out [N, 2F] (mean | max) or [N, F], arg-max neighbour index [N, F]).
     """
-    weights = torch.exp(-distances)
     if (not gl.acc_ops_use_tf_gradients) and (not force_tf):
+        weights = _ExpNegFn.apply(distances) if distances.dtype == torch.float32 else torch.exp(-distances)
         return _AccumulateFn.apply(weights, features, indices, bool(mean_and_max))
-    return _torch_composition(weights, features, indices, mean_and_max)
+    return _torch_composition(torch.exp(-distances), features, indices, mean_and_max)
 
 
 def _sumw(acc, x, features, indices, mean_and_max):

@@ -216,6 +216,34 @@ int launch_push_grad_wave(const float *grad, const float *w, const float *feat, 
 
 using namespace hgc;
 
+namespace {
+
+// weights of AccumulateKnn, w = exp(-d) (modules/accknn_op.py:86), and the chain rule back to
+// the distances, gd = -(gw * w): one pass each instead of two framework kernels
+__global__ __launch_bounds__(256) void exp_neg_kernel(const float *__restrict__ d, float *__restrict__ w,
+                                                      long long n) {
+    const long long i = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i + 4 <= n) {
+        const float4 v = *reinterpret_cast<const float4 *>(d + i);
+        *reinterpret_cast<float4 *>(w + i) = float4{expf(-v.x), expf(-v.y), expf(-v.z), expf(-v.w)};
+    } else {
+        for (long long j = i; j < n; ++j) w[j] = expf(-d[j]);
+    }
+}
+
+__global__ __launch_bounds__(256) void exp_neg_grad_kernel(const float *__restrict__ gw, const float *__restrict__ w,
+                                                           float *__restrict__ gd, long long n) {
+    const long long i = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i + 4 <= n) {
+        const float4 a = *reinterpret_cast<const float4 *>(gw + i), b = *reinterpret_cast<const float4 *>(w + i);
+        *reinterpret_cast<float4 *>(gd + i) = float4{-(a.x * b.x), -(a.y * b.y), -(a.z * b.z), -(a.w * b.w)};
+    } else {
+        for (long long j = i; j < n; ++j) gd[j] = -(gw[j] * w[j]);
+    }
+}
+
+}  // namespace
+
 extern "C" {
 
 int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const float *d_dist, const float *d_coord,
@@ -277,6 +305,30 @@ int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *
     // vertex's own row (feat) and the gathered rows (grad) as in the accumulation's
     return accumulate_gradient(d_feat, nullptr, d_grad, nullptr, nullptr, d_idxs, nullptr, nullptr, d_w_grad, nullptr,
                                n_vert, n_neigh, n_feat, n_feat, 0, 1.f, nullptr, stream);
+}
+
+int hgc_exp_neg(const float *d_distances, float *d_weights, long long n_values, hgc_stream_t stream) {
+    HGC_REQUIRE(n_values >= 0, "bad sizes");
+    if (n_values == 0) return HGC_OK;
+    HGC_REQUIRE(d_distances && d_weights, "null pointer");
+    HGC_REQUIRE(((reinterpret_cast<uintptr_t>(d_distances) | reinterpret_cast<uintptr_t>(d_weights)) & 15u) == 0,
+                "arrays must start on a 16-byte boundary");
+    exp_neg_kernel<<<ceil_div(ceil_div(n_values, 4), 256), 256, 0, as_stream(stream)>>>(d_distances, d_weights,
+                                                                                       n_values);
+    return check_launch("exp_neg");
+}
+
+int hgc_exp_neg_grad(const float *d_weight_grad, const float *d_weights, float *d_distance_grad, long long n_values,
+                     hgc_stream_t stream) {
+    HGC_REQUIRE(n_values >= 0, "bad sizes");
+    if (n_values == 0) return HGC_OK;
+    HGC_REQUIRE(d_weight_grad && d_weights && d_distance_grad, "null pointer");
+    HGC_REQUIRE(((reinterpret_cast<uintptr_t>(d_weight_grad) | reinterpret_cast<uintptr_t>(d_weights) |
+                  reinterpret_cast<uintptr_t>(d_distance_grad)) & 15u) == 0,
+                "arrays must start on a 16-byte boundary");
+    exp_neg_grad_kernel<<<ceil_div(ceil_div(n_values, 4), 256), 256, 0, as_stream(stream)>>>(
+        d_weight_grad, d_weights, d_distance_grad, n_values);
+    return check_launch("exp_neg_grad");
 }
 
 }  // extern "C"

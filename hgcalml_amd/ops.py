@@ -455,3 +455,27 @@ def build_and_assign_condensates(ccoords, betas, dist, mask, row_splits, beta_th
     total = int(ncond[-1]) if n > 0 else 0
     return assignment, asso, alpha[:total], is_cond, ncond
 
+
+def exp_neg(distances):
+    """exp(-distances) in one pass"""
+    require_device(distances)
+    d = f32(distances)
+    if d.data_ptr() % 16:
+        d = d.clone()
+    w = torch.empty_like(d)
+    check(lib.hgc_exp_neg(p(d), p(w), d.numel(), stream()))
+    return w
+
+
+def exp_neg_grad(weight_grad, weights):
+    """-(weight_grad * weights): the gradient of exp(-d) w.r.t. d"""
+    require_device(weight_grad, weights)
+    g, w = f32(weight_grad), f32(weights)
+    if g.data_ptr() % 16:
+        g = g.clone()
+    if w.data_ptr() % 16:
+        w = w.clone()
+    out = torch.empty_like(w)
+    check(lib.hgc_exp_neg_grad(p(g), p(w), p(out), w.numel(), stream()))
+    return out
+

@@ -313,6 +313,14 @@ int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *
                       const int *d_idxs, float *d_feat_grad, float *d_w_grad,
                       int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
 
+/* The elementwise glue of the AccumulateKnn wrapper (modules/accknn_op.py:86,
+ * `tf.exp(-distsq)`) and of its gradient, one pass each: d_weights[i] =
+ * exp(-d_distances[i]); d_distance_grad[i] = -(d_weight_grad[i] * d_weights[i]).
+ * Arrays of n_values floats on 16-byte boundaries. */
+int hgc_exp_neg(const float *d_distances, float *d_weights, long long n_values, hgc_stream_t stream);
+int hgc_exp_neg_grad(const float *d_weight_grad, const float *d_weights, float *d_distance_grad,
+                     long long n_values, hgc_stream_t stream);
+
 /* Measurement aid without a counterpart in the reference: out[v,:] = sum over
  * the K rows d_feat[d_idxs[v,n],:] with the forward kernel's access pattern and
  * no other arithmetic. Its run time is the rate at which the memory system

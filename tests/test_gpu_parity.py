@@ -843,6 +843,26 @@ def test_refused_arguments():
     assert rc == -1 and b"n_out_feat" in lib.hgc_last_error()
 
 
+def test_accumulate_knn_weights_and_their_gradient_in_one_pass():
+    """exp(-d) and -(g*w) of the AccumulateKnn wrapper: the library's one-pass kernels return the
+    bits of the framework's elementwise ops, for sizes that are no multiple of four and views that
+    do not start on a 16-byte boundary"""
+    from hgcalml_amd import ops
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    for n in (1, 3, 64, 1001, 150000 * 64 + 3):
+        d = (torch.rand(n + 1, device=DEV, generator=gen) * 30 - 2)[1:]
+        w = ops.exp_neg(d)
+        assert (w.view(torch.int32) == torch.exp(-d).view(torch.int32)).all()
+        g = torch.randn(n + 1, device=DEV, generator=gen)[1:]
+        assert (ops.exp_neg_grad(g, w).view(torch.int32) == (-(g * w)).view(torch.int32)).all()
+    assert ops.exp_neg(torch.empty(0, device=DEV)).numel() == 0
+    d = torch.rand(50, 7, device=DEV, generator=gen).requires_grad_(True)
+    from hgcalml_amd.accknn_op import _ExpNegFn
+    w = _ExpNegFn.apply(d)
+    w.backward(torch.ones_like(w))
+    assert torch.equal(d.grad, -torch.exp(-d.detach()))
+
+
 # ------------------------------------------------------------------ condensates
 
 def run_condensates(oracle, cfg, by_max_beta, mask=None):
