@@ -884,6 +884,29 @@ def run_condensates(oracle, cfg, by_max_beta, mask=None):
     return got
 
 
+@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensate_op_on_the_reference_wrappers_arrays(oracle, by_max_beta, masked):
+    """the op itself (modules/compiled/binned_assign_to_condensates_module.cc:7-31) on the arrays
+    the reference wrapper hands it: bin-sorted hits plus the filtered high-beta copy"""
+    cfg = workloads.cfg5(scale=0.1, n_events=3)
+    mask = None
+    if masked:
+        mask = (np.random.default_rng(27).random(len(cfg["betas"])) < 0.03).astype(np.int32)[:, None]
+    _, k = oracle.BuildAndAssignCondensatesBinned(cfg["ccoords"], cfg["betas"], cfg["dist"], cfg["row_splits"],
+                                                  cfg["beta_threshold"], no_condensation_mask=mask,
+                                                  assign_by_max_beta=by_max_beta, return_kernel_inputs=True)
+    want = oracle.assign_to_condensates_kernel(**k)
+    bins_flat = np.zeros(len(k["beta"]), np.int32)  # carried by the op, not read
+    got = torch.ops.hgcalml.binned_assign_to_condensates(
+        t(k["ccoords"]), t(k["dist"]), t(k["beta"]), t(k["mask"]), t(bins_flat), t(k["bin_splits"]),
+        t(k["to_filtered"]), t(k["orig_h"]), t(k["row_splits"]), t(k["n_bins"]), t(np.reshape(k["bin_width"], [1])),
+        t(k["ccoords_h"]), t(k["dist_h"]), t(k["beta_h"]), t(k["mask_h"]), t(k["row_splits_h"]),
+        float(cfg["beta_threshold"]), bool(by_max_beta))
+    for name, g, w in zip(("is_alpha_h", "assignment", "alpha_indices", "association", "n_condensates"), got, want):
+        assert (g.cpu().numpy() == w).all(), name
+
+
 @pytest.mark.parametrize("by_max_beta", [True, False])
 def test_condensates_cfg5_scaled(oracle, by_max_beta):
     cfg = workloads.cfg5(scale=0.1)
