@@ -74,6 +74,7 @@ class RaggedGravNet(nn.Module):
         # same vertices row by row, so the kNN's processing order applies to it too
         nidx, ndist = idx[:, 1:].contiguous(), dist[:, 1:].contiguous()
         ops.share_vertex_order(idx, nidx)
+        ops.declare_without_first_column(nidx, idx)
         if self.return_self:
             return nidx, ndist, idx, dist
         return nidx, ndist, None, None

@@ -37,6 +37,8 @@ _SIGNATURES = {
     "hgc_accumulate_knn_slots": (_c_int, [_ptr] * 7 + [_c_int] * 6 + [_ptr]),
     "hgc_inverse_neighbour_index_workspace_bytes": (_c_size, [_c_int, _c_int]),
     "hgc_inverse_neighbour_index": (_c_int, [_ptr, _c_int, _c_int, _ptr, _ptr, _ptr, _c_size, _ptr]),
+    "hgc_inverse_index_without_first_column_workspace_bytes": (_c_size, [_c_int]),
+    "hgc_inverse_index_without_first_column": (_c_int, [_ptr, _ptr, _c_int, _c_int, _ptr, _ptr, _ptr, _c_size, _ptr]),
     "hgc_accumulate_knn_grad": (_c_int, [_ptr] * 9 + [_c_int] * 6 + [_ptr]),
     "hgc_accumulate_knn_grad_slots": (_c_int, [_ptr] * 11 + [_c_int] * 6 + [_ptr]),
     "hgc_select_knn_grad": (_c_int, [_ptr] * 7 + [_c_int] * 3 + [_ptr]),

@@ -535,6 +535,48 @@ __global__ __launch_bounds__(256) void inverse_offsets_kernel(const unsigned int
     offsets[m] = (int)lo;
 }
 
+// The inverse index of a neighbour table without its first column, from the inverse
+// index of the whole table: the entries of column 0 leave every target's list and
+// flat slot v*K+n becomes v*(K-1)+n-1. One wave per target, its list across the lanes.
+__global__ __launch_bounds__(256) void first_column_entries_kernel(const int *__restrict__ inv_off,
+                                                                   const int *__restrict__ inv_slots, int n_vert,
+                                                                   const acc::FastDiv div_k, int K,
+                                                                   int *__restrict__ dropped) {
+    const int m = blockIdx.x * (blockDim.x / kWave) + (int)(threadIdx.x / kWave);
+    if (m > n_vert) return;
+    int count = 0;
+    if (m < n_vert) {
+        const int begin = inv_off[m], end = inv_off[m + 1];
+        for (int e = begin + lane_id(); e - lane_id() < end; e += kWave) {
+            const int slot = e < end ? inv_slots[e] : 1;
+            count += __popcll(__ballot(e < end && slot - acc::fast_div(slot, div_k) * K == 0));
+        }
+    }
+    if (lane_id() == 0) dropped[m] = count;
+}
+
+__global__ __launch_bounds__(256) void drop_first_column_kernel(const int *__restrict__ inv_off,
+                                                                const int *__restrict__ inv_slots,
+                                                                const int *__restrict__ dropped_before, int n_vert,
+                                                                const acc::FastDiv div_k, int K,
+                                                                int *__restrict__ out_off,
+                                                                int *__restrict__ out_slots) {
+    const int m = blockIdx.x * (blockDim.x / kWave) + (int)(threadIdx.x / kWave);
+    if (m > n_vert) return;
+    int at = inv_off[m] - dropped_before[m];
+    if (lane_id() == 0) out_off[m] = at;
+    if (m == n_vert) return;
+    const int begin = inv_off[m], end = inv_off[m + 1];
+    for (int e = begin + lane_id(); e - lane_id() < end; e += kWave) {
+        const int slot = e < end ? inv_slots[e] : 0;
+        const int v = acc::fast_div(slot, div_k), n = slot - v * K;
+        const bool keep = e < end && n != 0;
+        const uint64_t kept = __ballot(keep);
+        if (keep) out_slots[at + __popcll(kept & ((1ull << lane_id()) - 1ull))] = v * (K - 1) + n - 1;
+        at += __popcll(kept);
+    }
+}
+
 // ------------------------------------------------------------------ feature gradient
 
 // gfeat[m, f] = sum over (v, n) naming m, ascending, of ((g[v,f]/K)*w[v,n] + max part)
@@ -821,6 +863,41 @@ int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh, int 
                                       inverse_key_bits(n_vert), s));
     inverse_offsets_kernel<<<ceil_div((long long)n_vert + 1, 256), 256, 0, s>>>(keys_sorted, total, d_inv_offsets, n_vert);
     return check_launch("inverse_offsets");
+}
+
+size_t hgc_inverse_index_without_first_column_workspace_bytes(int n_vert) {
+    size_t temp = 0;
+    (void)rocprim::exclusive_scan(nullptr, temp, (const int *)nullptr, (int *)nullptr, 0, (size_t)std::max(n_vert, 0) + 1,
+                                  rocprim::plus<int>(), (hipStream_t) nullptr);
+    return align_up(temp) + 2 * align_up(((size_t)std::max(n_vert, 0) + 1) * sizeof(int));
+}
+
+int hgc_inverse_index_without_first_column(const int *d_inv_offsets, const int *d_inv_slots, int n_vert, int n_neigh,
+                                           int *d_out_offsets, int *d_out_slots, void *workspace,
+                                           size_t workspace_bytes, hgc_stream_t stream) {
+    HGC_REQUIRE(n_vert >= 0 && n_neigh >= 2, "needs a table of at least two columns");
+    HGC_REQUIRE(d_out_offsets, "null pointer");
+    hipStream_t s = as_stream(stream);
+    if (n_vert == 0) return launch_fill_i32(d_out_offsets, 0, 1, s);
+    HGC_REQUIRE(d_inv_offsets && d_inv_slots && d_out_slots, "null pointer");
+    if (!workspace || !aligned256(workspace) ||
+        workspace_bytes < hgc_inverse_index_without_first_column_workspace_bytes(n_vert))
+        return fail(HGC_ERR_WORKSPACE, "inverse index workspace missing, misaligned or too small");
+    Carver carve(workspace);
+    int *dropped = carve.take<int>((size_t)n_vert + 1);
+    int *dropped_before = carve.take<int>((size_t)n_vert + 1);
+    void *temp = carve.base + carve.used;
+    size_t temp_bytes = workspace_bytes - carve.used;
+    const int blocks = ceil_div((long long)n_vert + 1, 256 / kWave);
+    const acc::FastDiv div_k = acc::make_fast_div(n_neigh);
+    first_column_entries_kernel<<<blocks, 256, 0, s>>>(d_inv_offsets, d_inv_slots, n_vert, div_k, n_neigh, dropped);
+    int rc = check_launch("first_column_entries");
+    if (rc) return rc;
+    HGC_HIP(rocprim::exclusive_scan(temp, temp_bytes, dropped, dropped_before, 0, (size_t)n_vert + 1,
+                                    rocprim::plus<int>(), s));
+    drop_first_column_kernel<<<blocks, 256, 0, s>>>(d_inv_offsets, d_inv_slots, dropped_before, n_vert, div_k,
+                                                    n_neigh, d_out_offsets, d_out_slots);
+    return check_launch("drop_first_column");
 }
 
 }  // extern "C"

@@ -253,6 +253,26 @@ def inverse_neighbour_index(indices):
 _INVERSE_CACHE = {}
 
 
+def inverse_index_without_first_column(inverse, n, k):
+    """inverse index of table[:, 1:] from the inverse index of the [n, k] table"""
+    offsets, slots = inverse
+    dev = offsets.device
+    out_offsets = torch.empty((n + 1,), dtype=torch.int32, device=dev)
+    out_slots = torch.empty((max(n * (k - 1), 1),), dtype=torch.int32, device=dev)
+    ws = workspace(lib.hgc_inverse_index_without_first_column_workspace_bytes(n), dev)
+    check(lib.hgc_inverse_index_without_first_column(p(offsets), p(slots), n, k, p(out_offsets), p(out_slots), p(ws),
+                                                     ws.numel(), stream()))
+    return out_offsets, out_slots
+
+
+def declare_without_first_column(part, whole):
+    """`part` holds the columns 1.. of `whole` (GravNet drops the self column of its kNN result):
+    its inverse index is then derived from that of `whole`, which the distance gradient needs
+    anyway, instead of being sorted a second time. `part` keeps `whole` alive."""
+    if part.dim() == 2 and whole.dim() == 2 and part.shape[0] == whole.shape[0] and part.shape[1] + 1 == whole.shape[1]:
+        part._hgc_without_first_column_of = (whole, part._version, whole._version)
+
+
 def cached_inverse_neighbour_index(indices):
     """The inverse index depends only on the neighbour table; GravNet-style
     models run several accumulations (and their gradients) over one table, so
@@ -263,7 +283,21 @@ def cached_inverse_neighbour_index(indices):
         ref, version, ptr, value = hit
         if ref() is indices and version == indices._version and ptr == indices.data_ptr():
             return value
-    value = inverse_neighbour_index(indices)
+    # the same memory through another tensor object (autograd hands saved outputs back as new objects)
+    for ref, version, ptr, value in _INVERSE_CACHE.values():
+        other = ref()
+        if (other is not None and ptr == indices.data_ptr() == other.data_ptr() and other.shape == indices.shape
+                and other.stride() == indices.stride() and version == other._version == indices._version):
+            return value
+    value = None
+    declared = getattr(indices, "_hgc_without_first_column_of", None)
+    if declared is not None:
+        whole, part_version, whole_version = declared
+        if part_version == indices._version and whole_version == whole._version:
+            value = inverse_index_without_first_column(cached_inverse_neighbour_index(whole), whole.shape[0],
+                                                       whole.shape[1])
+    if value is None:
+        value = inverse_neighbour_index(indices)
     if len(_INVERSE_CACHE) > 64:
         for k in [k for k, v in _INVERSE_CACHE.items() if v[0]() is None]:
             del _INVERSE_CACHE[k]

@@ -233,6 +233,17 @@ int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh,
                                 int *d_inv_offsets, int *d_inv_slots,
                                 void *workspace, size_t workspace_bytes, hgc_stream_t stream);
 
+/* The inverse neighbour index of a table without its first column (GravNet
+ * drops the self column of the kNN result before it accumulates,
+ * modules/GravNetLayersRagged.py:3095-3283), derived from the index of the whole
+ * [n_vert, n_neigh] table in one pass instead of a second sort. No counterpart in
+ * the reference. d_out_offsets [n_vert+1], d_out_slots [n_vert*(n_neigh-1)]. */
+size_t hgc_inverse_index_without_first_column_workspace_bytes(int n_vert);
+int hgc_inverse_index_without_first_column(const int *d_inv_offsets, const int *d_inv_slots,
+                                           int n_vert, int n_neigh, int *d_out_offsets,
+                                           int *d_out_slots, void *workspace, size_t workspace_bytes,
+                                           hgc_stream_t stream);
+
 /* Gradients of hgc_accumulate_knn w.r.t. the weights and the features.
  * Replaces AccumulateKnnGradOpFunctor
  * (modules/compiled/accumulate_knn_grad_kernel.h, _kernel.cc:24-227); the

@@ -19,6 +19,13 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True, scope="module")
+def registered_ops():
+    """torch.ops.hgcalml.* exist once hgcalml_amd.ops is imported (the package imports it lazily)"""
+    from hgcalml_amd import ops
+    return ops
+
+
 def t(a, dtype=None):
     return torch.as_tensor(np.ascontiguousarray(a), dtype=dtype).to(DEV)
 
@@ -841,6 +848,31 @@ def test_refused_arguments():
     assert rc == -1 and b"d_out_maxidxs" in lib.hgc_last_error()
     rc = lib.hgc_accumulate_knn(p(w), p(x), p(i), p(out), None, 10, 4, 8, 99, 0, 0, stream())
     assert rc == -1 and b"n_out_feat" in lib.hgc_last_error()
+
+
+@pytest.mark.parametrize("n,k", [(1, 2), (300, 5), (5000, 17), (20000, 65)])
+def test_inverse_index_without_first_column(n, k):
+    """derived from the whole table's inverse index = built from table[:, 1:] directly, for tables
+    with padding, out-of-range entries and any content in column 0"""
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(n + k)
+    idx = rng.integers(0, n, (n, k)).astype(np.int32)
+    idx[:, 0] = np.where(rng.random(n) < 0.8, np.arange(n), idx[:, 0])   # mostly self, as the kNN writes it
+    idx[rng.random((n, k)) < 0.1] = -1
+    idx[rng.random((n, k)) < 0.01] = n + 5
+    whole = t(idx)
+    part = t(idx[:, 1:])
+    off_w, slots_w = ops.inverse_neighbour_index(whole)
+    off_d, slots_d = ops.inverse_index_without_first_column((off_w, slots_w), n, k)
+    off_p, slots_p = ops.inverse_neighbour_index(part)
+    assert torch.equal(off_d, off_p)
+    used = int(off_p[-1])
+    assert torch.equal(slots_d[:used], slots_p[:used])
+    # through the cache: declared once, derived on demand, also via another object on the same memory
+    ops.declare_without_first_column(part, whole)
+    off_c, slots_c = ops.cached_inverse_neighbour_index(part)
+    assert torch.equal(off_c, off_p) and torch.equal(slots_c[:used], slots_p[:used])
+    assert ops.cached_inverse_neighbour_index(whole.view(n, k))[0] is ops.cached_inverse_neighbour_index(whole)[0]
 
 
 def test_accumulate_knn_weights_and_their_gradient_in_one_pass():
