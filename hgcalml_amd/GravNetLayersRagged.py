@@ -26,6 +26,49 @@ def eye_init_(weight, mean=0.0, stddev=0.1, eye_scaling=1.0):
     return weight
 
 
+class _TallLinearFn(torch.autograd.Function):
+    """y = x W^T + b for x of very many rows. The weight gradient g^T x reduces over those rows
+    into a small matrix; as one GEMM it runs on a handful of workgroups (0.35-0.44 ms for 150k rows
+    of 64-192 columns), as a batch of 64 row slices added up afterwards it takes 0.07-0.11 ms."""
+
+    SLICES = 64
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, weight = ctx.saved_tensors
+        g = g.contiguous()
+        grad_x = g @ weight if ctx.needs_input_grad[0] else None
+        grad_w = None
+        if ctx.needs_input_grad[1]:
+            n, s = x.shape[0], _TallLinearFn.SLICES
+            whole = n // s * s
+            if whole >= 64 * s:
+                grad_w = torch.bmm(g[:whole].view(s, -1, g.shape[1]).transpose(1, 2),
+                                   x[:whole].view(s, -1, x.shape[1])).sum(0)
+                if whole < n:
+                    grad_w = grad_w + g[whole:].t() @ x[whole:]
+            else:
+                grad_w = g.t() @ x
+        grad_b = g.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        return grad_x, grad_w, grad_b
+
+
+class TallLinear(nn.Linear):
+    """nn.Linear whose weight gradient is formed slice-wise (see _TallLinearFn); same parameters and results
+    up to the summation order of that gradient"""
+
+    def forward(self, x):
+        if x.dim() == 2 and x.is_contiguous():
+            return _TallLinearFn.apply(x, self.weight, self.bias)
+        return super().forward(x)
+
+
 _ACTIVATIONS = {None: nn.Identity, "linear": nn.Identity, "relu": nn.ReLU, "elu": nn.ELU, "tanh": nn.Tanh,
                 "sigmoid": nn.Sigmoid, "selu": nn.SELU, "gelu": nn.GELU}
 
@@ -46,11 +89,11 @@ class RaggedGravNet(nn.Module):
         self.return_self = return_self
         self.sumwnorm = sumwnorm
         self.n_knn_bins = n_knn_bins
-        self.input_feature_transform = nn.Linear(in_features, n_propagate)
+        self.input_feature_transform = TallLinear(in_features, n_propagate)
         self.feature_activation = _ACTIVATIONS[feature_activation]()
-        self.input_spatial_transform = nn.Linear(in_features, n_dimensions, bias=False)
+        self.input_spatial_transform = TallLinear(in_features, n_dimensions, bias=False)
         eye_init_(self.input_spatial_transform.weight, 0.0, coord_initialiser_noise)
-        self.output_feature_transform = nn.Linear(2 * n_propagate + in_features, n_filters)
+        self.output_feature_transform = TallLinear(2 * n_propagate + in_features, n_filters)
         # bookkeeping of the reference (GravNetLayersRagged.py:3180-3193); the exact kNN does not use it
         self.register_buffer("dynamic_radius", torch.tensor(1.0))
 
