@@ -507,6 +507,45 @@ def test_accumulate_cfg4_full_size_properties(oracle):
     assert torch.allclose(total, mean_total + max_total, rtol=1e-6, atol=1e-3)
 
 
+def test_accumulate_matrices_beyond_4_gib():
+    """Output and upstream-gradient matrices of more than 2^32 bytes are addressed with
+    64-bit offsets by the thread-per-element kernels; smaller ones take the wave kernels'
+    32-bit buffer offsets. Neighbours stay inside blocks of 3000 rows, so the first block
+    and the last two are closed sub-problems: run alone they take the wave kernels (pinned
+    against the oracle above) and must give the rows of the large run, bit for bit (forward,
+    arg-max, feature gradient) or within the weight gradient's tolerance."""
+    from hgcalml_amd import AccumulateLinKnn, ops
+    n, F, K, blk = 2_200_000, 256, 4, 3000
+    assert n * 2 * F * 4 >= 1 << 32 and n * 2 * F < 1 << 31
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    x = torch.randn(n, F, generator=gen, device=DEV)
+    w = torch.exp(-torch.rand(n, K, generator=gen, device=DEV))
+    row = torch.arange(n, device=DEV)
+    base = (row // blk) * blk
+    size = torch.clamp(n - base, max=blk)                    # 3000, and 1000 for the last block
+    third = size // 3
+    # distinct non-zero steps inside the block: slot 0 is the vertex itself, no repeated neighbour
+    step = torch.stack([torch.zeros_like(size)] +
+                       [1 + i * third + torch.randint(0, 1 << 30, (n,), generator=gen, device=DEV) % (third - 1)
+                        for i in range(K - 1)], 1)
+    idx = (base[:, None] + (row[:, None] - base[:, None] + step) % size[:, None]).to(torch.int32)
+    out, arg = AccumulateLinKnn(w, x, idx)
+    g = torch.randn(n, 2 * F, generator=gen, device=DEV)
+    gw, gx = torch.ops.hgcalml.accumulate_knn_grad(g, w, x, idx, arg, *ops.inverse_neighbour_index(idx))
+    tail = (n // blk - 1) * blk
+    for lo, hi in ((0, blk), (tail, n)):
+        xs, ws, gs = x[lo:hi].contiguous(), w[lo:hi].contiguous(), g[lo:hi].contiguous()
+        ids = (idx[lo:hi] - lo).contiguous()
+        assert int(ids.min()) >= 0 and int(ids.max()) < hi - lo
+        out_s, arg_s = AccumulateLinKnn(ws, xs, ids)
+        assert torch.equal(out[lo:hi].view(torch.int32), out_s.view(torch.int32))
+        assert torch.equal(arg[lo:hi], arg_s + lo)
+        gw_s, gx_s = torch.ops.hgcalml.accumulate_knn_grad(gs, ws, xs, ids, arg_s, *ops.inverse_neighbour_index(ids))
+        assert torch.equal(gx[lo:hi].view(torch.int32), gx_s.view(torch.int32))
+        tol = grad_tolerance(gs.cpu().numpy(), xs.cpu().numpy(), ids.cpu().numpy(), ws.cpu().numpy(), K)
+        assert (np.abs(gw[lo:hi].cpu().numpy() - gw_s.cpu().numpy()) <= 2 * tol).all()
+
+
 # ------------------------------------------------------------------ ops next to the accumulation
 
 @pytest.mark.parametrize("K,C", [(16, 3), (64, 4), (5, 8)])
