@@ -507,6 +507,22 @@ def test_accumulate_cfg4_full_size_properties(oracle):
     assert torch.allclose(total, mean_total + max_total, rtol=1e-6, atol=1e-3)
 
 
+def blocked_neighbour_table(n, K, blk, gen):
+    """weights and a neighbour table on the device whose rows name K distinct vertices of
+    their own block of `blk` rows (slot 0 = the vertex itself): every block is a closed
+    sub-problem of the accumulation, of its gradient and of the push"""
+    w = torch.exp(-torch.rand(n, K, generator=gen, device=DEV))
+    row = torch.arange(n, device=DEV)
+    base = (row // blk) * blk
+    size = torch.clamp(n - base, max=blk)
+    third = size // (K - 1)
+    step = torch.stack([torch.zeros_like(size)] +
+                       [1 + i * third + torch.randint(0, 1 << 30, (n,), generator=gen, device=DEV) % (third - 1)
+                        for i in range(K - 1)], 1)
+    idx = (base[:, None] + (row[:, None] - base[:, None] + step) % size[:, None]).to(torch.int32)
+    return w, idx
+
+
 def test_accumulate_matrices_beyond_4_gib():
     """Output and upstream-gradient matrices of more than 2^32 bytes are addressed with
     64-bit offsets by the thread-per-element kernels; smaller ones take the wave kernels'
@@ -519,16 +535,7 @@ def test_accumulate_matrices_beyond_4_gib():
     assert n * 2 * F * 4 >= 1 << 32 and n * 2 * F < 1 << 31
     gen = torch.Generator(device=DEV).manual_seed(77)
     x = torch.randn(n, F, generator=gen, device=DEV)
-    w = torch.exp(-torch.rand(n, K, generator=gen, device=DEV))
-    row = torch.arange(n, device=DEV)
-    base = (row // blk) * blk
-    size = torch.clamp(n - base, max=blk)                    # 3000, and 1000 for the last block
-    third = size // 3
-    # distinct non-zero steps inside the block: slot 0 is the vertex itself, no repeated neighbour
-    step = torch.stack([torch.zeros_like(size)] +
-                       [1 + i * third + torch.randint(0, 1 << 30, (n,), generator=gen, device=DEV) % (third - 1)
-                        for i in range(K - 1)], 1)
-    idx = (base[:, None] + (row[:, None] - base[:, None] + step) % size[:, None]).to(torch.int32)
+    w, idx = blocked_neighbour_table(n, K, blk, gen)
     out, arg = AccumulateLinKnn(w, x, idx)
     g = torch.randn(n, 2 * F, generator=gen, device=DEV)
     gw, gx = torch.ops.hgcalml.accumulate_knn_grad(g, w, x, idx, arg, *ops.inverse_neighbour_index(idx))
