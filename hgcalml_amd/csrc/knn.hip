@@ -582,6 +582,9 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
     HGC_REQUIRE(n_vert >= 0, "negative number of points");
     HGC_REQUIRE(n_neigh >= 1 && n_neigh <= 8 * kWave + 1, "1 <= n_neighbours <= %d", 8 * kWave + 1);
     HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neighbours overflows int32");
+    // candidate rows are addressed by 32-bit byte offsets
+    HGC_REQUIRE((unsigned long long)n_vert * (unsigned long long)n_coords * sizeof(float) < (1ull << 32),
+                "coordinate matrix must stay below 4 GiB");
     HGC_REQUIRE(n_bboundaries >= 2, "bin boundary table too short");
     HGC_REQUIRE(boundary_shift >= 0 && boundary_shift < 8, "bad boundary stride");
     if (n_vert == 0) return HGC_OK;

@@ -129,7 +129,8 @@ int hgc_gather_rows(const void *d_in, const int *d_rows, void *d_out, int n_rows
  * (or (self, 0.0) if tf_compat) at the tail. The reference leaves the slots in
  * fill/replacement order; the neighbour SET is the same except where the K-th
  * and (K+1)-th distances are exactly equal, where the lower index is kept.
- * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, 1 <= n_neigh <= 513. */
+ * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, 1 <= n_neigh <= 513,
+ * n_vert * n_neigh < 2^31, coordinate matrix below 4 GiB. */
 int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int *d_direction,
                           const int *d_dim_bin_idx, const int *d_bin_boundaries,
                           const int *d_n_bins, const float *d_bin_width,

@@ -66,6 +66,7 @@ def test_host_side_argument_checks(capi):
     assert f(*args_tail, 10, 4, 1, 2, 5, 0, 0, null) == -1
     assert f(*args_tail, 10, 4, 3, 3, 5, 0, 0, null) == -1 and b"null pointer" in capi.hgc_last_error()
     assert f(*args_tail, 0, 4, 3, 3, 5, 0, 0, null) == 0  # empty input is fine
+    assert f(*args_tail, 150_000_000, 1, 8, 3, 5, 0, 0, null) == -1 and b"4 GiB" in capi.hgc_last_error()
     # accumulate: output width must match mean_and_max
     g = capi.hgc_accumulate_knn
     g.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 6 + [ctypes.c_void_p]
