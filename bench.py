@@ -20,8 +20,7 @@ K iterations, HIP events on the stream the kernels are launched on) at cfg4
 (N=1,000,000, K=64, F=128, banded neighbour table): the dominant kernel, one
 launch of the accumulate_knn gradient (algorithmic bytes 4*N*(3K+5F)), with
 the forward launch (4*N*(2K+4F)) and the forward+gradient pair next to it,
-against the 8 TB/s HBM peak; plus the bare K-fold row gather of the same
-table, the rate the memory system delivers those rows at.
+against the 8 TB/s HBM peak.
 
 `cpu_baseline` times the CPU oracle (a single-threaded C restatement of the
 reference CPU kernels) on this box's host: the binned kNN kernel over the full
@@ -39,6 +38,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+sys.path.insert(1, os.path.join(ROOT, "tests"))  # workloads.py: the seeded inputs shared with the tests
 
 HBM_PEAK_GBS = 8000.0
 
@@ -128,7 +128,8 @@ def main():
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
-    from hgcalml_amd import AccumulateKnn, AccumulateLinKnn, BinnedSelectKnn, BuildAndAssignCondensatesBinned, ops, workloads
+    from hgcalml_amd import AccumulateKnn, AccumulateLinKnn, BinnedSelectKnn, BuildAndAssignCondensatesBinned, ops
+    import workloads
     dev = "cuda:0"
     torch.cuda.set_device(0)
 
@@ -222,14 +223,11 @@ def main():
     inv = ops.inverse_neighbour_index(i4)
     grad_ms = event_ms(lambda: torch.ops.hgcalml.accumulate_knn_grad_slots(g4, w4, x4, i4, arg4, slots4, *inv),
                        args.steps, args.warmup)
-    # the bare K-fold row gather of the same neighbour table: what the memory system delivers
-    probe_ms = event_ms(lambda: ops.probe_row_gather(x4, i4), args.steps, 2)
-    gathered_bytes = 4.0 * n4 * K4 * F4
     bytes_fwd = 4.0 * n4 * (2 * K4 + 4 * F4)
     bytes_bwd = 4.0 * n4 * (3 * K4 + 5 * F4)
     achieved = (bytes_fwd + bytes_bwd) / ((fwd_ms[0] + grad_ms[0]) * 1e-3) / 1e9
-    log("bench: cfg4 fwd %.3f ms, grad %.3f ms, inverse index (one-off) %.3f ms -> %.1f GB/s; bare row gather %.3f ms" %
-        (fwd_ms[0], grad_ms[0], inv_ms[0], achieved, probe_ms[0]))
+    log("bench: cfg4 fwd %.3f ms, grad %.3f ms, inverse index (one-off) %.3f ms -> %.1f GB/s" %
+        (fwd_ms[0], grad_ms[0], inv_ms[0], achieved))
 
     if args.section == "roofline":
         return
@@ -335,11 +333,7 @@ def main():
                                                "algorithmic_bytes": bytes_fwd + bytes_bwd,
                                                "traffic": (CFG4_FWD_MEASURED_HBM_BYTES + CFG4_GRAD_MEASURED_HBM_BYTES)
                                                if args.roofline_scale == 1.0 else None},
-                     "inverse_index_build_ms": round(inv_ms[0], 3),
-                     "row_gather_probe": {"ms": round(probe_ms[0], 4),
-                                          "gathered_TBps": round(gathered_bytes / (probe_ms[0] * 1e-3) / 1e12, 2),
-                                          "forward_over_probe": round(fwd_ms[0] / probe_ms[0], 3),
-                                          "note": "K rows of 4F bytes per vertex through L2, no arithmetic"}},
+                     "inverse_index_build_ms": round(inv_ms[0], 3)},
         "cpu_baseline": cpu,
         "extra": extra,
     }

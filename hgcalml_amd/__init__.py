@@ -12,8 +12,7 @@ __all__ = ["BinByCoordinates", "BinnedSelectKnn", "IndexReplacer", "AccumulateKn
 
 
 def __getattr__(name):
-    # lazy: importing the package alone (e.g. for hgcalml_amd.workloads or the
-    # build script) must not require the compiled library
+    # lazy: importing the package alone (e.g. for the build script) must not require the compiled library
     if name in __all__:
         import importlib
         mod = {

@@ -45,7 +45,6 @@ _SIGNATURES = {
     "hgc_local_distance": (_c_int, [_ptr] * 3 + [_c_int] * 4 + [_ptr]),
     "hgc_push_knn": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),
     "hgc_push_knn_grad": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),
-    "hgc_probe_row_gather": (_c_int, [_ptr] * 3 + [_c_int] * 3 + [_ptr]),
     "hgc_exp_neg": (_c_int, [_ptr, _ptr, ctypes.c_longlong, _ptr]),
     "hgc_exp_neg_grad": (_c_int, [_ptr, _ptr, _ptr, ctypes.c_longlong, _ptr]),
     "hgc_binned_assign_to_condensates_workspace_bytes": (_c_size, [_c_int, _c_int, _c_int]),

@@ -413,15 +413,6 @@ def push_knn_grad(grad: torch.Tensor, weights: torch.Tensor, features: torch.Ten
     return wgrad, fgrad
 
 
-def probe_row_gather(features, indices):
-    """measurement aid: sum of the K gathered rows per vertex, nothing else"""
-    require_device(features, indices)
-    x, idx = f32(features), i32(indices)
-    out = torch.empty_like(x)
-    check(lib.hgc_probe_row_gather(p(x), p(idx), p(out), idx.shape[0], idx.shape[1], x.shape[1], stream()))
-    return out
-
-
 # --------------------------------------------------------------------------- condensates
 
 @torch.library.custom_op("hgcalml::binned_assign_to_condensates", mutates_args=())

@@ -333,14 +333,6 @@ int hgc_exp_neg(const float *d_distances, float *d_weights, long long n_values, 
 int hgc_exp_neg_grad(const float *d_weight_grad, const float *d_weights, float *d_distance_grad,
                      long long n_values, hgc_stream_t stream);
 
-/* Measurement aid without a counterpart in the reference: out[v,:] = sum over
- * the K rows d_feat[d_idxs[v,n],:] with the forward kernel's access pattern and
- * no other arithmetic. Its run time is the rate at which the memory system
- * delivers the K-fold re-read rows; bench.py reports the accumulation kernels
- * against it. n_feat must be a multiple of 64. */
-int hgc_probe_row_gather(const float *d_feat, const int *d_idxs, float *d_out,
-                         int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
-
 /* ------------------------------------------------------------------ */
 /* Condensate assignment                                               */
 /* ------------------------------------------------------------------ */

@@ -17,6 +17,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, ROOT)
+sys.path.insert(1, os.path.dirname(HERE))  # tests/workloads.py
 
 import oracle  # noqa: E402
 
@@ -35,7 +36,7 @@ def g1_binning():
 
 
 def g2_knn():
-    from hgcalml_amd import workloads
+    import workloads
     cfg = workloads.cfg2(scale=512 / 150000, seed=102)
     coords = cfg["coords"][:512].copy()
     rs = np.array([0, 200, 512], np.int32)
@@ -82,7 +83,7 @@ def g3_accumulate():
 
 
 def g5_condensates():
-    from hgcalml_amd import workloads
+    import workloads
     cfg = workloads.cfg5(scale=1000 / 62500, seed=105, n_events=2)
     out = dict(ccoords=cfg["ccoords"], betas=cfg["betas"], dist=cfg["dist"], row_splits=cfg["row_splits"])
     for mode in (True, False):

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from hgcalml_amd import workloads
+import workloads
 from helpers import check_knn_rows
 
 pytestmark = pytest.mark.gpu
@@ -683,19 +683,6 @@ def test_gravnet_block_forward_and_all_gradients(n_propagate, n_neighbours, sumw
     assert close(x.grad, x64.grad)
     for k, v in layer.named_parameters():
         assert close(v.grad, p64[k].grad), k
-
-
-def test_row_gather_probe():
-    from hgcalml_amd import ops
-    rng = np.random.default_rng(80)
-    n, K, F = 1000, 20, 128
-    x = rng.standard_normal((n, F)).astype(np.float32)
-    idx = rng.integers(0, n, size=(n, K)).astype(np.int32)
-    got = ops.probe_row_gather(t(x), t(idx)).cpu().numpy()
-    want = np.zeros((n, F), np.float32)
-    for k in range(K):
-        want = (want + x[idx[:, k]]).astype(np.float32)
-    assert (bits(got) == bits(want)).all()
 
 
 def test_local_distance_and_gradient(oracle):

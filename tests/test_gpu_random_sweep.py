@@ -23,7 +23,8 @@ def bits(a):
 @pytest.mark.parametrize("seed", range(24))
 def test_random_configuration(oracle, seed):
     from hgcalml_amd import (AccumulateLinKnn, BinnedSelectKnn, BuildAndAssignCondensatesBinned, LocalDistance,
-                             PushKnn, ops, workloads)
+                             PushKnn, ops)
+    import workloads
     rng = np.random.default_rng(1000 + seed)
     n = int(rng.integers(50, 5000))
     C = int(rng.integers(2, 7))

@@ -8,7 +8,7 @@ cases chosen so that a wrong sign, index, tie rule or summation order fails.
 import numpy as np
 import pytest
 
-from hgcalml_amd import workloads
+import workloads
 
 
 from helpers import brute_knn_row, check_knn_rows, serial_distsq  # noqa: E402,F401
