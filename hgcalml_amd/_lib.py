@@ -32,6 +32,7 @@ _SIGNATURES = {
     "hgc_binned_select_knn_fused": (_c_int, [_ptr] * 9 + [_c_float] + [_ptr] * 2 + [_c_int] * 7 + [_ptr]),
     "hgc_binned_select_knn_pipeline_workspace_bytes": (_c_size, [_c_int] * 6),
     "hgc_binned_select_knn_pipeline": (_c_int, [_ptr] * 3 + [_c_int] * 7 + [_c_float, _ptr, _ptr, _ptr, _ptr, _c_size, _ptr]),
+    "hgc_binned_select_knn_pipeline_static": (_c_int, [_ptr] * 3 + [_c_int] * 7 + [_c_float, _ptr, _ptr, _ptr, _ptr]),
     "hgc_index_replacer": (_c_int, [_ptr, _ptr, _ptr, _c_int, _c_int, _ptr]),
     "hgc_accumulate_knn": (_c_int, [_ptr] * 5 + [_c_int] * 6 + [_ptr]),
     "hgc_accumulate_knn_slots": (_c_int, [_ptr] * 7 + [_c_int] * 6 + [_ptr]),

@@ -11,6 +11,7 @@
 #include "hgc_common.hpp"
 
 #include <algorithm>
+#include <mutex>
 
 namespace hgc {
 int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
@@ -18,7 +19,34 @@ int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
 
 using namespace hgc;
 
+// Scratch memory of hgc_binned_select_knn_pipeline_static, part of the library's
+// device image: every GPU the library runs on holds its own copy at its own
+// address from the first use to the end of the process. In host code this name
+// is only a handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) unsigned char scratch[HGC_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` per device, looked up once
+
+// the current device's copy of `scratch` (nullptr + error text on failure)
+int static_scratch(void **out) {
+    int dev = -1;
+    HGC_HIP(hipGetDevice(&dev));
+    HGC_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d beyond the %d this library keeps scratch for", dev,
+                kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        HGC_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr || !aligned256(ptr)) return fail(HGC_ERR_LAUNCH, "static scratch array has no usable device address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return HGC_OK;
+}
 
 struct KnnPipelineLayout {
     size_t shift, bin_width, n_bins, sorting, bounds, scoords, sflat, sbinass, sdir, grouping_ws, total;
@@ -329,6 +357,24 @@ size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, 
     const int n_bin_dims = std::min(max_bin_dims, n_coords);
     if (n_vert < 0 || n_coords < 1 || n_rs < 2 || n_bins_scalar < 1 || n_bin_dims < 1 || n_bin_dims > 5) return 0;
     return knn_layout(n_vert, n_coords, n_bin_dims, n_rs, n_bins_scalar, use_direction).total;
+}
+
+int hgc_binned_select_knn_pipeline_static(const float *d_coords, const int *d_row_splits, const int *d_direction,
+                                          int n_vert, int n_coords, int n_rs, int n_neigh, int n_bins_scalar,
+                                          int max_bin_dims, int tf_compat, float max_radius, int *d_indices,
+                                          float *d_dist, int *d_out_sorting, hgc_stream_t stream) {
+    const size_t need = hgc_binned_select_knn_pipeline_workspace_bytes(n_vert, n_coords, n_rs, n_bins_scalar,
+                                                                       max_bin_dims, d_direction != nullptr);
+    if (need > (size_t)HGC_STATIC_SCRATCH_BYTES)
+        return fail(HGC_ERR_WORKSPACE,
+                    "this call needs %zu bytes of scratch, the built-in array holds %zu: use "
+                    "hgc_binned_select_knn_pipeline with a workspace of your own", need,
+                    (size_t)HGC_STATIC_SCRATCH_BYTES);
+    void *ptr = nullptr;
+    if (int rc = static_scratch(&ptr)) return rc;
+    return hgc_binned_select_knn_pipeline(d_coords, d_row_splits, d_direction, n_vert, n_coords, n_rs, n_neigh,
+                                          n_bins_scalar, max_bin_dims, tf_compat, max_radius, d_indices, d_dist,
+                                          d_out_sorting, ptr, HGC_STATIC_SCRATCH_BYTES, stream);
 }
 
 int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_splits, const int *d_direction,

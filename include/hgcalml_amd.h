@@ -178,6 +178,25 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
                                    float max_radius, int *d_indices, float *d_dist, int *d_out_sorting,
                                    void *workspace, size_t workspace_bytes, hgc_stream_t stream);
 
+/* hgc_binned_select_knn_pipeline for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): same arguments without the workspace, same results. It has no
+ * counterpart in the reference. The scratch memory is an array of
+ * HGC_STATIC_SCRATCH_BYTES inside the library's device image; every GPU the
+ * library is used on holds it from the first call to the end of the process.
+ * The call allocates and frees nothing. A problem whose
+ * hgc_binned_select_knn_pipeline_workspace_bytes(...) exceeds
+ * HGC_STATIC_SCRATCH_BYTES is refused with HGC_ERR_WORKSPACE (N = 150,000 points
+ * with 4 coordinates, one event and n_bins = 30 need 19.3 MiB). All calls on
+ * one GPU share that GPU's array: calls that overlap on one GPU (different
+ * streams or threads) race and must be ordered by the caller. */
+#define HGC_STATIC_SCRATCH_BYTES (32u << 20)
+int hgc_binned_select_knn_pipeline_static(const float *d_coords, const int *d_row_splits,
+                                          const int *d_direction, int n_vert, int n_coords, int n_rs,
+                                          int n_neigh, int n_bins_scalar, int max_bin_dims, int tf_compat,
+                                          float max_radius, int *d_indices, float *d_dist,
+                                          int *d_out_sorting, hgc_stream_t stream);
+
 /* out[i] = v < 0 ? v : replacements[v]; entries with v >= n_replacements are
  * left untouched. Replaces IndexReplacerOpFunctor
  * (modules/compiled/index_replacer_kernel.h, _kernel.cc:17-42). */
