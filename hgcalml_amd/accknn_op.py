@@ -86,7 +86,10 @@ def _sumw(acc, x, features, indices, mean_and_max):
     f, midx = acc(x, features, indices, mean_and_max=mean_and_max)
     fmean = f[:, :origshape]
     fnorm = f[:, origshape:origshape + 1]
-    fmean = torch.where(fnorm == 0, torch.zeros_like(fmean), fmean / fnorm)
+    # tf.math.divide_no_nan: 0 where the accumulated weight is 0, and a zero gradient there too
+    # (dividing by the raw denominator would send 0/0 = NaN into the backward pass)
+    empty = fnorm == 0
+    fmean = torch.where(empty, torch.zeros_like(fmean), fmean / torch.where(empty, torch.ones_like(fnorm), fnorm))
     if mean_and_max:
         fmean = torch.cat([fmean, f[:, origshape + 1:-1]], dim=1)
     return fmean, midx

@@ -173,13 +173,16 @@ def set_vertex_order(indices, order):
     """Remembers a processing order (a permutation of the vertices with spatial
     locality) for the neighbour table `indices`; the accumulation ops look it up
     by tensor object. Results never depend on it, only how well the gathered
-    rows are found in cache."""
-    if len(_VERTEX_ORDER) > 64:
-        for k in [k for k, v in _VERTEX_ORDER.items() if v[0]() is None]:
-            del _VERTEX_ORDER[k]
-        if len(_VERTEX_ORDER) > 64:
-            _VERTEX_ORDER.clear()
-    _VERTEX_ORDER[id(indices)] = (weakref.ref(indices), order)
+    rows are found in cache. The entry goes away with the table."""
+    key = id(indices)
+    _VERTEX_ORDER[key] = (weakref.ref(indices), order)
+    weakref.finalize(indices, _drop_if_dead, _VERTEX_ORDER, key)
+
+
+def _drop_if_dead(cache, key):
+    hit = cache.get(key)
+    if hit is not None and hit[0]() is None:
+        del cache[key]
 
 
 def vertex_order_of(indices):
@@ -276,7 +279,12 @@ def declare_without_first_column(part, whole):
 def cached_inverse_neighbour_index(indices):
     """The inverse index depends only on the neighbour table; GravNet-style
     models run several accumulations (and their gradients) over one table, so
-    it is built once per tensor object and version."""
+    it is built once per tensor object and version and dropped when the table
+    dies. Validity is judged by the tensor's version counter and data pointer:
+    a table that is refilled IN PLACE behind torch's back (a kernel of this
+    library or a HIP graph replay writing through its raw pointer, `out=`
+    reuse in foreign code) must be announced with `invalidate_neighbour_table`
+    before the next gradient, push or distance-gradient call on it."""
     key = id(indices)
     hit = _INVERSE_CACHE.get(key)
     if hit is not None:
@@ -298,13 +306,24 @@ def cached_inverse_neighbour_index(indices):
                                                        whole.shape[1])
     if value is None:
         value = inverse_neighbour_index(indices)
-    if len(_INVERSE_CACHE) > 64:
-        for k in [k for k, v in _INVERSE_CACHE.items() if v[0]() is None]:
-            del _INVERSE_CACHE[k]
-        if len(_INVERSE_CACHE) > 64:
-            _INVERSE_CACHE.clear()
     _INVERSE_CACHE[key] = (weakref.ref(indices), indices._version, indices.data_ptr(), value)
+    weakref.finalize(indices, _drop_if_dead, _INVERSE_CACHE, key)
     return value
+
+
+def invalidate_neighbour_table(indices):
+    """Forgets what is cached for the neighbour table `indices` (inverse index, processing
+    order), also under other tensor objects on the same memory. Needed only after the table
+    was rewritten in place without torch noticing (see cached_inverse_neighbour_index)."""
+    ptr = indices.data_ptr()
+    for cache in (_INVERSE_CACHE, _VERTEX_ORDER):
+        cache.pop(id(indices), None)
+    for key in [k for k, v in _INVERSE_CACHE.items() if v[2] == ptr]:
+        del _INVERSE_CACHE[key]
+    for key in [k for k, v in _VERTEX_ORDER.items() if v[0]() is not None and v[0]().data_ptr() == ptr]:
+        del _VERTEX_ORDER[key]
+    if hasattr(indices, "_hgc_without_first_column_of"):
+        del indices._hgc_without_first_column_of
 
 
 def _accumulate_backward(grad_from_out_features, distances, features, neigh_indices, max_feat_indices, max_slots,

@@ -399,6 +399,40 @@ def AccumulateKnnGrad(grad_out, distances, features, indices, maxidx, linear=Fal
     return (-(w * gw)).astype(np.float32), gx
 
 
+def merge_noise_as_indiv_cp(assignment, asso_idx, alpha_idx, is_cond, n_condensates, row_splits):
+    """modules/assign_condensate_op.py:9-44 (the keep_noise post-pass) on flat arrays.
+    The reference numbers the noise hits of an event with a cumulative sum over ALL
+    hits minus the previous event's running maximum (`cumsum_ragged`, :9-13), gives
+    noise hit number j the shower index j-1, lifts the event's real showers by the
+    event's noise count, lists `noise indices ++ condensation points` per event and
+    recounts the condensation points per event from the merged flags. Events
+    without hits are outside what it defines (reduce_max of an empty row)."""
+    a = np.asarray(assignment, np.int32).reshape(-1)
+    asso_idx = np.asarray(asso_idx, np.int32)
+    alpha_idx = np.asarray(alpha_idx, np.int32)
+    cond = np.asarray(is_cond, bool).reshape(-1)
+    ncond = np.asarray(n_condensates, np.int32)
+    rs = np.asarray(row_splits, np.int64)
+    n = len(a)
+    noise = a < 0
+    running = np.cumsum(noise.astype(np.int32))                     # tf.cumsum over the flat values
+    at_event_end = np.array([running[rs[e + 1] - 1] for e in range(len(rs) - 1)], np.int32)
+    carried = np.concatenate([np.zeros(1, np.int32), at_event_end[:-1]])
+    x = running - np.repeat(carried, np.diff(rs))
+    x = np.where(noise, x, 0)
+    n_noise = np.array([x[rs[e]:rs[e + 1]].max() for e in range(len(rs) - 1)], np.int32)
+    new_assignment = np.where(noise, x - 1, a + np.repeat(n_noise, np.diff(rs))).astype(np.int32)
+    allrange = np.arange(n, dtype=np.int32)
+    merged = [np.concatenate([allrange[rs[e]:rs[e + 1]][noise[rs[e]:rs[e + 1]]], alpha_idx[ncond[e]:ncond[e + 1]]])
+              for e in range(len(rs) - 1)]
+    new_alpha = np.concatenate(merged).astype(np.int32) if merged else np.zeros(0, np.int32)
+    new_cond = np.where(asso_idx < 0, True, cond)
+    new_asso = np.where(asso_idx < 0, allrange, asso_idx).astype(np.int32)
+    per_event = np.array([new_cond[rs[e]:rs[e + 1]].sum() for e in range(len(rs) - 1)], np.int32)
+    new_ncond = np.concatenate([ncond[0:1], np.cumsum(per_event, dtype=np.int32)]).astype(np.int32)
+    return new_assignment[:, None], new_asso, new_alpha, new_cond[:, None], new_ncond
+
+
 def BuildAndAssignCondensatesBinned(ccoords, betas, dist, row_splits, beta_threshold,
                                     no_condensation_mask=None, distance_threshold=1.,
                                     assign_by_max_beta=False, nbin_dims=3, keep_noise=False,
@@ -406,8 +440,6 @@ def BuildAndAssignCondensatesBinned(ccoords, betas, dist, row_splits, beta_thres
     assert 1 <= nbin_dims <= 6
     assert 0. <= beta_threshold <= 1.
     assert distance_threshold > 0.
-    if keep_noise:
-        raise NotImplementedError("keep_noise post-pass is outside the oracle")
     ccoords = np.asarray(ccoords, np.float32)
     betas = np.asarray(betas, np.float32).reshape(-1)
     row_splits = np.asarray(row_splits, np.int32)
@@ -452,6 +484,8 @@ def BuildAndAssignCondensatesBinned(ccoords, betas, dist, row_splits, beta_thres
     is_cond = np.zeros(n, bool)
     is_cond[alpha_idx] = True
     out = (assignment[:, None], asso, alpha_idx, is_cond[:, None], ncond)
+    if keep_noise:
+        out = merge_noise_as_indiv_cp(*out, row_splits)
     if return_kernel_inputs:
         return out, kernel_inputs
     return out

@@ -507,6 +507,74 @@ def test_accumulate_cfg4_full_size_properties(oracle):
     assert torch.allclose(total, mean_total + max_total, rtol=1e-6, atol=1e-3)
 
 
+def test_accumulate_cfg4_full_size_slot_kernels_vs_oracle(oracle, capsys):
+    """N=1M through the kernels bench.py times (forward with the arg-max slot table, one-pass
+    gradient fed with it) against the oracle on closed sub-problems: the table's neighbours lie
+    within a band of rows, so rows [r0, r1) with the features of [r0-band, r1+band) reproduce the
+    forward and the weight gradient of those rows, and the feature gradient of the targets
+    [r0+band, r1-band) (every row naming them is inside, in the same order). Windows at both ends
+    and in the middle. Feature gradient bitwise, weight gradient within 1e-5 of sum |terms|; the
+    worst weight-gradient error relative to the VALUE is printed."""
+    from hgcalml_amd import ops
+    c = workloads.cfg4()
+    n, K, F = len(c["indices"]), c["K"], c["F"]
+    band = int(np.abs(c["indices"] - np.arange(n)[:, None]).max())   # 2000, and up to twice that where the ends reflect
+    assert band <= 4000
+    w = np.exp(-c["distsq"]).astype(np.float32)
+    tw, tx, ti, tg = t(w), t(c["features"]), t(c["indices"]), t(c["grad_out"])
+    out, arg, slots = torch.ops.hgcalml.accumulate_knn_slots(tw, tx, ti, 0, True)
+    inv = ops.inverse_neighbour_index(ti)
+    gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(tg, tw, tx, ti, arg, slots, *inv)
+    assert int(c["indices"].min()) >= 0
+    worst_rel, worst_scaled = 0.0, 0.0
+    for r0, r1 in ((0, 10000), (n // 2 - 6000, n // 2 + 6000), (n - 10000, n)):
+        f0, f1 = max(0, r0 - band), min(n, r1 + band)
+        m = f1 - f0
+        idx = np.full((m, K), -1, np.int32)
+        idx[r0 - f0:r1 - f0] = c["indices"][r0:r1] - f0
+        ws = np.zeros((m, K), np.float32)
+        ws[r0 - f0:r1 - f0] = w[r0:r1]
+        g = np.zeros((m, 2 * F), np.float32)
+        g[r0 - f0:r1 - f0] = c["grad_out"][r0:r1]
+        ref, rarg = oracle.accumulate_knn_kernel(ws, c["features"][f0:f1], idx)
+        got = out[r0:r1].cpu().numpy()
+        assert (bits(got) == bits(ref[r0 - f0:r1 - f0])).all()
+        assert (arg[r0:r1].cpu().numpy() == rarg[r0 - f0:r1 - f0] + f0).all()
+        rgw, rgx = oracle.accumulate_knn_grad_kernel(g, ws, c["features"][f0:f1], idx, rarg)
+        t0 = r0 if r0 == 0 else r0 + band          # targets whose whole inverse list lies inside
+        t1 = r1 if r1 == n else r1 - band
+        assert (bits(gx[t0:t1].cpu().numpy()) == bits(rgx[t0 - f0:t1 - f0])).all()
+        got_w, want_w = gw[r0:r1].cpu().numpy(), rgw[r0 - f0:r1 - f0]
+        tol = grad_tolerance(c["grad_out"][r0:r1], c["features"], c["indices"][r0:r1], w[r0:r1], K)
+        err = np.abs(got_w - want_w)
+        assert (err <= tol).all()
+        worst_scaled = max(worst_scaled, float((err / tol).max()) * 1e-5)
+        big = np.abs(want_w) > 1e-3
+        worst_rel = max(worst_rel, float((err[big] / np.abs(want_w[big])).max()))
+    with capsys.disabled():
+        print("\ncfg4 N=1M weight gradient, 32000 rows x 64 slots: worst |error| / sum|terms| = %.2e, "
+              "worst |error| / |value| (|value| > 1e-3) = %.2e" % (worst_scaled, worst_rel))
+    assert worst_rel < 1e-3
+
+
+def test_cfg2_full_size_accumulate_in_bin_order_vs_oracle(oracle):
+    """the accumulate leg of the headline step at N=150k: neighbour table and processing order from
+    the kNN, weights exp(-10 d^2), F=64, against the oracle over all rows, bit for bit"""
+    from hgcalml_amd import AccumulateKnn, AccumulateLinKnn, BinnedSelectKnn, ops
+    c = workloads.cfg2()
+    idx, dist = BinnedSelectKnn(c["K"], t(c["coords"]), t(c["row_splits"]), n_bins=c["n_bins"])
+    order = ops.vertex_order_of(idx)
+    assert order is not None and sorted(order.cpu().tolist()) == list(range(len(c["coords"])))
+    w = torch.exp(-(10. * dist))
+    out, arg = AccumulateLinKnn(w, t(c["features"]), idx)
+    ref, rarg = oracle.accumulate_knn_kernel(w.cpu().numpy(), c["features"], idx.cpu().numpy())
+    assert (bits(out.cpu().numpy()) == bits(ref)).all()
+    assert (arg.cpu().numpy() == rarg).all()
+    # the wrapper that computes the weights itself (one-pass exp kernel): same bits as torch.exp
+    out2, arg2 = AccumulateKnn(10. * dist, t(c["features"]), idx)
+    assert torch.equal(out2, out) and torch.equal(arg2, arg)
+
+
 def blocked_neighbour_table(n, K, blk, gen):
     """weights and a neighbour table on the device whose rows name K distinct vertices of
     their own block of `blk` rows (slot 0 = the vertex itself): every block is a closed
@@ -630,6 +698,74 @@ def test_accumulate_sumw_wrappers(oracle, linear):
             assert (bits(out.cpu().numpy()) == bits(ref)).all()
         else:
             assert np.allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("linear", [True, False])
+def test_accumulate_sumw_gradients_stay_finite_without_weight(linear):
+    """a vertex without neighbours (row of -1) and one whose weights are all 0 (exp(-d) underflows from
+    d ~ 104 on) have accumulated weight 0: output 0 and, like tf.math.divide_no_nan, gradient 0 there
+    instead of 0/0; every other row keeps its float64 gradients"""
+    from hgcalml_amd import AccumulateKnnSumw, AccumulateLinKnnSumw
+    rng = np.random.default_rng(71)
+    n, K, F = 200, 8, 16
+    d, x, idx = make_acc_case(rng, n, K, F, holes=False)
+    idx[5] = -1
+    d[9] = 500.0
+    assert float(np.exp(np.float32(-500.0))) == 0.0
+    w = np.exp(-d).astype(np.float32) if linear else d
+    tw, tx = t(w).requires_grad_(True), t(x).requires_grad_(True)
+    fn = AccumulateLinKnnSumw if linear else AccumulateKnnSumw
+    out, _ = fn(tw, tx, t(idx), mean_and_max=False)
+    g = t(rng.standard_normal(out.shape).astype(np.float32))
+    (out * g).sum().backward()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(tw.grad).all()) and bool(torch.isfinite(tx.grad).all())
+    assert (out[5] == 0).all() and (out[9] == 0).all()
+    assert (tw.grad[5] == 0).all() and (tw.grad[9] == 0).all()
+    # float64 closed form sum(w x) / sum(w) over the rows that have weight
+    keep = np.ones(n, bool)
+    keep[[5, 9]] = False
+    w64 = torch.tensor(w[keep], dtype=torch.float64, requires_grad=True)
+    x64 = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    ti = torch.tensor(idx[keep], dtype=torch.int64)
+    ww = w64 if linear else torch.exp(-w64)
+    comp = (x64[ti] * ww[:, :, None]).sum(1) / ww.sum(1, keepdim=True)
+    (comp * g.cpu().double()[torch.tensor(keep)]).sum().backward()
+    assert np.allclose(out.detach().cpu().numpy()[keep], comp.detach().numpy(), rtol=1e-4, atol=1e-5)
+    assert np.allclose(tw.grad.cpu().numpy()[keep], w64.grad.numpy(), rtol=1e-3, atol=1e-5)
+    assert np.allclose(tx.grad.cpu().numpy(), x64.grad.numpy(), rtol=1e-3, atol=1e-5)
+
+
+def test_inverse_index_cache_follows_the_table():
+    """the cached inverse index dies with its table, follows torch-visible in-place writes by itself,
+    and a table rewritten through its raw pointer is announced with invalidate_neighbour_table"""
+    import gc
+    from hgcalml_amd import ops
+    from hgcalml_amd._lib import check, lib, p, stream
+    rng = np.random.default_rng(72)
+    n, K, F = 400, 6, 8
+    _, x, idx_a = make_acc_case(rng, n, K, F)
+    _, _, idx_b = make_acc_case(rng, n, K, F)
+    w = rng.random((n, K)).astype(np.float32)
+
+    def push(table):
+        return torch.ops.hgcalml.push_knn(t(w), t(x), table)
+    want_a, want_b = push(t(idx_a)), push(t(idx_b))
+    assert not torch.equal(want_a, want_b)
+    before = len(ops._INVERSE_CACHE)
+    table = t(idx_a)
+    assert torch.equal(push(table), want_a)
+    assert len(ops._INVERSE_CACHE) == before + 1
+    table.copy_(t(idx_b))                                  # torch sees this write: version counter
+    assert torch.equal(push(table), want_b)
+    # a write torch does not see: the library's own gather kernel fills the buffer through its pointer
+    src, rows = t(idx_a), torch.arange(n, dtype=torch.int32, device=DEV)
+    check(lib.hgc_gather_rows(p(src), p(rows), p(table), n, K, stream()))
+    assert torch.equal(table, src)
+    ops.invalidate_neighbour_table(table)
+    assert torch.equal(push(table), want_a)
+    del table, src
+    gc.collect()
+    assert len(ops._INVERSE_CACHE) <= before
 
 
 @pytest.mark.parametrize("n_propagate,n_neighbours,sumwnorm", [(64, 16, False), (8, 15, False), (64, 16, True)])
@@ -1044,6 +1180,49 @@ def test_condensates_with_no_condensation_mask(oracle, by_max_beta):
     rng = np.random.default_rng(26)
     mask = (rng.random(len(cfg["betas"])) < 0.01).astype(np.int32)[:, None]
     run_condensates(oracle, cfg, by_max_beta, mask=mask)
+
+
+def test_condensates_hand_computed_cases():
+    """literal expectations worked out from the reference text (tests/condensate_cases.py), no oracle
+    involved: min-distance claim rule, per-hit radii, mask indexing of the pick loop"""
+    from condensate_cases import CASES
+    from hgcalml_amd import BuildAndAssignCondensatesBinned
+    for case in CASES:
+        a, s, alpha, is_cond, ncond = BuildAndAssignCondensatesBinned(
+            t(case["ccoords"]), t(case["betas"]), t(case["dist"]), t(case["row_splits"]), case["beta_threshold"],
+            no_condensation_mask=t(case["mask"]), assign_by_max_beta=case["assign_by_max_beta"])
+        assert a[:, 0].cpu().tolist() == case["assignment"].tolist(), case["name"]
+        assert s.cpu().tolist() == case["asso"].tolist(), case["name"]
+        assert alpha.cpu().tolist() == case["alpha"].tolist(), case["name"]
+        assert ncond.cpu().tolist() == case["ncond"].tolist(), case["name"]
+        want_cond = np.zeros(len(case["asso"]), bool)
+        want_cond[case["alpha"]] = True
+        assert is_cond[:, 0].cpu().tolist() == want_cond.tolist(), case["name"]
+
+
+@pytest.mark.parametrize("by_max_beta", [True, False])
+def test_condensates_keep_noise_matches_oracle(oracle, by_max_beta):
+    """keep_noise=True: all five outputs against the oracle's restatement of the post-pass (numbering of
+    the noise hits, order of the merged condensation point list, flags, recount); uneven events, one
+    without noise (radius covers everything around its points), one of noise only (betas below threshold)"""
+    from hgcalml_amd import BuildAndAssignCondensatesBinned
+    cfg = workloads.cfg5(scale=0.03, n_events=3)
+    n = len(cfg["betas"])
+    rs = np.array([0, n // 5, n // 5 + n // 2, n], np.int32)
+    cfg["row_splits"] = rs
+    cfg["dist"] = cfg["dist"] * 0.2
+    cfg["dist"][rs[1]:rs[2]] = 50.0          # event 1: the first point claims every hit
+    cfg["betas"][rs[2]:] = 0.01              # event 2: nothing above the threshold
+    args = (cfg["ccoords"], cfg["betas"], cfg["dist"], cfg["row_splits"], cfg["beta_threshold"])
+    ref = oracle.BuildAndAssignCondensatesBinned(*args, assign_by_max_beta=by_max_beta, keep_noise=True)
+    got = BuildAndAssignCondensatesBinned(*[t(a) for a in args[:4]], args[4], assign_by_max_beta=by_max_beta,
+                                          keep_noise=True)
+    plain = oracle.BuildAndAssignCondensatesBinned(*args, assign_by_max_beta=by_max_beta)
+    assert (plain[0][rs[0]:rs[1]] < 0).any() and (plain[0][rs[1]:rs[2]] >= 0).all() and (plain[0][rs[2]:] < 0).all()
+    for name, g, r in zip(("assignment", "association", "alpha_idx", "is_cond", "n_condensates"), got, ref):
+        g = g.cpu().numpy()
+        assert g.shape == r.shape and g.dtype == r.dtype, name
+        assert (g == r).all(), name
 
 
 def test_condensates_keep_noise_structure(oracle):

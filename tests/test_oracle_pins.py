@@ -259,6 +259,41 @@ def test_accumulate_grad_vs_autograd(oracle):
     assert np.allclose(gx1, tx.grad.numpy(), rtol=1e-5, atol=1e-5)
 
 
+def test_accumulate_knn_grad_chain_through_exp_vs_autograd(oracle):
+    """oracle.AccumulateKnnGrad (the wrapper's gradient w.r.t. the DISTANCES, chained through
+    w = exp(-d) as TF autodiff does, modules/accknn_op.py:52,71-89) against float64 autograd of
+    the whole composition exp -> gather -> mean|max; a missing minus sign, a missing factor w or a
+    gradient taken w.r.t. w instead of d each change the result by O(1)."""
+    import torch
+    rng = np.random.default_rng(17)
+    n, K, F = 80, 7, 4
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    idx = np.stack([np.concatenate([[v], rng.permutation(np.delete(np.arange(n), v))[:K - 1]])
+                    for v in range(n)]).astype(np.int32)
+    idx[5:20, 5:] = -1
+    d = (rng.random((n, K)) * 2.0).astype(np.float32)
+    g = rng.standard_normal((n, 2 * F)).astype(np.float32)
+    out, arg = oracle.AccumulateKnn(d, x, idx)
+    gd, gx = oracle.AccumulateKnnGrad(g, d, x, idx, arg)
+
+    td = torch.tensor(d, dtype=torch.float64, requires_grad=True)
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    tidx = torch.tensor(idx, dtype=torch.int64)
+    valid = (tidx >= 0)[:, :, None]
+    gath = tx[tidx.clamp(min=0)] * torch.exp(-td)[:, :, None]
+    mean = torch.where(valid, gath, torch.zeros_like(gath)).sum(1) / K
+    mx = torch.where(valid, gath, torch.full_like(gath, -1e30)).max(1).values
+    comp = torch.cat([mean, mx], 1)
+    assert np.allclose(comp.detach().numpy(), out, rtol=1e-5, atol=1e-6)
+    (comp * torch.tensor(g, dtype=torch.float64)).sum().backward()
+    assert np.allclose(gd, td.grad.numpy(), rtol=1e-5, atol=1e-6)
+    assert np.allclose(gx, tx.grad.numpy(), rtol=1e-5, atol=1e-5)
+    assert np.abs(td.grad.numpy()).max() > 0.1            # the comparison is not vacuous
+    # linear=True hands the weights through untouched: gradient w.r.t. the weights themselves
+    gw_lin, _ = oracle.AccumulateKnnGrad(g, np.exp(-d).astype(np.float32), x, idx, arg, linear=True)
+    assert np.allclose(-(np.exp(-d.astype(np.float64)) * gw_lin), td.grad.numpy(), rtol=1e-5, atol=1e-6)
+
+
 def test_accumulate_grad_summation_order_and_self_rule(oracle):
     """Feature gradient = ordered scatter of ((g/K)*w + max part); the ordered
     unbuffered numpy scatter reproduces the ascending (vertex, slot) order."""
@@ -613,3 +648,90 @@ def test_condensates_degenerate_coordinates_and_thresholds(oracle, t_b):
                     top = h[np.argmax(beta[h, 0])]
                     assert (asso[rs[e]:rs[e + 1]] == top).all()
         assert (a[alpha, 0] >= 0).all()
+
+
+# ------------------------------------------------------------------ condensates: hand-computed cases
+
+from condensate_cases import CASES as HAND_CASES  # noqa: E402
+
+
+@pytest.mark.parametrize("case", HAND_CASES, ids=[c["name"] for c in HAND_CASES])
+def test_condensates_hand_computed(oracle, case):
+    """literal expectations (tests/condensate_cases.py): the min-distance claim rule
+    `best * r^2 >= d^2` where a plain arg-min, "the first coverer keeps it" and the reference all
+    differ, per-hit radii, a claimed high-beta hit that changes hands, and the pick loop's mask
+    indexing with entry 0 / entry 1 / a later entry set, in one and in two events"""
+    a, s, alpha, is_cond, ncond = oracle.BuildAndAssignCondensatesBinned(
+        case["ccoords"], case["betas"], case["dist"], case["row_splits"], case["beta_threshold"],
+        no_condensation_mask=case["mask"], assign_by_max_beta=case["assign_by_max_beta"])
+    assert a[:, 0].tolist() == case["assignment"].tolist()
+    assert s.tolist() == case["asso"].tolist()
+    assert alpha.tolist() == case["alpha"].tolist()
+    assert ncond.tolist() == case["ncond"].tolist()
+    want_cond = np.zeros(len(s), bool)
+    want_cond[case["alpha"]] = True
+    assert is_cond[:, 0].tolist() == want_cond.tolist()
+
+
+# ------------------------------------------------------------------ keep_noise post-pass
+
+def merge_noise_per_event_loop(assignment, asso, alpha, is_cond, ncond, rs):
+    """modules/assign_condensate_op.py:16-44 event by event with plain lists: noise hit number j of an
+    event (ascending hit index) becomes shower j, the event's real showers move up by its noise count,
+    its list of condensation points is its noise hits followed by its original points, every noise hit
+    is its own condensation point and association target, and the counts are recounted"""
+    new_a, new_alpha, new_n = [], [], [int(ncond[0])]
+    new_asso, new_cond = list(asso), [bool(c) for c in is_cond[:, 0]]
+    for e in range(len(rs) - 1):
+        hits = range(rs[e], rs[e + 1])
+        noise_hits = [i for i in hits if assignment[i, 0] < 0]
+        seen = 0
+        for i in hits:
+            if assignment[i, 0] < 0:
+                new_a.append(seen)
+                seen += 1
+                new_asso[i] = i
+                new_cond[i] = True
+            else:
+                new_a.append(int(assignment[i, 0]) + len(noise_hits))
+        new_alpha += noise_hits + [int(v) for v in alpha[ncond[e]:ncond[e + 1]]]
+        new_n.append(new_n[-1] + sum(new_cond[i] for i in hits))
+    return new_a, new_asso, new_alpha, new_cond, new_n
+
+
+def test_keep_noise_vs_per_event_loop(oracle):
+    rng = np.random.default_rng(61)
+    # three events: mixed, without any noise, all noise
+    rs = np.array([0, 9, 14, 20], np.int32)
+    assignment = np.array([1, -1, 0, -1, -1, 2, 0, 1, -1,   0, 1, 1, 0, 2,   -1, -1, -1, -1, -1, -1], np.int32)[:, None]
+    ncond = np.array([0, 3, 6, 6], np.int32)
+    alpha = np.array([2, 0, 5,   9, 10, 13], np.int32)          # shower s of event e is led by alpha[ncond[e] + s]
+    asso = np.full(20, -1, np.int32)
+    for e in range(3):
+        for i in range(rs[e], rs[e + 1]):
+            if assignment[i, 0] >= 0:
+                asso[i] = alpha[ncond[e] + assignment[i, 0]]
+    is_cond = np.zeros((20, 1), bool)
+    is_cond[alpha, 0] = True
+    got = oracle.merge_noise_as_indiv_cp(assignment, asso, alpha, is_cond, ncond, rs)
+    want = merge_noise_per_event_loop(assignment, asso, alpha, is_cond, ncond, rs)
+    assert got[0][:, 0].tolist() == want[0]
+    assert got[1].tolist() == want[1]
+    assert got[2].tolist() == want[2]
+    assert got[3][:, 0].tolist() == want[3]
+    assert got[4].tolist() == want[4]
+    # spelled out for the first event: noise hits 1, 3, 4, 8 -> showers 0..3, real showers 0, 1, 2 -> 4, 5, 6
+    assert got[0][:9, 0].tolist() == [5, 0, 4, 1, 2, 6, 4, 5, 3]
+    assert got[2][:7].tolist() == [1, 3, 4, 8, 2, 0, 5]
+    assert got[4].tolist() == [0, 7, 10, 16]
+    assert got[1][:9].tolist() == [0, 1, 2, 3, 4, 5, 2, 0, 8]
+    # random events through the whole wrapper
+    cfg = workloads.cfg5(scale=0.004, n_events=3)
+    args = (cfg["ccoords"], cfg["betas"], cfg["dist"], cfg["row_splits"], 0.4)
+    plain = oracle.BuildAndAssignCondensatesBinned(*args, assign_by_max_beta=True)
+    kept = oracle.BuildAndAssignCondensatesBinned(*args, assign_by_max_beta=True, keep_noise=True)
+    want = merge_noise_per_event_loop(*plain, cfg["row_splits"])
+    assert (plain[0] < 0).any()
+    assert kept[0][:, 0].tolist() == want[0] and kept[1].tolist() == want[1] and kept[2].tolist() == want[2]
+    assert kept[3][:, 0].tolist() == want[3] and kept[4].tolist() == want[4]
+    del rng

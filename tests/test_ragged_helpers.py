@@ -89,3 +89,37 @@ def test_ragged_indices_single_event_and_all_noise():
     assert calc_ragged_shower_indices(a, rs, gather_noise=False).to_list() == [[]]
     rc, rev, flat = calc_ragged_cond_indices(a, torch.empty((0,), dtype=torch.int32), None, rs)
     assert rc.to_list() == [[[2]]] and rev.tolist() == [[0, 0]] * 3 and flat[:, 0].tolist() == [0, 0, 0]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_merge_noise_as_indiv_cp_vs_per_event_loop(seed):
+    """the keep_noise post-pass (modules/assign_condensate_op.py:16-44) of the package, on CPU tensors,
+    against the per-event list loop that also pins the oracle: numbering of the noise hits (ascending
+    hit index, before the real showers), order of the merged condensation point list, flags, counts"""
+    from hgcalml_amd.assign_condensate_op import merge_noise_as_indiv_cp
+    from test_oracle_pins import merge_noise_per_event_loop
+    rng = np.random.default_rng(100 + seed)
+    a, rs, alpha = random_assignment(rng, 5, True)
+    if seed == 0:   # one event that is all noise, at the end
+        a = np.concatenate([a, -np.ones(4, np.int32)])
+        rs = np.concatenate([rs, [rs[-1] + 4]]).astype(np.int32)
+    n_events = len(rs) - 1
+    per_event = [int(a[rs[e]:rs[e + 1]].max()) + 1 for e in range(n_events)]
+    ncond = np.concatenate([[0], np.cumsum(per_event)]).astype(np.int32)
+    asso = np.full(len(a), -1, np.int32)
+    for e in range(n_events):
+        for i in range(rs[e], rs[e + 1]):
+            if a[i] >= 0:
+                asso[i] = alpha[ncond[e] + a[i]]
+    is_cond = np.zeros((len(a), 1), bool)
+    is_cond[alpha, 0] = True
+    assert any((a[rs[e]:rs[e + 1]] >= 0).all() for e in range(n_events))       # an event without noise
+    got = merge_noise_as_indiv_cp(torch.from_numpy(a)[:, None], torch.from_numpy(asso), torch.from_numpy(alpha),
+                                  torch.from_numpy(is_cond), torch.from_numpy(ncond), torch.from_numpy(rs))
+    want = merge_noise_per_event_loop(a[:, None], asso, alpha, is_cond, ncond, rs)
+    assert got[0][:, 0].tolist() == want[0]
+    assert got[1].tolist() == want[1]
+    assert got[2].tolist() == want[2]
+    assert got[3][:, 0].tolist() == want[3]
+    assert got[4].tolist() == want[4]
+    assert got[0].dtype == torch.int32 and got[3].dtype == torch.bool
