@@ -239,7 +239,7 @@ def main():
         m3 = event_ms(lambda: BinnedSelectKnn(c3["K"], co3, rs3, n_bins=c3["n_bins"], max_radius=c3["max_radius"]), 5, 2)
         extra["cfg3_knn_ms"] = round(m3[0], 3)
         extra["cfg3_queries_per_s"] = round(len(c3["coords"]) / (m3[0] * 1e-3), 1)
-        c5 = workloads.cfg5()
+        c5 = workloads.cfg5(ragged=True)
         a5 = [torch.from_numpy(c5[k]).to(dev) for k in ("ccoords", "betas", "dist", "row_splits")]
         for mode in (True, False):
             m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode), 5, 2)
@@ -279,7 +279,7 @@ def main():
         f_s, b_s = cpu_baseline_accumulate(small)
         ns = len(small["indices"])
         import oracle
-        c5_cpu = workloads.cfg5()
+        c5_cpu = workloads.cfg5(ragged=True)
         t_c = time.perf_counter()
         oracle.BuildAndAssignCondensatesBinned(c5_cpu["ccoords"], c5_cpu["betas"], c5_cpu["dist"], c5_cpu["row_splits"],
                                                c5_cpu["beta_threshold"], assign_by_max_beta=True)
@@ -291,7 +291,7 @@ def main():
                                                  (f_s + b_s) / 1e9, 4),
                "accumulate_sample": "cfg4 at N=%d (fwd %.2f s, grad %.2f s)" % (ns, f_s, b_s),
                "condensates_cfg5_ms": round(cond_s * 1e3, 1),
-               "condensates_sample": "all of cfg5 (8 events, 500k hits, max-beta mode) through the oracle's wrapper "
+               "condensates_sample": "all of cfg5 (8 uneven events, 500k hits, max-beta mode) through the oracle's wrapper "
                                      "(numpy glue + C kernel)",
                "value_unoptimised_build": None if qps_o0 is None else round(qps_o0, 1),
                "unoptimised_note": "same kernel built -O0 (the reference's Makefile passes no -O flag), one pass",

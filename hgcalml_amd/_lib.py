@@ -20,6 +20,7 @@ _ptr = ctypes.c_void_p
 _SIGNATURES = {
     "hgc_version": (_c_int, []),
     "hgc_last_error": (ctypes.c_char_p, []),
+    "hgc_set_status_word": (_c_int, [_ptr]),
     "hgc_bin_by_coordinates_total_bins": (_c_int, [_ptr, _c_int, _c_int, _ptr]),
     "hgc_bin_by_coordinates": (_c_int, [_ptr] * 7 + [_c_int] * 5 + [_ptr]),
     "hgc_bin_by_coordinates_strided": (_c_int, [_ptr, _c_int] + [_ptr] * 8 + [_c_int] * 5 + [_ptr]),

@@ -5,7 +5,24 @@ import math
 
 import torch
 
+from . import globals as gl
 from . import ops
+
+
+def check_condensate_counts(assignment, n_condensates, row_splits):
+    """the reference's closing sanity check (modules/assign_condensate_op.py:334-343):
+    n_condensates == [0] ++ cumsum(per event: largest shower index + 1). Events without hits
+    count as 0 (the reference's reduce_max has no value there). One host synchronisation."""
+    a = assignment[:, 0].to(torch.int64)
+    rs = row_splits.to(device=a.device, dtype=torch.int64)
+    n_events = rs.numel() - 1
+    seg = torch.searchsorted(rs[1:].contiguous(), torch.arange(a.numel(), device=a.device), right=True)
+    per_event = torch.full((n_events,), -1, dtype=torch.int64, device=a.device).scatter_reduce(
+        0, seg, a, reduce="amax", include_self=True) + 1
+    expected = torch.cat([torch.zeros(1, dtype=torch.int64, device=a.device), torch.cumsum(per_event, 0)])
+    if not torch.equal(expected, n_condensates.to(torch.int64)):
+        raise RuntimeError("BuildAndAssignCondensatesBinned: n_condensates %s does not match the assignment (%s)"
+                           % (n_condensates.tolist(), expected.tolist()))
 
 
 def merge_noise_as_indiv_cp(assignment, asso_idx, alpha_idx, is_cond, n_condensates, row_splits):
@@ -72,6 +89,8 @@ def BuildAndAssignCondensatesBinned(ccoords, betas, dist, row_splits, beta_thres
     out = (assignment[:, None], asso, alpha_idx, is_cond[:, None], n_condensates)
     if keep_noise:
         out = merge_noise_as_indiv_cp(*out, row_splits)
+    if gl.debug_checks:
+        check_condensate_counts(out[0], out[4], row_splits)
     return out
 
 

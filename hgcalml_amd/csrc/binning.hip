@@ -24,6 +24,9 @@ namespace hgc {
 thread_local char g_last_error[512] = "";
 char *last_error_buffer() { return g_last_error; }
 
+thread_local int *g_status_word = nullptr;
+int *status_word() { return g_status_word; }
+
 namespace {
 
 constexpr int kMaxBinDims = 8;
@@ -149,13 +152,15 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
     const float *__restrict__ coords, int stride, const float *__restrict__ shift,
     const int *__restrict__ row_splits, const float *__restrict__ bin_width, const int *__restrict__ n_bins,
     int *__restrict__ binass, int *__restrict__ flat, int *__restrict__ n_per_bin,
-    int *__restrict__ n_out_of_range, int n_vert, int n_dims, int n_rs, int n_total_bins, int calc_n_per_bin) {
+    int *__restrict__ n_out_of_range, int *__restrict__ status, int n_vert, int n_dims, int n_rs, int n_total_bins,
+    int calc_n_per_bin) {
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= n_vert) return;
     const float bw = bin_width[0];
-    int mul = 1, cell = 0, bad = 0;
+    int mul = 1, cell = 0, bad = 0, flags = 0;
     for (int c = n_dims - 1; c >= 0; --c) {
         float x = coords[(size_t)p * stride + c];
+        if (!isfinite(x)) flags |= HGC_FLAG_COORDINATE_NOT_FINITE;
         if (shift) x = x - shift[c];
         int k = (int)(x / bw);
         const int nb = n_bins[c];
@@ -180,6 +185,8 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
     const int ev = lo - 1;
     cell += ev * mul;
     if (bad && n_out_of_range) atomicAdd(n_out_of_range, bad);
+    if (bad) flags |= HGC_FLAG_COORDINATE_OUT_OF_GRID;
+    if (flags && status) atomicOr(status, flags);
     if (cell >= n_total_bins) return;
     binass[(size_t)p * (n_dims + 1)] = ev;
     flat[p] = cell;
@@ -214,7 +221,8 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const uint32_t *__rest
 }
 
 __global__ __launch_bounds__(256) void index_replacer_kernel(const int *__restrict__ tbr, const int *__restrict__ repl,
-                                                             int *__restrict__ out, int n, int n_repl) {
+                                                             int *__restrict__ out, int *__restrict__ status, int n,
+                                                             int n_repl) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const int v = tbr[i];
@@ -222,6 +230,8 @@ __global__ __launch_bounds__(256) void index_replacer_kernel(const int *__restri
         out[i] = v;
     else if (v < n_repl)
         out[i] = repl[v];
+    else if (status)
+        atomicOr(status, HGC_FLAG_REPLACEMENT_OUT_OF_RANGE);
 }
 
 // ---- bin order by counting (no order guarantee inside a bin) -------------------
@@ -237,7 +247,7 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
     const int *__restrict__ row_splits, int n_vert, int n_dims, int n_rs, int n_bins_scalar,
     float *__restrict__ shift_out, float *__restrict__ bin_width_out, int *__restrict__ n_bins_out,
     int *__restrict__ binass, int *__restrict__ flat, int *__restrict__ rank, int *__restrict__ counts,
-    int n_bins_bound, int sub_shift) {
+    int n_bins_bound, int sub_shift, int *__restrict__ status) {
     __shared__ float s_lo[4][kMaxBinDims], s_hi[4][kMaxBinDims];
     __shared__ float s_shift[kMaxBinDims], s_bw;
     __shared__ int s_nb[kMaxBinDims];
@@ -276,12 +286,17 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
     __syncthreads();
     const float bw = s_bw;
     for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < n_vert; p += gridDim.x * blockDim.x) {
-        int mul = 1, cell = 0;
+        int mul = 1, cell = 0, flags = 0;
         for (int c = n_dims - 1; c >= 0; --c) {
-            const float x = coords[(size_t)p * stride + c] - s_shift[c];
+            const float raw = coords[(size_t)p * stride + c];
+            if (!isfinite(raw)) flags |= HGC_FLAG_COORDINATE_NOT_FINITE;
+            const float x = raw - s_shift[c];
             int k = (int)(x / bw);
             const int nb = s_nb[c];
-            if (k < 0 || k >= nb) k = 0;
+            if (k < 0 || k >= nb) {
+                k = 0;
+                flags |= HGC_FLAG_COORDINATE_OUT_OF_GRID;
+            }
             binass[(size_t)p * (n_dims + 1) + c + 1] = k;
             cell += k * mul;
             mul *= nb;
@@ -296,6 +311,7 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
         }
         const int ev = lo - 1;
         cell += ev * mul;
+        if (flags && status) atomicOr(status, flags);
         cell = min(cell, n_bins_bound - 1);  // no effect for row splits that end at n_vert
         binass[(size_t)p * (n_dims + 1)] = ev;
         flat[p] = cell;
@@ -390,7 +406,8 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
     if (rc) return rc;
     bin_points_ranked_kernel<<<std::min(4096, ceil_div(n_vert, 256)), 256, 0, s>>>(d_coords, n_coords, partial, blocks, d_row_splits, n_vert,
                                                     n_bin_dims, n_rs, n_bins_scalar, d_shift, d_bin_width, d_n_bins,
-                                                    binass, flat, rank, counts, n_bins_bound, sub_shift);
+                                                    binass, flat, rank, counts, n_bins_bound, sub_shift,
+                                                    status_word());
     rc = check_launch("bin_points_ranked");
     if (rc) return rc;
     // boundaries[b << sub_shift] = number of points in bins below b
@@ -410,7 +427,12 @@ using namespace hgc;
 
 extern "C" {
 
-int hgc_version(void) { return 100; }
+int hgc_version(void) { return 101; }
+
+int hgc_set_status_word(int *d_word) {
+    hgc::g_status_word = d_word;
+    return HGC_OK;
+}
 
 const char *hgc_last_error(void) { return hgc::last_error_buffer(); }
 
@@ -449,8 +471,8 @@ int hgc_bin_by_coordinates_strided(const float *d_coords, int coord_stride, cons
     HGC_REQUIRE(!calc_n_per_bin || d_n_per_bin, "calc_n_per_bin needs d_n_per_bin");
     bin_points_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, coord_stride, d_shift, d_rs, d_binswidth,
                                                             d_n_bins, d_assigned_bin, d_flat_assigned_bin,
-                                                            d_n_per_bin, d_n_out_of_range, n_vert, n_bin_dims,
-                                                            n_rs, n_total_bins, calc_n_per_bin);
+                                                            d_n_per_bin, d_n_out_of_range, status_word(), n_vert,
+                                                            n_bin_dims, n_rs, n_total_bins, calc_n_per_bin);
     return check_launch("bin_points");
 }
 
@@ -553,7 +575,7 @@ int hgc_index_replacer(const int *d_to_be_replaced, const int *d_replacements, i
     if (n_to_be_replaced == 0) return HGC_OK;
     HGC_REQUIRE(d_to_be_replaced && d_replaced && (d_replacements || n_replacements == 0), "null pointer");
     index_replacer_kernel<<<ceil_div(n_to_be_replaced, 256), 256, 0, as_stream(stream)>>>(
-        d_to_be_replaced, d_replacements, d_replaced, n_to_be_replaced, n_replacements);
+        d_to_be_replaced, d_replacements, d_replaced, status_word(), n_to_be_replaced, n_replacements);
     return check_launch("index_replacer");
 }
 

@@ -18,6 +18,9 @@ constexpr int kNumXcd = 8;  // MI355X: 8 accelerator complex dies, one L2 each
 
 char *last_error_buffer();  // thread local, 512 bytes
 
+// device status word of the calling thread (hgc_set_status_word), or nullptr
+int *status_word();
+
 inline int fail(int code, const char *fmt, ...) {
     va_list ap;
     va_start(ap, fmt);

@@ -50,6 +50,7 @@ struct KnnParams {
     const float *shift;  // may be null: what the binning subtracted from the binned coordinates
     int *out_idx;
     float *out_dist;
+    int *status;      // may be null: device status word for data errors
     float radius_sq;  // < 0: no radius
     int n_vert, K, n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction;
     int boundary_shift;  // the boundary of bin b sits at bin_boundaries[b << boundary_shift]
@@ -246,7 +247,7 @@ constexpr int kMarkCap = 2048;
 // against 0.78 ms with 4 and 0.95 ms with 8).
 constexpr int kQueriesPerBlock = 1;
 
-// q = x / w, r = x % w for 0 <= x < 2^23 and small w, without an integer divide:
+// q = x / w, r = x % w for 0 <= x < 2^24 and w < 2^13, without an integer divide:
 // the float quotient is off by at most one, the remainder says which way
 __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, int &r) {
     q = (int)((float)x * inv_w);
@@ -360,10 +361,17 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                                    p.bin_boundaries[(size_t)own << p.boundary_shift] <= Kn;
         }
         for (int d = with_own_bin ? 1 : 0; d <= reach_max; ++d) {
+            // a shell is walked as W^(B-1) rows of bins; the row number has to stay exact as a float
+            // (divmod_small) and 2 * rows inside an int
+            long long rows64 = d < (1 << 12) ? 1 : 1ll << 24;
+            for (int i = 0; i < B - 1; ++i) rows64 = min(rows64 * (2 * min(d, 1 << 12) + 1), 1ll << 24);
+            if (rows64 >= 1ll << 24) {
+                if (p.status && lane == 0) atomicOr(p.status, HGC_FLAG_SHELL_TOO_WIDE);
+                break;
+            }
             const int W = 2 * d + 1;
             const float inv_W = 1.f / (float)W;
-            int n_rows = 1;
-            for (int i = 0; i < B - 1; ++i) n_rows *= W;
+            const int n_rows = (int)rows64;
             const int n_slots = d == 0 ? 1 : 2 * n_rows;
 
             for (int slot0 = 0; slot0 < n_slots; slot0 += kWave) {
@@ -431,6 +439,8 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                         if (last < p.n_bboundaries) {
                             seg_start = p.bin_boundaries[(size_t)first << p.boundary_shift];
                             seg_len = p.bin_boundaries[(size_t)last << p.boundary_shift] - seg_start;
+                        } else if (p.status) {  // the reference prints "idx out of range" and skips the bin
+                            atomicOr(p.status, HGC_FLAG_BIN_BEYOND_TABLE);
                         }
                     }
                 }
@@ -609,6 +619,7 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
     p.shift = d_shift;
     p.out_idx = d_indices;
     p.out_dist = d_dist;
+    p.status = status_word();
     p.radius_sq = max_radius > 0.f ? max_radius * max_radius : -1.f;
     p.n_vert = n_vert;
     p.K = n_neigh;

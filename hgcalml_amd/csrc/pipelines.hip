@@ -387,6 +387,12 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
     HGC_REQUIRE(n_bins_scalar >= 1, "n_bins must be positive");
     HGC_REQUIRE(n_bin_dims > 1, "BinnedSelectKnnOp expects at least 2 binning dimensions.");
     HGC_REQUIRE(n_bin_dims < 6, "BinnedSelectKnnOp expects maximum 5 binning dimensions.");
+    {   // the widest shell a query can reach, (2 (n_bins + 1) + 1)^(B - 1) rows of bins, has to stay below 2^24
+        long long rows = 1;
+        for (int i = 0; i < n_bin_dims - 1; ++i) rows = std::min(rows * (2ll * (n_bins_scalar + 1) + 1), 1ll << 40);
+        HGC_REQUIRE(rows < (1ll << 24), "n_bins = %d is too fine for %d binned dimensions (a shell of the walk would "
+                    "have %lld rows of bins, the limit is 2^24)", n_bins_scalar, n_bin_dims, rows);
+    }
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_coords && d_row_splits && d_indices && d_dist, "null pointer");
     const int use_direction = d_direction != nullptr;

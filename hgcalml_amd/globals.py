@@ -1,5 +1,18 @@
-"""Module-level switches with the names of the reference's modules/globals.py:91-92.
-When set, the wrappers use plain torch compositions (differentiable by autograd)
-instead of the custom kernels."""
+"""Module-level switches.
+
+`knn_ops_use_tf_gradients` and `acc_ops_use_tf_gradients` have the names of the
+reference's modules/globals.py:91-92: when set, the wrappers use plain torch
+compositions (differentiable by autograd) instead of the custom kernels.
+
+`debug_checks` has no counterpart there. The reference's kernels print a line
+when they meet bad data and its wrappers run tf.debugging.check_numerics and a
+consistency assert on every call; here those checks cost a device-to-host read,
+so they run only while this switch is on: the wrappers then read the library's
+device status word after each call, raise on non finite coordinates
+(modules/bin_by_coordinates_op.py:46) and on the condensate count relation
+(modules/assign_condensate_op.py:334-343), and warn where the reference prints
+and continues (a coordinate outside the grid, a bin beyond the boundary table,
+an index beyond the replacement table)."""
 knn_ops_use_tf_gradients = False
 acc_ops_use_tf_gradients = False
+debug_checks = False

@@ -5,12 +5,63 @@ Inputs/outputs follow the reference's REGISTER_OP blocks
 (modules/compiled/*_module.cc): same order, same dtypes. All tensors live on
 the GPU; the work is enqueued on torch's current HIP stream.
 """
+import contextlib
+import warnings
 import weakref
 
 import torch
 
 from . import _lib
+from . import globals as gl
 from ._lib import check, f32, i32, lib, p, require_device, stream, workspace
+
+
+# --------------------------------------------------------------------------- data errors
+
+FLAG_COORDINATE_OUT_OF_GRID = 1
+FLAG_COORDINATE_NOT_FINITE = 2
+FLAG_BIN_BEYOND_TABLE = 4
+FLAG_REPLACEMENT_OUT_OF_RANGE = 8
+FLAG_SHELL_TOO_WIDE = 16
+
+
+class DataWarning(UserWarning):
+    """bad data the kernels worked around with the reference's fallback (the reference prints a line)"""
+
+
+def report_data_flags(flags, what):
+    """Turns the bits of the library's status word into the reference's reactions: an exception
+    for non finite coordinates (tf.debugging.check_numerics, modules/bin_by_coordinates_op.py:46),
+    warnings where its kernels print and continue (bin_by_coordinates_kernel.cc:75-78,
+    binned_select_knn_kernel.cc:146-149, index_replacer_kernel.cc:35-38)."""
+    if flags & FLAG_COORDINATE_NOT_FINITE:
+        raise ValueError("%s: input coordinates : Tensor had NaN or Inf values" % what)
+    if flags & FLAG_COORDINATE_OUT_OF_GRID:
+        warnings.warn("%s: coordinate outside the grid, assigned to bin 0 in that dimension" % what, DataWarning)
+    if flags & FLAG_BIN_BEYOND_TABLE:
+        warnings.warn("%s: bin index out of range of the bin boundaries, bin skipped" % what, DataWarning)
+    if flags & FLAG_REPLACEMENT_OUT_OF_RANGE:
+        warnings.warn("%s: index out of range of the replacements, entry left untouched" % what, DataWarning)
+    if flags & FLAG_SHELL_TOO_WIDE:
+        warnings.warn("%s: the grid is too fine for the walk over shells of bins; the neighbours of some points "
+                      "are incomplete" % what, DataWarning)
+
+
+@contextlib.contextmanager
+def data_checks(what, device):
+    """While hgcalml_amd.globals.debug_checks is set: the library calls made inside report the bad
+    data they meet into a status word on the device, which is read (one synchronisation) and
+    acted upon at the end. Otherwise nothing happens and nothing is synchronised."""
+    if not gl.debug_checks:
+        yield
+        return
+    word = torch.zeros(1, dtype=torch.int32, device=device)
+    check(lib.hgc_set_status_word(p(word)))
+    try:
+        yield
+    finally:
+        check(lib.hgc_set_status_word(None))
+    report_data_flags(int(word.item()), what)
 
 
 # --------------------------------------------------------------------------- binning
@@ -31,8 +82,10 @@ def bin_by_coordinates(coordinates: torch.Tensor, row_splits: torch.Tensor, bin_
     binass = torch.zeros((n, c + 1), dtype=torch.int32, device=dev)
     flat = torch.zeros((n,), dtype=torch.int32, device=dev)
     nper = torch.empty((n_total_bins,), dtype=torch.int32, device=dev)
-    check(lib.hgc_bin_by_coordinates(p(coordinates), p(row_splits), p(bin_width), p(nbins), p(binass), p(flat),
-                                     p(nper), n, c, row_splits.numel(), n_total_bins, int(calc_n_per_bin), stream()))
+    with data_checks("BinByCoordinates", dev):
+        check(lib.hgc_bin_by_coordinates(p(coordinates), p(row_splits), p(bin_width), p(nbins), p(binass), p(flat),
+                                         p(nper), n, c, row_splits.numel(), n_total_bins, int(calc_n_per_bin),
+                                         stream()))
     return binass, flat, nper
 
 
@@ -57,9 +110,10 @@ def bin_points(coords, n_bin_dims, shift, row_splits, bin_width, nbins, n_total_
     binass = torch.zeros((n, n_bin_dims + 1), dtype=torch.int32, device=dev)
     flat = torch.zeros((n,), dtype=torch.int32, device=dev)
     nper = torch.empty((n_total_bins,), dtype=torch.int32, device=dev) if calc_n_per_bin else None
-    check(lib.hgc_bin_by_coordinates_strided(p(coords), c, p(shift), p(row_splits), p(bin_width), p(nbins), p(binass),
-                                             p(flat), p(nper), None, n, n_bin_dims, row_splits.numel(), n_total_bins,
-                                             int(calc_n_per_bin), stream()))
+    with data_checks("BinByCoordinates", dev):
+        check(lib.hgc_bin_by_coordinates_strided(p(coords), c, p(shift), p(row_splits), p(bin_width), p(nbins),
+                                                 p(binass), p(flat), p(nper), None, n, n_bin_dims, row_splits.numel(),
+                                                 n_total_bins, int(calc_n_per_bin), stream()))
     return binass, flat, nper
 
 
@@ -126,11 +180,12 @@ def binned_select_knn_fused(coords, bin_idx, dim_bin_idx, bin_boundaries, n_bins
     n, c = coords.shape
     idx = torch.empty((n, n_neighbours), dtype=torch.int32, device=dev)
     dist = torch.empty((n, n_neighbours), dtype=torch.float32, device=dev)
-    check(lib.hgc_binned_select_knn_fused(p(coords), p(bin_idx), p(direction), p(dim_bin_idx), p(bin_boundaries),
-                                          p(n_bins), p(bin_width), p(sorting), None,
-                                          float(max_radius) if max_radius is not None else -1.0, p(idx), p(dist), n,
-                                          int(n_neighbours), c, n_bins.numel(), bin_boundaries.numel(),
-                                          int(tf_compatible), int(use_direction), stream()))
+    with data_checks("BinnedSelectKnn", dev):
+        check(lib.hgc_binned_select_knn_fused(p(coords), p(bin_idx), p(direction), p(dim_bin_idx), p(bin_boundaries),
+                                              p(n_bins), p(bin_width), p(sorting), None,
+                                              float(max_radius) if max_radius is not None else -1.0, p(idx), p(dist),
+                                              n, int(n_neighbours), c, n_bins.numel(), bin_boundaries.numel(),
+                                              int(tf_compatible), int(use_direction), stream()))
     return idx, dist
 
 
@@ -145,10 +200,12 @@ def binned_select_knn_pipeline(coords, row_splits, direction, n_neighbours, n_bi
     nbytes = lib.hgc_binned_select_knn_pipeline_workspace_bytes(n, c, row_splits.numel(), int(n_bins), int(max_bin_dims),
                                                                 int(direction is not None))
     ws = workspace(nbytes, dev)
-    check(lib.hgc_binned_select_knn_pipeline(p(coords), p(row_splits), p(direction), n, c, row_splits.numel(),
-                                             int(n_neighbours), int(n_bins), int(max_bin_dims), int(tf_compatible),
-                                             float(max_radius) if max_radius is not None else -1.0, p(idx), p(dist),
-                                             p(sorting), p(ws), ws.numel(), stream()))
+    with data_checks("BinnedSelectKnn", dev):
+        check(lib.hgc_binned_select_knn_pipeline(p(coords), p(row_splits), p(direction), n, c, row_splits.numel(),
+                                                 int(n_neighbours), int(n_bins), int(max_bin_dims),
+                                                 int(tf_compatible),
+                                                 float(max_radius) if max_radius is not None else -1.0, p(idx),
+                                                 p(dist), p(sorting), p(ws), ws.numel(), stream()))
     # the points' bin order is a processing order with locality for everything that runs over this table
     set_vertex_order(idx, sorting)
     return idx, dist
@@ -157,10 +214,11 @@ def binned_select_knn_pipeline(coords, row_splits, direction, n_neighbours, n_bi
 @torch.library.custom_op("hgcalml::index_replacer", mutates_args=())
 def index_replacer(to_be_replaced: torch.Tensor, replacements: torch.Tensor) -> torch.Tensor:
     """modules/compiled/index_replacer_module.cc:7-10"""
-    require_device(to_be_replaced, replacements)
+    dev = require_device(to_be_replaced, replacements)
     tbr, rep = i32(to_be_replaced), i32(replacements)
     out = torch.zeros_like(tbr)
-    check(lib.hgc_index_replacer(p(tbr), p(rep), p(out), tbr.numel(), rep.numel(), stream()))
+    with data_checks("IndexReplacer", dev):
+        check(lib.hgc_index_replacer(p(tbr), p(rep), p(out), tbr.numel(), rep.numel(), stream()))
     return out
 
 
@@ -492,10 +550,12 @@ def build_and_assign_condensates(ccoords, betas, dist, mask, row_splits, beta_th
     is_cond = torch.empty((n,), dtype=torch.bool, device=dev)
     ncond = torch.empty((num_rows + 1,), dtype=torch.int32, device=dev)
     ws = workspace(lib.hgc_build_and_assign_condensates_workspace_bytes(n, c, num_rows, n_bins_scalar, nbin_dims), dev)
-    check(lib.hgc_build_and_assign_condensates(p(ccoords), p(betas), p(dist), p(mask), p(row_splits), n, c, num_rows,
-                                               float(beta_threshold), float(distance_threshold),
-                                               int(assign_by_max_beta), nbin_dims, n_bins_scalar, p(assignment),
-                                               p(asso), p(alpha), p(is_cond), p(ncond), p(ws), ws.numel(), stream()))
+    with data_checks("BuildAndAssignCondensatesBinned", dev):
+        check(lib.hgc_build_and_assign_condensates(p(ccoords), p(betas), p(dist), p(mask), p(row_splits), n, c,
+                                                   num_rows, float(beta_threshold), float(distance_threshold),
+                                                   int(assign_by_max_beta), nbin_dims, n_bins_scalar, p(assignment),
+                                                   p(asso), p(alpha), p(is_cond), p(ncond), p(ws), ws.numel(),
+                                                   stream()))
     total = int(ncond[-1]) if n > 0 else 0
     return assignment, asso, alpha[:total], is_cond, ncond
 

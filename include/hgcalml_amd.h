@@ -46,6 +46,29 @@ int hgc_version(void);
 /* Human readable text for the last error raised on the calling thread. */
 const char *hgc_last_error(void);
 
+/* Data errors. The reference's kernels print a line and carry on with a
+ * fallback when they meet bad DATA (a coordinate outside the grid goes to bin 0,
+ * modules/compiled/bin_by_coordinates_kernel.cc:75-78; a shell bin beyond the
+ * boundary table is skipped, binned_select_knn_kernel.cc:146-149; an index
+ * beyond the replacement table is left alone, index_replacer_kernel.cc:35-38),
+ * and the Python wrapper refuses non finite coordinates
+ * (modules/bin_by_coordinates_op.py:46, tf.debugging.check_numerics). Here the
+ * fallbacks are the same and the print becomes a bit in a device status word:
+ * after hgc_set_status_word(d_word) every call made by the calling thread ORs
+ * the hgc_data_flag bits of what its kernels met into *d_word (one int32 of
+ * device memory, owned and zeroed by the caller, read after the stream has been
+ * synchronised). NULL (the initial state) switches the reporting off. The
+ * setting is per thread; it adds no launch and no synchronisation. */
+enum hgc_data_flag {
+    HGC_FLAG_COORDINATE_OUT_OF_GRID = 1,  /* a binned coordinate fell outside the grid: bin 0 in that dimension */
+    HGC_FLAG_COORDINATE_NOT_FINITE = 2,   /* NaN or Inf among the binned coordinates */
+    HGC_FLAG_BIN_BEYOND_TABLE = 4,        /* kNN: a bin of the walk lies beyond d_bin_boundaries: skipped */
+    HGC_FLAG_REPLACEMENT_OUT_OF_RANGE = 8, /* index replacer: entry >= n_replacements: left untouched */
+    HGC_FLAG_SHELL_TOO_WIDE = 16          /* kNN: a query's walk reached a shell of 2^24 or more rows of bins
+                                             ((2d+1)^(n_bin_dim-1) at shell distance d) and ended there */
+};
+int hgc_set_status_word(int *d_word);
+
 /* ------------------------------------------------------------------ */
 /* Spatial binning                                                     */
 /* ------------------------------------------------------------------ */
@@ -129,8 +152,13 @@ int hgc_gather_rows(const void *d_in, const int *d_rows, void *d_out, int n_rows
  * (or (self, 0.0) if tf_compat) at the tail. The reference leaves the slots in
  * fill/replacement order; the neighbour SET is the same except where the K-th
  * and (K+1)-th distances are exactly equal, where the lower index is kept.
- * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, 1 <= n_neigh <= 513,
- * n_vert * n_neigh < 2^31, coordinate matrix below 4 GiB. */
+ * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, 1 <= n_neigh <= 513 (the
+ * reference has no limit on n_neigh), n_vert * n_neigh < 2^31, coordinate matrix
+ * below 4 GiB. A shell at distance d is walked as (2d+1)^(n_bin_dim-1) rows of
+ * bins; a query whose walk would reach a shell of 2^24 rows or more (grids far
+ * finer than the points are dense, e.g. 5 binned dimensions with more than 30
+ * bins each) ends there and sets HGC_FLAG_SHELL_TOO_WIDE in the status word;
+ * hgc_binned_select_knn_pipeline refuses such grids on the host instead. */
 int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int *d_direction,
                           const int *d_dim_bin_idx, const int *d_bin_boundaries,
                           const int *d_n_bins, const float *d_bin_width,

@@ -1115,9 +1115,14 @@ def test_condensates_cfg5_scaled(oracle, by_max_beta):
     assert int(got[4][-1]) > 50
 
 
+@pytest.mark.parametrize("ragged", [True, False])
 @pytest.mark.parametrize("by_max_beta", [True, False])
-def test_condensates_cfg5_full(oracle, by_max_beta):
-    run_condensates(oracle, workloads.cfg5(), by_max_beta)
+def test_condensates_cfg5_full(oracle, by_max_beta, ragged):
+    """500,000 hits in 8 events, uneven (26k to 112k hits) or equal"""
+    cfg = workloads.cfg5(ragged=ragged)
+    sizes = np.diff(cfg["row_splits"])
+    assert sizes.sum() == 500000 and (not ragged or sizes.max() > 3 * sizes.min())
+    run_condensates(oracle, cfg, by_max_beta)
 
 
 @pytest.mark.parametrize("radius", [0.004, 0.03])

@@ -108,19 +108,27 @@ def cfg4(scale=1.0, seed=1004, window=2000):
                 grad_out=rng.standard_normal((n, 2 * F), dtype=np.float32))
 
 
-def cfg5(scale=1.0, seed=1005, n_events=8):
+def cfg5(scale=1.0, seed=1005, n_events=8, ragged=False):
+    """ragged=True: event sizes drawn from U{20k..120k} and rescaled to the same total
+    (500,000 * scale for 8 events); otherwise equal events."""
     rng = np.random.default_rng(seed)
     per = max(64, int(62500 * scale))
+    sizes = np.full(n_events, per, np.int64)
+    if ragged:
+        draw = np.random.default_rng(seed + 7).integers(20000, 120001, n_events).astype(np.float64)
+        sizes = np.maximum(64, np.floor(draw / draw.sum() * per * n_events)).astype(np.int64)
+        sizes[-1] += per * n_events - sizes.sum()
     coords, betas = [], []
-    for _ in range(n_events):
-        x, _, rel = cluster_mixture(rng, per, 4, return_truth=True)
-        b = rng.beta(0.5, 2.0, size=per).astype(np.float32)
+    for m in sizes:
+        m = int(m)
+        x, _, rel = cluster_mixture(rng, m, 4, return_truth=True)
+        b = rng.beta(0.5, 2.0, size=m).astype(np.float32)
         core = rel < 1.0  # "core" = within one sigma of the own cluster centre
         b = np.where(core, np.minimum(b + np.float32(0.5), np.float32(0.999)), b).astype(np.float32)
         coords.append(x)
         betas.append(b)
-    n = per * n_events
+    n = int(sizes.sum())
     return dict(name="cfg5", ccoords=np.concatenate(coords), betas=np.concatenate(betas)[:, None],
                 dist=np.full((n, 1), 0.5, np.float32),
-                row_splits=(np.arange(n_events + 1) * per).astype(np.int32),
+                row_splits=np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32),
                 beta_threshold=0.1, distance_threshold=1.0)
