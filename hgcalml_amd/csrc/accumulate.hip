@@ -514,27 +514,6 @@ __global__ __launch_bounds__(256) void weight_grad_wave_kernel(const float *__re
 
 // ------------------------------------------------------------------ inverse index
 
-// sort key of a neighbour slot: its target, or n_vert for "no neighbour" (sorts last)
-struct InverseKey {
-    unsigned n_vert;
-    __host__ __device__ unsigned operator()(int j) const { return (unsigned)j < n_vert ? (unsigned)j : n_vert; }
-};
-
-__global__ __launch_bounds__(256) void inverse_offsets_kernel(const unsigned int *__restrict__ sorted_keys,
-                                                              long long total, int *__restrict__ offsets, int n_vert) {
-    const int m = blockIdx.x * blockDim.x + threadIdx.x;
-    if (m > n_vert) return;
-    long long lo = 0, hi = total;  // first position whose key is >= m
-    while (lo < hi) {
-        long long mid = (lo + hi) >> 1;
-        if (sorted_keys[mid] < (unsigned)m)
-            lo = mid + 1;
-        else
-            hi = mid;
-    }
-    offsets[m] = (int)lo;
-}
-
 // The inverse index of a neighbour table without its first column, from the inverse
 // index of the whole table: the entries of column 0 leave every target's list and
 // flat slot v*K+n becomes v*(K-1)+n-1. One wave per target, its list across the lanes.
@@ -742,13 +721,6 @@ __global__ __launch_bounds__(256) void weight_grad_kernel(const float *__restric
     }
 }
 
-int inverse_key_bits(int n_vert) {
-    int bits = 1;
-    while (bits < 32 && (1ll << bits) <= (long long)n_vert) ++bits;  // keys go up to n_vert inclusive
-    return bits;
-}
-
-
 }  // namespace
 }  // namespace hgc
 
@@ -827,42 +799,6 @@ int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int 
                        int mean_and_max, hgc_stream_t stream) {
     return hgc_accumulate_knn_slots(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, nullptr, nullptr, n_vert,
                                     n_neigh, n_feat, n_out_feat, n_moments, mean_and_max, stream);
-}
-
-size_t hgc_inverse_neighbour_index_workspace_bytes(int n_vert, int n_neigh) {
-    const size_t total = std::max<size_t>((size_t)n_vert * n_neigh, 1);
-    size_t temp = 0;
-    (void)rocprim::radix_sort_pairs(nullptr, temp, rocprim::make_transform_iterator((const int *)nullptr, InverseKey{1u}),
-                                    (unsigned int *)nullptr, rocprim::counting_iterator<int>(0), (int *)nullptr, total, 0,
-                                    inverse_key_bits(std::max(n_vert, 1)), (hipStream_t) nullptr);
-    return align_up(temp) + align_up(total * sizeof(int));
-}
-
-int hgc_inverse_neighbour_index(const int *d_idxs, int n_vert, int n_neigh, int *d_inv_offsets, int *d_inv_slots,
-                                void *workspace, size_t workspace_bytes, hgc_stream_t stream) {
-    HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1, "bad sizes");
-    HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neigh overflows int32");
-    HGC_REQUIRE(d_inv_offsets, "null pointer");
-    hipStream_t s = as_stream(stream);
-    if (n_vert == 0) return launch_fill_i32(d_inv_offsets, 0, 1, s);
-    HGC_REQUIRE(d_idxs && d_inv_slots, "null pointer");
-    if (!workspace || !aligned256(workspace) ||
-        workspace_bytes < hgc_inverse_neighbour_index_workspace_bytes(n_vert, n_neigh))
-        return fail(HGC_ERR_WORKSPACE, "inverse_neighbour_index workspace missing, misaligned or too small");
-    const long long total = (long long)n_vert * n_neigh;
-    Carver carve(workspace);
-    unsigned int *keys_sorted = carve.take<unsigned int>(total);
-    void *temp = carve.base + carve.used;
-    size_t temp_bytes = workspace_bytes - carve.used;
-    // Keys and values are generated on the fly: key = the slot's target (invalid
-    // ones sort last), value = the flat slot itself. Stable: inside one target the
-    // flat slots stay ascending, i.e. (vertex, slot) order.
-    const auto keys_in = rocprim::make_transform_iterator(d_idxs, InverseKey{(unsigned)n_vert});
-    const rocprim::counting_iterator<int> slots_in(0);
-    HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, keys_sorted, slots_in, d_inv_slots, (size_t)total, 0,
-                                      inverse_key_bits(n_vert), s));
-    inverse_offsets_kernel<<<ceil_div((long long)n_vert + 1, 256), 256, 0, s>>>(keys_sorted, total, d_inv_offsets, n_vert);
-    return check_launch("inverse_offsets");
 }
 
 size_t hgc_inverse_index_without_first_column_workspace_bytes(int n_vert) {

@@ -395,6 +395,34 @@ def test_inverse_neighbour_index_is_ordered():
         assert (mine == np.nonzero(flat == m)[0]).all()
 
 
+@pytest.mark.parametrize("n,k,kind", [(1, 1, "random"), (70, 3, "random"), (4000, 64, "hubs"), (30000, 5, "random"),
+                                      (100000, 16, "banded"), (300000, 2, "random"), (5000, 300, "random"),
+                                      (1200000, 2, "banded"), (4300000, 1, "random")])
+def test_inverse_neighbour_index_shapes_and_hubs(n, k, kind):
+    """the builder against a stable argsort: tables of one column and of hundreds, a handful of
+    vertices that everybody names (their lists exceed what one workgroup stages), padding and
+    out-of-range entries, tile widths from 32 to 1024 vertices, and a table beyond the two-level
+    split (library sort)"""
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(n + k)
+    if kind == "banded":
+        idx = (np.arange(n)[:, None] + rng.integers(-500, 501, (n, k))).clip(0, n - 1).astype(np.int32)
+    else:
+        idx = rng.integers(0, n, (n, k)).astype(np.int32)
+    if kind == "hubs":
+        idx[rng.random((n, k)) < 0.5] = 7            # ~128,000 slots name vertex 7
+        idx[:, 3] = n - 1
+    idx[rng.random((n, k)) < 0.05] = -1
+    idx[rng.random((n, k)) < 0.01] = n + 3
+    off, slots = ops.inverse_neighbour_index(t(idx))
+    off, slots = off.cpu().numpy(), slots.cpu().numpy()
+    flat = idx.reshape(-1).astype(np.int64)
+    key = np.where((flat >= 0) & (flat < n), flat, n)
+    order = np.argsort(key, kind="stable")
+    assert (slots[:len(flat)] == order).all()
+    assert (off == np.searchsorted(key[order], np.arange(n + 1))).all()
+
+
 def test_accumulate_autograd_chain(oracle):
     from hgcalml_amd import AccumulateKnn
     rng = np.random.default_rng(22)
