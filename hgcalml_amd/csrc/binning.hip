@@ -193,6 +193,70 @@ __global__ __launch_bounds__(256) void bin_points_kernel(
     if (calc_n_per_bin) atomicAdd(&n_per_bin[cell], 1);
 }
 
+// The same assignment fused with the condensate wrapper's shift to the column minima: every
+// block derives the grid from the column ranges itself (pre-normalised coordinates: shift 0,
+// extent = largest shifted value = max - min, rounding is monotonic).
+__device__ __forceinline__ float from_ordered_pattern(uint32_t u) {
+    return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
+}
+
+__global__ __launch_bounds__(256) void shift_and_bin_kernel(
+    const float *__restrict__ coords, const uint32_t *__restrict__ min_bits, const uint32_t *__restrict__ max_bits_inv,
+    const int *__restrict__ row_splits, int n_vert, int n_coords, int n_dims, int n_rs, int n_bins_scalar,
+    int n_total_bins, float *__restrict__ shifted, float *__restrict__ bin_width_out, int *__restrict__ n_bins_out,
+    int *__restrict__ binass, int *__restrict__ flat, int *__restrict__ status) {
+    __shared__ float s_min[16], s_bw;
+    __shared__ int s_nb[kMaxBinDims];
+    if (threadIdx.x < n_coords) s_min[threadIdx.x] = from_ordered_pattern(min_bits[threadIdx.x]);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float lo[kMaxBinDims], hi[kMaxBinDims], unused_shift[kMaxBinDims];
+        for (int c = 0; c < n_dims; ++c) {
+            lo[c] = s_min[c] - s_min[c];
+            hi[c] = from_ordered_pattern(~max_bits_inv[c]) - s_min[c];
+        }
+        derive_grid(lo, hi, n_dims, 1, n_bins_scalar, nullptr, unused_shift, &s_bw, s_nb);
+        if (blockIdx.x == 0) {
+            for (int c = 0; c < n_dims; ++c) n_bins_out[c] = s_nb[c];
+            bin_width_out[0] = s_bw;
+        }
+    }
+    __syncthreads();
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_vert) return;
+    const float bw = s_bw;
+    int mul = 1, cell = 0, flags = 0;
+    for (int c = n_coords - 1; c >= 0; --c) {
+        const float x = coords[(size_t)p * n_coords + c] - s_min[c];
+        shifted[(size_t)p * n_coords + c] = x;
+        if (c >= n_dims) continue;
+        if (!isfinite(x)) flags |= HGC_FLAG_COORDINATE_NOT_FINITE;
+        int k = (int)(x / bw);
+        const int nb = s_nb[c];
+        if (k < 0 || k >= nb) {
+            k = 0;
+            flags |= HGC_FLAG_COORDINATE_OUT_OF_GRID;
+        }
+        binass[(size_t)p * (n_dims + 1) + c + 1] = k;
+        cell += k * mul;
+        mul *= nb;
+    }
+    int lo = 1, hi = n_rs;  // event: number of row splits (from the second on) that are <= p
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (row_splits[mid] > p)
+            hi = mid;
+        else
+            lo = mid + 1;
+    }
+    const int ev = lo - 1;
+    cell += ev * mul;
+    if (flags && status) atomicOr(status, flags);
+    if (cell >= n_total_bins) return;
+    binass[(size_t)p * (n_dims + 1)] = ev;
+    flat[p] = cell;
+}
+
 // ---- boundaries from the sorted keys -----------------------------------------
 
 __global__ __launch_bounds__(256) void bin_boundaries_kernel(const int *__restrict__ sorted_bins, int n_vert,
@@ -350,6 +414,21 @@ int key_bits(int n_total_bins) {
 }
 
 }  // namespace
+
+int shift_and_bin(const float *d_coords, const uint32_t *d_min_bits, const uint32_t *d_max_bits_inverted,
+                  const int *d_row_splits, int n_vert, int n_coords, int n_bin_dims, int n_rs, int n_bins_scalar,
+                  int n_total_bins, float *d_shifted, float *d_bin_width, int *d_n_bins, int *d_assigned_bin,
+                  int *d_flat_bin, hipStream_t s) {
+    HGC_REQUIRE(n_coords >= 1 && n_coords <= 16 && n_bin_dims >= 1 && n_bin_dims <= kMaxBinDims &&
+                    n_bin_dims <= n_coords,
+                "bad coordinate or binning dimensions");
+    if (n_vert <= 0) return HGC_OK;
+    shift_and_bin_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, d_min_bits, d_max_bits_inverted, d_row_splits,
+                                                               n_vert, n_coords, n_bin_dims, n_rs, n_bins_scalar,
+                                                               n_total_bins, d_shifted, d_bin_width, d_n_bins,
+                                                               d_assigned_bin, d_flat_bin, status_word());
+    return check_launch("shift_and_bin");
+}
 
 int launch_fill_i32(int *p, int value, long long n, hipStream_t s) {
     if (n <= 0) return HGC_OK;
@@ -514,9 +593,13 @@ int hgc_bin_setup(const float *d_coords, int coord_stride, int n_vert, int n_bin
     return check_launch("grid_params");
 }
 
+static int hits_per_bin(int n_vert, int n_total_bins) { return std::max(1, n_vert / std::max(n_total_bins, 1)); }
+
 size_t hgc_sort_by_bin_workspace_bytes(int n_vert, int n_total_bins) {
     size_t temp = 0;
     const int n = std::max(n_vert, 1);
+    if (stable_key_sort_supported(n, std::max(n_total_bins, 1), hits_per_bin(n, n_total_bins)))
+        return stable_key_sort_workspace_bytes(n, std::max(n_total_bins, 1), hits_per_bin(n, n_total_bins));
     (void)rocprim::radix_sort_pairs(nullptr, temp, (const unsigned int *)nullptr, (unsigned int *)nullptr,
                                     (const int *)nullptr, (int *)nullptr, (size_t)n, 0,
                                     key_bits(std::max(n_total_bins, 2)), (hipStream_t) nullptr);
@@ -533,6 +616,10 @@ int hgc_sort_by_bin(const int *d_flat_bin, int n_vert, int n_total_bins, int *d_
     if (!workspace || !aligned256(workspace) ||
         workspace_bytes < hgc_sort_by_bin_workspace_bytes(n_vert, n_total_bins))
         return fail(HGC_ERR_WORKSPACE, "sort_by_bin workspace missing, misaligned or too small");
+    // a stable counting sort by bin yields the order and the boundary table at once
+    if (stable_key_sort_supported(n_vert, n_total_bins, hits_per_bin(n_vert, n_total_bins)))
+        return stable_key_sort(d_flat_bin, nullptr, n_vert, n_total_bins, hits_per_bin(n_vert, n_total_bins),
+                               d_bin_boundaries, d_sorting, workspace, workspace_bytes, s);
     Carver carve(workspace);
     int *iota = carve.take<int>(n_vert);
     unsigned int *keys_out = carve.take<unsigned int>(n_vert);

@@ -84,6 +84,28 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
                  int *d_n_bins, int *d_boundaries, int *d_sorting, float *d_scoords, int *d_sflat, int *d_sbinass,
                  int *d_sdir, void *workspace, size_t workspace_bytes, hipStream_t s);
 
+int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
+
+// The front end of the condensate wrapper (modules/assign_condensate_op.py:269-274) in one pass:
+// d_shifted = d_coords minus the column minima (all n_coords columns), the grid of n_bins_scalar
+// bins over the first n_bin_dims shifted columns (what BinByCoordinates derives with
+// pre_normalized=True), and the bin of every hit. d_min_bits / d_max_bits_inverted [n_coords]:
+// column minima as order-preserving bit patterns, maxima as the complement of theirs.
+int shift_and_bin(const float *d_coords, const uint32_t *d_min_bits, const uint32_t *d_max_bits_inverted,
+                  const int *d_row_splits, int n_vert, int n_coords, int n_bin_dims, int n_rs, int n_bins_scalar,
+                  int n_total_bins, float *d_shifted, float *d_bin_width, int *d_n_bins, int *d_assigned_bin,
+                  int *d_flat_bin, hipStream_t s);
+
+// Stable sort of `total` items by integer key (split_sort.hip). Item i has the key
+// d_keys[d_values ? d_values[i] : i] and the value d_values ? d_values[i] : i; keys outside
+// [0, n_keys) count as n_keys and sort last. d_order [total] receives the values in key order,
+// d_offsets (may be null) [n_keys + 1] the first position of every key. `per_key_hint`: items
+// expected per key (sizes the tiles). Not every shape is supported (key ranges of 2^22 and more).
+bool stable_key_sort_supported(long long total, int n_keys, int per_key_hint);
+size_t stable_key_sort_workspace_bytes(long long total, int n_keys, int per_key_hint);
+int stable_key_sort(const int *d_keys, const int *d_values, long long total, int n_keys, int per_key_hint,
+                    int *d_offsets, int *d_order, void *workspace, size_t workspace_bytes, hipStream_t s);
+
 // hgc_binned_select_knn_fused over a boundary table with stride 2^boundary_shift
 int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const int *d_direction,
                               const int *d_dim_bin_idx, const int *d_bin_boundaries, int boundary_shift,

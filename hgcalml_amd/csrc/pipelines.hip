@@ -92,41 +92,46 @@ __device__ __forceinline__ float from_ordered_bits(uint32_t u) {
     return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
 }
 
-// column minima (NaN ignored) as order-preserving bit patterns, combined with atomicMin
-__global__ __launch_bounds__(256) void column_min_kernel(const float *__restrict__ x, int n, int C,
-                                                         uint32_t *__restrict__ mins) {
-    __shared__ uint32_t s_min[kMaxCoordDims];
-    if (threadIdx.x < kMaxCoordDims) s_min[threadIdx.x] = 0xffffffffu;
+// Column minima and maxima (NaN ignored) as order-preserving bit patterns, combined with
+// atomicMin: range[c] = pattern of the minimum, range[kMaxCoordDims + c] = complement of the
+// pattern of the maximum. Both start at 0xffffffff.
+__global__ __launch_bounds__(256) void column_range_kernel(const float *__restrict__ x, int n, int C,
+                                                           uint32_t *__restrict__ range) {
+    __shared__ uint32_t s_range[2 * kMaxCoordDims];
+    if (threadIdx.x < 2 * kMaxCoordDims) s_range[threadIdx.x] = 0xffffffffu;
     __syncthreads();
-    uint32_t lo[kMaxCoordDims];
+    uint32_t lo[kMaxCoordDims], hi[kMaxCoordDims];
 #pragma unroll
-    for (int c = 0; c < kMaxCoordDims; ++c) lo[c] = 0xffffffffu;
+    for (int c = 0; c < kMaxCoordDims; ++c) lo[c] = hi[c] = 0xffffffffu;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x)
 #pragma unroll
         for (int c = 0; c < kMaxCoordDims; ++c)
             if (c < C) {
                 const float v = x[(size_t)i * C + c];
-                if (v == v) lo[c] = min(lo[c], ordered_bits(v));
+                if (v == v) {
+                    lo[c] = min(lo[c], ordered_bits(v));
+                    hi[c] = min(hi[c], ~ordered_bits(v));
+                }
             }
 #pragma unroll
     for (int c = 0; c < kMaxCoordDims; ++c) {
         if (c < C) {
-            uint32_t v = lo[c];
-            for (int off = 32; off > 0; off >>= 1) v = min(v, (uint32_t)__shfl_xor((int)v, off, kWave));
-            if (lane_id() == 0) atomicMin(&s_min[c], v);
+            uint32_t a = lo[c], b = hi[c];
+            for (int off = 32; off > 0; off >>= 1) {
+                a = min(a, (uint32_t)__shfl_xor((int)a, off, kWave));
+                b = min(b, (uint32_t)__shfl_xor((int)b, off, kWave));
+            }
+            if (lane_id() == 0) {
+                atomicMin(&s_range[c], a);
+                atomicMin(&s_range[kMaxCoordDims + c], b);
+            }
         }
     }
     __syncthreads();
-    if (threadIdx.x < C) atomicMin(&mins[threadIdx.x], s_min[threadIdx.x]);
-}
-
-// coordinates minus their column minimum: the wrapper's ccoords - min(ccoords)
-__global__ __launch_bounds__(256) void shift_to_minimum_kernel(const float *__restrict__ x, long long n_values, int C,
-                                                               const uint32_t *__restrict__ mins,
-                                                               float *__restrict__ out) {
-    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n_values) return;
-    out[e] = x[e] - from_ordered_bits(mins[e % C]);
+    if (threadIdx.x < C) {
+        atomicMin(&range[threadIdx.x], s_range[threadIdx.x]);
+        atomicMin(&range[kMaxCoordDims + threadIdx.x], s_range[kMaxCoordDims + threadIdx.x]);
+    }
 }
 
 // inputs moved into bin order, local radii scaled, the high-beta subset marked
@@ -238,7 +243,7 @@ bool cond_layout(int n_vert, int n_coords, int num_rows, int n_bins_scalar, int 
         off += align_up(bytes);
         return at;
     };
-    L.mins = take(kMaxCoordDims * sizeof(uint32_t));
+    L.mins = take(2 * kMaxCoordDims * sizeof(uint32_t));
     L.shifted = take(n * n_coords * sizeof(float));
     L.shift = take(8 * sizeof(float));
     L.bin_width = take(sizeof(float));
@@ -313,21 +318,14 @@ int hgc_build_and_assign_condensates(const float *d_ccoords, const float *d_beta
     const int B = L.n_bin_dims;
     int rc;
 
-    if ((rc = launch_fill_i32(reinterpret_cast<int *>(mins), -1, kMaxCoordDims, s))) return rc;
-    column_min_kernel<<<std::max(1, std::min(512, ceil_div(n_vert, 1024))), 256, 0, s>>>(d_ccoords, n_vert, n_coords,
-                                                                                          mins);
-    if ((rc = check_launch("column_min"))) return rc;
-    const long long n_values = (long long)n_vert * n_coords;
-    shift_to_minimum_kernel<<<ceil_div(n_values, 256), 256, 0, s>>>(d_ccoords, n_values, n_coords, mins,
-                                                                    F(L.shifted));
-    if ((rc = check_launch("shift_to_minimum"))) return rc;
-    // grid over the already shifted coordinates, hits into stable bin order
-    if ((rc = hgc_bin_setup(F(L.shifted), n_coords, n_vert, B, 1, n_bins_scalar, nullptr, F(L.shift), F(L.bin_width),
-                            I(L.n_bins), ws + L.setup_ws, L.setup_bytes, stream)))
-        return rc;
-    if ((rc = hgc_bin_by_coordinates_strided(F(L.shifted), n_coords, nullptr, d_row_splits, F(L.bin_width),
-                                             I(L.n_bins), I(L.binass), I(L.flat), nullptr, nullptr, n_vert, B,
-                                             num_rows + 1, L.cells_bound, 0, stream)))
+    if ((rc = launch_fill_i32(reinterpret_cast<int *>(mins), -1, 2 * kMaxCoordDims, s))) return rc;
+    column_range_kernel<<<std::max(1, std::min(512, ceil_div(n_vert, 1024))), 256, 0, s>>>(d_ccoords, n_vert,
+                                                                                            n_coords, mins);
+    if ((rc = check_launch("column_range"))) return rc;
+    // coordinates shifted to their minimum, grid over the shifted coordinates, bin of every hit
+    if ((rc = shift_and_bin(d_ccoords, mins, mins + kMaxCoordDims, d_row_splits, n_vert, n_coords, B, num_rows + 1,
+                            n_bins_scalar, L.cells_bound, F(L.shifted), F(L.bin_width), I(L.n_bins), I(L.binass),
+                            I(L.flat), s)))
         return rc;
     if ((rc = hgc_sort_by_bin(I(L.flat), n_vert, L.cells_bound, I(L.sorting), I(L.bin_splits), ws + L.sort_ws,
                               L.sort_bytes, stream)))
