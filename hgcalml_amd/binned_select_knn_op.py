@@ -77,8 +77,11 @@ def BinnedSelectKnn(K, coords, row_splits, direction=None, n_bins=None, max_bin_
     max_bin_dims = min(max_bin_dims, n_coords)
 
     if n_bins is None:
-        first = int(rs_host[1]) if rs_host is not None else int(rs_dev[1])
-        n_bins = default_n_bins(first, K, max_bin_dims)
+        if gl.knn_callers_grid:
+            first = int(rs_host[1]) if rs_host is not None else int(rs_dev[1])
+            n_bins = default_n_bins(first, K, max_bin_dims)
+        else:
+            n_bins = 30  # the library searches on a grid of its own: no read of the first event's size
     n_bins = int(n_bins)
     if n == 0:
         return (torch.empty((0, K), dtype=torch.int32, device=dev),

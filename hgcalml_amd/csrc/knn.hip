@@ -569,6 +569,7 @@ int launch_coords(const KnnParams &p, hipStream_t s) {
     if (p.n_coords == 2 && p.n_bin_dim == 2) return launch_levels<2, 2, MAPPED>(p, s);
     if (p.n_coords == 3 && p.n_bin_dim == 3) return launch_levels<3, 3, MAPPED>(p, s);
     if (p.n_coords == 4 && p.n_bin_dim == 3) return launch_levels<4, 3, MAPPED>(p, s);
+    if (p.n_coords == 4 && p.n_bin_dim == 4) return launch_levels<4, 4, MAPPED>(p, s);
     if (p.n_coords == 5 && p.n_bin_dim == 3) return launch_levels<5, 3, MAPPED>(p, s);
     if (p.n_coords == 6 && p.n_bin_dim == 3) return launch_levels<6, 3, MAPPED>(p, s);
     if (p.n_coords == 7 && p.n_bin_dim == 3) return launch_levels<7, 3, MAPPED>(p, s);

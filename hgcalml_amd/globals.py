@@ -12,7 +12,14 @@ device status word after each call, raise on non finite coordinates
 (modules/bin_by_coordinates_op.py:46) and on the condensate count relation
 (modules/assign_condensate_op.py:334-343), and warn where the reference prints
 and continues (a coordinate outside the grid, a bin beyond the boundary table,
-an index beyond the replacement table)."""
+an index beyond the replacement table).
+
+`knn_callers_grid` has no counterpart either. BinnedSelectKnn normally lets the
+library choose the grid it searches on (the neighbour sets of the exact search do
+not depend on it, the run time does); when set, the search bins exactly as the
+reference would: `n_bins` (or its default formula, which reads the first event's
+size) over `max_bin_dims` dimensions."""
 knn_ops_use_tf_gradients = False
 acc_ops_use_tf_gradients = False
 debug_checks = False
+knn_callers_grid = False

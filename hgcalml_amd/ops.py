@@ -200,6 +200,7 @@ def binned_select_knn_pipeline(coords, row_splits, direction, n_neighbours, n_bi
     nbytes = lib.hgc_binned_select_knn_pipeline_workspace_bytes(n, c, row_splits.numel(), int(n_bins), int(max_bin_dims),
                                                                 int(direction is not None))
     ws = workspace(nbytes, dev)
+    check(lib.hgc_set_knn_grid(int(gl.knn_callers_grid)))
     with data_checks("BinnedSelectKnn", dev):
         check(lib.hgc_binned_select_knn_pipeline(p(coords), p(row_splits), p(direction), n, c, row_splits.numel(),
                                                  int(n_neighbours), int(n_bins), int(max_bin_dims),

@@ -187,16 +187,24 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
                                 hgc_stream_t stream);
 
 /* The whole wrapper modules/binned_select_knn_op.py:33-104 in one call:
- * bounding box and grid (n_bins_scalar bins along the widest of the first
- * min(max_bin_dims, n_coords) coordinates), bin assignment, stable sort into bin
- * order, gather of the sorted inputs, search and un-sort. Inputs and outputs are
+ * bounding box and grid, bin assignment, grouping by bin with the inputs moved
+ * along, search and un-sort. Inputs and outputs are
  * in the caller's order and index space: d_coords [n_vert, n_coords],
  * d_row_splits [n_rs], d_direction [n_vert] or NULL; d_indices, d_dist
  * [n_vert, n_neigh]. d_out_sorting (may be NULL) [n_vert] receives the bin
  * order of the points (original index of the i-th point in bin order; the
  * order inside a bin is unspecified and can differ from run to run, the
  * neighbour results do not depend on it), a useful d_vertex_order for the
- * accumulation. No host synchronisation. */
+ * accumulation. No host synchronisation.
+ *
+ * The neighbour sets of an exact search do not depend on the grid it walks, so
+ * by default the pipeline searches on a grid of its own choice (up to four
+ * binned dimensions, about one point per cell) and takes n_bins_scalar and
+ * max_bin_dims only for the reference's argument checks; hgc_set_knn_grid(1)
+ * makes the calling thread's later calls bin exactly as asked
+ * (n_bins_scalar bins over min(max_bin_dims, n_coords) dimensions),
+ * hgc_set_knn_grid(0) returns to the default. The workspace query covers both. */
+int hgc_set_knn_grid(int use_callers_grid);
 size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, int n_rs,
                                                       int n_bins_scalar, int max_bin_dims,
                                                       int use_direction);

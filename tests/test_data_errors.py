@@ -116,10 +116,18 @@ def test_non_finite_coordinates_are_refused_on_the_pipelines(debug_checks):
         with pytest.raises(ValueError, match="NaN or Inf"):
             BuildAndAssignCondensatesBinned(torch.from_numpy(y).to(DEV), torch.rand(500, 1, device=DEV),
                                             torch.full((500, 1), 0.1, device=DEV), rs.to(DEV), 0.1)
-    # the fourth coordinate is not binned: the reference's check never sees it either
+    # binning as the reference does leaves the fourth coordinate out, and so does its check;
+    # the library's own grid bins (and checks) it too
+    from hgcalml_amd import globals as gl
     y = x.copy()
     y[7, 3] = np.inf
-    BinnedSelectKnn(8, torch.from_numpy(y).to(DEV), rs, n_bins=5)
+    gl.knn_callers_grid = True
+    try:
+        BinnedSelectKnn(8, torch.from_numpy(y).to(DEV), rs, n_bins=5)
+    finally:
+        gl.knn_callers_grid = False
+    with pytest.raises(ValueError, match="NaN or Inf"):
+        BinnedSelectKnn(8, torch.from_numpy(y).to(DEV), rs, n_bins=5)
     # clean data passes, including the condensate count relation
     BuildAndAssignCondensatesBinned(torch.from_numpy(x).to(DEV), torch.rand(500, 1, device=DEV),
                                     torch.full((500, 1), 0.1, device=DEV), rs.to(DEV), 0.1, keep_noise=True)
@@ -171,9 +179,17 @@ def test_replacement_out_of_range_is_flagged_and_left_alone(debug_checks):
 def test_too_fine_grid_is_refused_or_flagged():
     """5 binned dimensions, 40 bins each: a shell of the walk would have (2*41+1)^4 > 2^24 rows"""
     from hgcalml_amd import BinnedSelectKnn
+    from hgcalml_amd import globals as gl
     x = torch.rand((200, 5), device=DEV)
     rs = torch.tensor([0, 200], dtype=torch.int32)
-    with pytest.raises(ValueError, match="too fine"):
-        BinnedSelectKnn(4, x, rs, n_bins=40, max_bin_dims=5)
-    idx, _ = BinnedSelectKnn(4, x, rs, n_bins=20, max_bin_dims=5)
+    gl.knn_callers_grid = True          # bin exactly as asked
+    try:
+        with pytest.raises(ValueError, match="too fine"):
+            BinnedSelectKnn(4, x, rs, n_bins=40, max_bin_dims=5)
+        idx, _ = BinnedSelectKnn(4, x, rs, n_bins=20, max_bin_dims=5)
+    finally:
+        gl.knn_callers_grid = False
     assert (idx[:, 0].cpu() == torch.arange(200)).all() and (idx >= 0).all()
+    # on the library's own grid the same request is simply answered
+    idx2, _ = BinnedSelectKnn(4, x, rs, n_bins=40, max_bin_dims=5)
+    assert torch.equal(idx, idx2)

@@ -269,6 +269,40 @@ def test_knn_functor_level_entry_point(oracle):
     assert compare_knn(oracle, got_i, got_d, ref_i, ref_d, coords[order], rs, 20) == 0
 
 
+@pytest.mark.parametrize("C,K,n_events", [(2, 9, 1), (3, 16, 3), (4, 64, 1), (4, 20, 4), (5, 12, 2), (4, 130, 1),
+                                          (6, 33, 1)])
+def test_knn_result_does_not_depend_on_the_grid(oracle, C, K, n_events):
+    """the library's own search grid (up to four binned dimensions, about one point per cell) against
+    the caller's (the reference wrapper's n_bins over min(3, C) dimensions): same indices and distance
+    bits, with direction flags, a radius, tf_compatible padding, and an event with fewer than K points;
+    one of them is also checked against the oracle"""
+    from hgcalml_amd import BinnedSelectKnn
+    from hgcalml_amd import globals as gl
+    rng = np.random.default_rng(300 + C + K)
+    n = 9000
+    x = np.concatenate([workloads.cluster_mixture(rng, n - 40, 4)[:, :min(C, 4)],
+                        rng.random((40, min(C, 4))).astype(np.float32)])
+    if C > 4:
+        x = np.concatenate([x, rng.standard_normal((n, C - 4)).astype(np.float32) * 0.1], axis=1)
+    x = np.ascontiguousarray(x[:, :C])
+    cuts = np.sort(rng.choice(np.arange(1, n - 41), n_events - 1, replace=False)) if n_events > 1 else []
+    rs = np.array([0, *cuts, n - 40, n], np.int32)            # the last event has 40 points
+    direction = rng.integers(0, 5, n).astype(np.int32)
+    for kwargs in (dict(), dict(direction=direction), dict(max_radius=0.15, tf_compatible=True)):
+        tk = {k: (t(v) if k == "direction" else v) for k, v in kwargs.items()}
+        got = {}
+        for callers in (False, True):
+            gl.knn_callers_grid = callers
+            try:
+                got[callers] = BinnedSelectKnn(K, t(x), t(rs), n_bins=11, **tk)
+            finally:
+                gl.knn_callers_grid = False
+        assert torch.equal(got[False][0], got[True][0])
+        assert torch.equal(got[False][1].view(torch.int32), got[True][1].view(torch.int32))
+    ri, rd = oracle.BinnedSelectKnn(K, x, rs, n_bins=11, max_radius=0.15, tf_compatible=True)
+    assert compare_knn(oracle, got[False][0], got[False][1], ri, rd, x, rs, K, tf_compatible=True, radius=0.15) == 0
+
+
 # ------------------------------------------------------------------ accumulate
 
 def make_acc_case(rng, n, K, F, holes=True):
@@ -905,7 +939,12 @@ def test_knn_pipeline_bin_order_groups_points_by_bin(oracle, case):
         coords = rng.random((4000, 3), dtype=np.float32)
         rs = np.array([0, 900, 900, 2500, 4000], np.int32)
         n_bins = 6
-    idx, _ = run_knn_case(oracle, coords, rs, 8, n_bins, max_ties=len(coords))
+    from hgcalml_amd import globals as gl
+    gl.knn_callers_grid = True      # the grid of the reference wrapper, which the oracle bins on too
+    try:
+        idx, _ = run_knn_case(oracle, coords, rs, 8, n_bins, max_ties=len(coords))
+    finally:
+        gl.knn_callers_grid = False
     order = ops.vertex_order_of(idx).cpu().numpy()
     assert sorted(order.tolist()) == list(range(len(coords)))
     _, flat, _, _ = oracle.BinByCoordinates(coords[:, :3], rs, n_bins=n_bins, calc_n_per_bin=False)
