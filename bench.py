@@ -19,8 +19,8 @@ The `roofline` object is measured in a second timed loop of the same run (also
 K iterations, HIP events on the stream the kernels are launched on) at cfg4
 (N=1,000,000, K=64, F=128, banded neighbour table): the dominant kernel, one
 launch of the accumulate_knn gradient (algorithmic bytes 4*N*(3K+5F)), with
-the forward launch (4*N*(2K+4F)) and the forward+gradient pair next to it,
-against the 8 TB/s HBM peak.
+the forward launch (4*N*(2K+4F)), the forward+gradient pair and the pair plus
+one build of the inverse neighbour index next to it, against the 8 TB/s HBM peak.
 
 `cpu_baseline` times the CPU oracle (a single-threaded C restatement of the
 reference CPU kernels) on this box's host: the binned kNN kernel over the full
@@ -42,13 +42,26 @@ sys.path.insert(1, os.path.join(ROOT, "tests"))  # workloads.py: the seeded inpu
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch at full cfg4, from two hardware-counter runs of this
-# file's roofline section (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, both scaled
-# by what the counters read for the 512 MB calibration copy below); summary in
-# profiles/accumulate_knn_cfg4_hbm_counters.txt. Counters cannot be read from
-# inside the timed run, so these are the last profiled values.
-CFG4_FWD_MEASURED_HBM_BYTES = 3.22e9
-CFG4_GRAD_MEASURED_HBM_BYTES = 19.4e9
+# HBM bytes per launch at full cfg4 come from two hardware-counter runs of this file's
+# roofline section (FETCH_SIZE, WRITE_SIZE, scaled by what the counters read for the 512 MB
+# calibration copy below). Counters cannot be read from inside the timed run, so the line
+# carries what the committed summary profiles/accumulate_knn_cfg4_hbm_counters.txt holds
+# (its "bench.py reads" line, stamped with the commit it was measured at), or null.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "accumulate_knn_cfg4_hbm_counters.txt")
+
+
+def measured_traffic():
+    """{'forward': bytes, 'gradient': bytes, 'measured_at': commit} from the committed summary, or None"""
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            for line in f:
+                if line.startswith("bench.py reads:"):
+                    fields = dict(kv.split("=", 1) for kv in line.split(":", 1)[1].split())
+                    return {"forward": float(fields["forward_bytes"]), "gradient": float(fields["gradient_bytes"]),
+                            "measured_at": fields.get("measured_at", "unknown")}
+    except (OSError, KeyError, ValueError):
+        pass
+    return None
 
 
 def log(*a):
@@ -118,8 +131,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--roofline-scale", type=float, default=1.0, help="shrink cfg4 (debugging only)")
-    ap.add_argument("--section", choices=["all", "headline", "roofline"], default="all",
-                    help="run only one part (for profiling); the JSON line is printed for 'all' only")
+    ap.add_argument("--section", choices=["all", "headline", "roofline", "streams"], default="all",
+                    help="run only one part (for profiling); the JSON line is printed for 'all' only. 'streams': the "
+                         "cfg4 gradient next to its variants without the max half and without the weight gradient, "
+                         "whose counter differences split its L2 requests by data stream")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets ONE GPU (no collectives, no sharding); run with --gpus 1. "
@@ -136,7 +151,7 @@ def main():
     # ------------------------------------------------------------------ headline: cfg2
     c2 = workloads.cfg2()
     n2, K2 = len(c2["coords"]), c2["K"]
-    if args.section != "roofline":
+    if args.section not in ("roofline", "streams"):
         coords = torch.from_numpy(c2["coords"]).to(dev)
         rs = torch.from_numpy(c2["row_splits"]).to(dev)
         feat = torch.from_numpy(c2["features"]).to(dev)
@@ -229,6 +244,16 @@ def main():
     log("bench: cfg4 fwd %.3f ms, grad %.3f ms, inverse index (one-off) %.3f ms -> %.1f GB/s" %
         (fwd_ms[0], grad_ms[0], inv_ms[0], achieved))
 
+    if args.section == "streams":
+        # same table, same inputs: the gradient without the max half (no slot bytes, no max-half loads), and the
+        # ordered gather alone (push_knn: mean-half rows, weights and inverse slots; no own feature row, no
+        # weight-gradient writes)
+        g4_mean = g4[:, :F4].contiguous()
+        for _ in range(max(2, args.steps)):
+            torch.ops.hgcalml.accumulate_knn_grad_slots(g4_mean, w4, x4, i4, arg4, slots4, *inv)
+            torch.ops.hgcalml.push_knn(w4, g4_mean, i4)
+        torch.cuda.synchronize()
+        return
     if args.section == "roofline":
         return
     # ------------------------------------------------------------------ information: cfg3, cfg5
@@ -239,6 +264,10 @@ def main():
         m3 = event_ms(lambda: BinnedSelectKnn(c3["K"], co3, rs3, n_bins=c3["n_bins"], max_radius=c3["max_radius"]), 5, 2)
         extra["cfg3_knn_ms"] = round(m3[0], 3)
         extra["cfg3_queries_per_s"] = round(len(c3["coords"]) / (m3[0] * 1e-3), 1)
+        # a 4-D Gaussian blob (the shape of a learned coordinate space): N=150k, K=65
+        blob = torch.from_numpy(np.random.default_rng(5).standard_normal((150000, 4)).astype(np.float32)).to(dev)
+        mb = event_ms(lambda: BinnedSelectKnn(65, blob, rs, n_bins=30), 5, 2)
+        extra["knn_gaussian_blob_4d_N150k_K65_ms"] = round(mb[0], 3)
         c5 = workloads.cfg5(ragged=True)
         a5 = [torch.from_numpy(c5[k]).to(dev) for k in ("ccoords", "betas", "dist", "row_splits")]
         for mode in (True, False):
@@ -298,6 +327,8 @@ def main():
                "host_cpus": os.cpu_count(), "cpu_model": cpu_model()}
         log("bench: CPU oracle kNN %.0f queries/s (%.1f s)" % (qps, secs))
 
+    traffic = measured_traffic() if args.roofline_scale == 1.0 else None
+    with_build = (bytes_fwd + bytes_bwd) / ((fwd_ms[0] + grad_ms[0] + inv_ms[0]) * 1e-3) / 1e9
     line = {
         "metric": "kNN queries/s at N=150k,4D,K=64; accumulate_knn fwd+grad achieved HBM GB/s",
         "value": round(value, 1),
@@ -322,17 +353,22 @@ def main():
                                "(N=%d, K=%d, F=%d), one launch" % (n4, K4, F4),
                      "achieved": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "traffic": CFG4_GRAD_MEASURED_HBM_BYTES if args.roofline_scale == 1.0 else None,
+                     "traffic": traffic["gradient"] if traffic else None,
+                     "traffic_measured_at": traffic["measured_at"] if traffic else None,
                      "algorithmic_bytes": bytes_bwd, "launch_ms": round(grad_ms[0], 4),
                      "forward": {"kernel": "accumulate_fwd_wave_kernel, same workload, one launch",
                                  "achieved": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9, 1),
                                  "frac": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                                 "traffic": CFG4_FWD_MEASURED_HBM_BYTES if args.roofline_scale == 1.0 else None,
+                                 "traffic": traffic["forward"] if traffic else None,
                                  "algorithmic_bytes": bytes_fwd, "launch_ms": round(fwd_ms[0], 4)},
                      "forward_plus_gradient": {"achieved": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBS, 4),
                                                "algorithmic_bytes": bytes_fwd + bytes_bwd,
-                                               "traffic": (CFG4_FWD_MEASURED_HBM_BYTES + CFG4_GRAD_MEASURED_HBM_BYTES)
-                                               if args.roofline_scale == 1.0 else None},
+                                               "traffic": traffic["forward"] + traffic["gradient"] if traffic else None},
+                     # the inverse neighbour index is rebuilt once per neighbour table, i.e. once per layer and
+                     # training step: the pair with one build next to it
+                     "forward_plus_gradient_with_index_build": {
+                         "achieved": round(with_build, 1), "frac": round(with_build / HBM_PEAK_GBS, 4),
+                         "ms": round(fwd_ms[0] + grad_ms[0] + inv_ms[0], 4)},
                      "inverse_index_build_ms": round(inv_ms[0], 3)},
         "cpu_baseline": cpu,
         "extra": extra,
