@@ -343,7 +343,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "cfg2: one event, N=150000 hits, 4-D clusters+noise, BinnedSelectKnn K=64 "
-                               "(3 binned dims, n_bins=30) + AccumulateKnn(10 d^2) forward F=64",
+                               "(called with n_bins=30; the search runs on the library's own grid) + "
+                               "AccumulateKnn(10 d^2) forward F=64",
                    "launch": launch_mode, "eager_ms_per_step": round(eager_ms_per_step, 4),
                    "knn_op_ms": round(knn_ms[0], 4), "accumulate_fwd_ms": round(acc2_ms[0], 4)},
         "accumulate_fwd_grad_GBps": round(achieved, 1),
