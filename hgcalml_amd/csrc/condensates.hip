@@ -57,7 +57,7 @@ constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kFill = 4;         // windows of the sorted list looked at per refill of the queue
 constexpr int kQueueCap = kBlock + kFill * kBlock;
 constexpr int kScanBlock = 256;  // threads of the grid-wide kernels
-constexpr int kTile = 128;       // condensation points staged in LDS at a time there
+constexpr int kTile = 256;       // condensation points staged in LDS at a time there (one per thread)
 constexpr int kMaxLaunches = 4;  // launches of the event kernel
 
 struct CondParams {
@@ -553,6 +553,9 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
 //           launch of the event kernel added; closes what they cover
 //   MODE 1: items = all hits, all points; first point that covers the hit (max-beta)
 //   MODE 2: items = all hits, all points; the reference's running comparison (min-distance)
+// The hits come in bin order, so the 256 of a workgroup share a narrow range of bins in the
+// leading binned dimensions: only the points whose box of bins meets that range go into the
+// tile (a point outside it covers none of these hits, whatever its sphere), in their order.
 template <int CMAX, int MODE>
 __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams p, int launch) {
     constexpr int aw = alpha_words(CMAX), cw = cand_words(CMAX);
@@ -562,7 +565,11 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
     __shared__ __align__(16) float s_centre[CMAX][kTile];
     __shared__ __align__(16) float s_rsq[kTile];
     __shared__ __align__(16) uint32_t s_self[kTile];
+    __shared__ int s_rank[kTile];                // rank of a tile entry among the event's points
+    __shared__ int s_kept[kTile / kWave];        // entries each wave adds to the tile
+    __shared__ int s_bin_lo[kMaxBinDims], s_bin_hi[kMaxBinDims];
     const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid >> 6;
     const int C = p.C, B = p.B;
     const int n_items = MODE == 0 ? p.n_vert_h : p.n_vert;
     const int *splits = MODE == 0 ? p.row_splits_h : p.row_splits;
@@ -571,7 +578,10 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
     const bool valid = i < n_items;
     const int ev_lo = event_of(splits, p.num_rows, i_first);
     const int ev_hi = event_of(splits, p.num_rows, min(i_first + kScanBlock, n_items) - 1);
-    const int my_ev = valid ? event_of(splits, p.num_rows, i) : -1;
+    // the workgroup's items span few events: uniform loads instead of a search per thread
+    int my_ev = valid ? ev_lo : -1;
+    for (int ev = ev_lo + 1; ev <= ev_hi; ++ev)
+        if (valid && splits[ev] <= i) my_ev = ev;
 
     // ---- this thread's item ----
     float x[CMAX];
@@ -596,9 +606,14 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
     } else if (valid) {
         Grid g;
         g.load(p);
+        if (CMAX == 4 && C == 4 && p.rows_aligned) {
+            const float4 v = reinterpret_cast<const float4 *>(p.ccoords)[i];
+            x[0] = v.x, x[1] = v.y, x[2] = v.z, x[3] = v.w;
+        } else {
 #pragma unroll
-        for (int c = 0; c < CMAX; ++c)
-            if (c < C) x[c] = p.ccoords[(size_t)i * C + c];
+            for (int c = 0; c < CMAX; ++c)
+                if (c < C) x[c] = p.ccoords[(size_t)i * C + c];
+        }
         uncoverable = p.mask[i] != 0;
         self_q = p.to_filtered[i];
         g.split(p.hit_bin[i], B, k);
@@ -619,22 +634,103 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
         const int rank_lo = (MODE == 0 && launch > 0) ? p.n_alpha_at[(launch - 1) * p.num_rows + ev] : 0;
         const int rank_hi = p.n_alpha_at[launch * p.num_rows + ev];
         bool mine = alive && my_ev == ev;
+        // the bins of this workgroup's items of the event, per dimension
+        int bin_lo[kMaxBinDims], bin_hi[kMaxBinDims];
+#pragma unroll
+        for (int d = 0; d < kMaxBinDims; ++d) bin_lo[d] = INT_MIN, bin_hi[d] = INT_MAX;
+        if (MODE != 0 && rank_lo < rank_hi) {
+            __syncthreads();  // everyone is done with the previous event's range
+            if (tid < kMaxBinDims) s_bin_lo[tid] = INT_MAX, s_bin_hi[tid] = INT_MIN;
+            __syncthreads();
+#pragma unroll
+            for (int d = 0; d < kMaxBinDims; ++d) {
+                if (d >= B) continue;
+                int lo = mine ? k[d] : INT_MAX, hi = mine ? k[d] : INT_MIN;
+#pragma unroll
+                for (int m = 1; m < kWave; m <<= 1) {
+                    lo = min(lo, __shfl_xor(lo, m));
+                    hi = max(hi, __shfl_xor(hi, m));
+                }
+                if (lane == 0) {
+                    atomicMin(&s_bin_lo[d], lo);
+                    atomicMax(&s_bin_hi[d], hi);
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int d = 0; d < kMaxBinDims; ++d)
+                if (d < B) bin_lo[d] = s_bin_lo[d], bin_hi[d] = s_bin_hi[d];
+        }
         for (int base = rank_lo; base < rank_hi; base += kTile) {
             if (!__syncthreads_or(mine)) break;  // also: everyone is done with the previous tile
-            const int n_tile = min(kTile, rank_hi - base);
-            const uint4 *src = reinterpret_cast<const uint4 *>(p.points + (size_t)(first_h + base) * aw);
-            for (int e = tid; e < n_tile * (aw / 4); e += kScanBlock) reinterpret_cast<uint4 *>(s_tile)[e] = src[e];
-            __syncthreads();
+            int n_tile;
             bool solitary_here = false;
-            if (tid < kTile) {
-                const uint32_t *a = s_tile + (size_t)tid * aw;
-                const bool real = tid < n_tile;
-                const uint32_t solq = real ? a[CMAX + 1] : 0u;
-                solitary_here = solq >> 31;
+            if (MODE == 0) {
+                // the candidates come in selection order, their bins are anywhere: every point goes in
+                n_tile = min(kTile, rank_hi - base);
+                const uint4 *src = reinterpret_cast<const uint4 *>(p.points + (size_t)(first_h + base) * aw);
+                for (int e = tid; e < n_tile * (aw / 4); e += kScanBlock) reinterpret_cast<uint4 *>(s_tile)[e] = src[e];
+                __syncthreads();
+                if (tid < kTile) {
+                    const uint32_t *a = s_tile + (size_t)tid * aw;
+                    const bool real = tid < n_tile;
+                    const uint32_t solq = real ? a[CMAX + 1] : 0u;
+                    solitary_here = solq >> 31;
 #pragma unroll
-                for (int c = 0; c < CMAX; ++c) s_centre[c][tid] = real ? __uint_as_float(a[c]) : 0.f;
-                s_rsq[tid] = (real && !solitary_here) ? __uint_as_float(a[CMAX]) : -1.f;
-                s_self[tid] = solitary_here ? solq : 0u;
+                    for (int c = 0; c < CMAX; ++c) s_centre[c][tid] = real ? __uint_as_float(a[c]) : 0.f;
+                    s_rsq[tid] = (real && !solitary_here) ? __uint_as_float(a[CMAX]) : -1.f;
+                    s_self[tid] = solitary_here ? solq : 0u;
+                    s_rank[tid] = base + tid;
+                }
+            } else {
+                // one point per thread; it stays if its box meets the items' bins
+                const int n_chunk = min(kTile, rank_hi - base);
+                const uint32_t *src = p.points + (size_t)(first_h + base + tid) * aw;
+                uint32_t w[aw];
+                bool keep = false;
+                if (tid < n_chunk) {
+#pragma unroll
+                    for (int e = 0; e < aw / 4; ++e) {
+                        const uint4 v = reinterpret_cast<const uint4 *>(src)[e];
+                        w[4 * e] = v.x, w[4 * e + 1] = v.y, w[4 * e + 2] = v.z, w[4 * e + 3] = v.w;
+                    }
+                    keep = true;
+#pragma unroll
+                    for (int d = 0; d < kMaxBinDims; ++d) {
+                        const uint32_t box = w[CMAX + 4 + d];
+                        keep = keep && (int)(int16_t)(box & 0xffffu) <= bin_hi[d] && ((int)box >> 16) >= bin_lo[d];
+                    }
+                }
+                const uint64_t kept = __ballot(keep);
+                if (lane == 0) s_kept[wave] = __popcll(kept);
+                __syncthreads();
+                int at = 0;
+                n_tile = 0;
+#pragma unroll
+                for (int w = 0; w < kTile / kWave; ++w) {
+                    if (w == wave) at = n_tile;
+                    n_tile += s_kept[w];
+                }
+                if (keep) {
+                    const int t = at + __popcll(kept & ((1ull << lane) - 1ull));
+#pragma unroll
+                    for (int e = 0; e < aw / 4; ++e)
+                        reinterpret_cast<uint4 *>(s_tile + (size_t)t * aw)[e] =
+                            uint4{w[4 * e], w[4 * e + 1], w[4 * e + 2], w[4 * e + 3]};
+                    const uint32_t solq = w[CMAX + 1];
+                    solitary_here = solq >> 31;
+#pragma unroll
+                    for (int c = 0; c < CMAX; ++c) s_centre[c][t] = __uint_as_float(w[c]);
+                    s_rsq[t] = solitary_here ? -1.f : __uint_as_float(w[CMAX]);
+                    s_self[t] = solitary_here ? solq : 0u;
+                    s_rank[t] = base + tid;
+                }
+                if (tid >= n_tile && tid < ((n_tile + 3) & ~3)) {  // the four-wide test reads up to here
+#pragma unroll
+                    for (int c = 0; c < CMAX; ++c) s_centre[c][tid] = 0.f;
+                    s_rsq[tid] = -1.f;
+                    s_self[tid] = 0u;
+                }
             }
             const bool any_solitary = __syncthreads_or(solitary_here);
             if (mine) {
@@ -677,7 +773,7 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
                                 const float lhs = best * __uint_as_float(a[CMAX]);
                                 if (!(lhs >= dsq)) continue;
                                 best = dsq;
-                                shower = base + t4 + j;
+                                shower = s_rank[t4 + j];
                                 asso = (int)a[CMAX + 2];
                             }
                             continue;
@@ -694,7 +790,7 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
                     const uint32_t *a = s_tile + (size_t)found * aw;
                     float dsq;
                     if (!covers<CMAX>(a, x, uncoverable, self_q, k, dsq)) continue;
-                    shower = base + found;
+                    shower = s_rank[found];
                     asso = (int)a[CMAX + 2];
                     mine = alive = false;
                     break;
