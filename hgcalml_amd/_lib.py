@@ -32,6 +32,8 @@ _SIGNATURES = {
     "hgc_binned_select_knn": (_c_int, [_ptr] * 9 + [_c_int] * 7 + [_ptr]),
     "hgc_binned_select_knn_fused": (_c_int, [_ptr] * 9 + [_c_float] + [_ptr] * 2 + [_c_int] * 7 + [_ptr]),
     "hgc_set_knn_grid": (_c_int, [_c_int]),
+    "hgc_sort_distinct_keys_workspace_bytes": (_c_size, [ctypes.c_longlong]),
+    "hgc_sort_distinct_keys": (_c_int, [_ptr, ctypes.c_longlong, _c_int, _ptr, _ptr, _c_size, _c_int, _ptr]),
     "hgc_binned_select_knn_pipeline_workspace_bytes": (_c_size, [_c_int] * 6),
     "hgc_binned_select_knn_pipeline": (_c_int, [_ptr] * 3 + [_c_int] * 7 + [_c_float, _ptr, _ptr, _ptr, _ptr, _c_size, _ptr]),
     "hgc_binned_select_knn_pipeline_static": (_c_int, [_ptr] * 3 + [_c_int] * 7 + [_c_float, _ptr, _ptr, _ptr, _ptr]),

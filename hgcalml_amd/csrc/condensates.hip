@@ -149,8 +149,9 @@ __device__ __forceinline__ int event_of(const int *__restrict__ splits, int num_
 }
 
 // ascending sort key == selection order; clears the per-candidate outputs
+// position_bits > 0: the position goes into the key's low bits (all keys differ, the sort need not be stable)
 __global__ __launch_bounds__(256) void selection_keys_kernel(const CondParams p, uint64_t *__restrict__ keys,
-                                                             int *__restrict__ values) {
+                                                             int *__restrict__ values, int position_bits) {
     const int q = blockIdx.x * blockDim.x + threadIdx.x;
     if (q >= p.n_vert_h) return;
     const uint64_t ev = (uint64_t)event_of(p.row_splits_h, p.num_rows, q);
@@ -161,7 +162,8 @@ __global__ __launch_bounds__(256) void selection_keys_kernel(const CondParams p,
         u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // monotone map float -> uint
         low = (uint32_t)~u;                               // larger beta first
     }
-    keys[q] = (ev << 34) | (cls << 32) | low;
+    const uint64_t key = (ev << 34) | (cls << 32) | low;
+    keys[q] = position_bits ? ((key << position_bits) | (uint64_t)q) : key;
     values[q] = q;
     p.is_alpha_h[q] = 0;
     p.taken_h[q] = 0;
@@ -914,6 +916,7 @@ size_t condensates_workspace_bytes(int n_vert, int n_vert_h, int num_rows, int d
     (void)rocprim::radix_sort_pairs(nullptr, temp, (const uint64_t *)nullptr, (uint64_t *)nullptr,
                                     (const int *)nullptr, (int *)nullptr, nh, 0,
                                     selection_key_bits(std::max(num_rows, 1)), (hipStream_t) nullptr);
+    temp = std::max(temp, sample_sort_workspace_bytes());
     return align_up(temp) + carve_workspace(nullptr, n_vert, n_vert_h, num_rows, dimensions).used;
 }
 
@@ -991,11 +994,24 @@ int condensates_assign(int dimensions, int dimensions_binning, int *d_condensate
     int last_launch = 0;
     if (num_rows > 0) {
         if (n_vert_h > 0) {
-            selection_keys_kernel<<<ceil_div(n_vert_h, 256), 256, 0, s>>>(p, w.keys, w.values);
+            // The position of a hit completes its key where both fit into 64 bits: then the
+            // keys differ pairwise and the sample sort orders them; a stable library radix
+            // sort otherwise.
+            int position_bits = 1;
+            while ((1ll << position_bits) < (long long)n_vert_h) ++position_bits;
+            const bool own_sort =
+                sample_sort_supported(n_vert_h) && selection_key_bits(num_rows) + position_bits <= 64;
+            selection_keys_kernel<<<ceil_div(n_vert_h, 256), 256, 0, s>>>(p, w.keys, w.values,
+                                                                          own_sort ? position_bits : 0);
             int rc = check_launch("selection_keys");
             if (rc) return rc;
-            HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, w.keys, w.keys_sorted, w.values, w.order,
-                                              (size_t)n_vert_h, 0, selection_key_bits(num_rows), s));
+            if (own_sort) {
+                rc = sample_sort_values(w.keys, w.keys_sorted, n_vert_h, position_bits, w.order, temp, temp_bytes, 0, s);
+                if (rc) return rc;
+            } else {
+                HGC_HIP(rocprim::radix_sort_pairs(temp, temp_bytes, w.keys, w.keys_sorted, w.values, w.order,
+                                                  (size_t)n_vert_h, 0, selection_key_bits(num_rows), s));
+            }
         }
         const int slots = coordinate_slots(dimensions);
         const int rc = slots == 4   ? run<4>(p, s, last_launch)

@@ -70,6 +70,15 @@ struct Carver {
 
 // ---- internal entry points shared between translation units -----------------
 
+// Ascending sort of n pairwise different 64-bit keys (none of them all ones;
+// d_keys is overwritten, d_spare holds n more keys): the low `value_bits` bits of
+// the i-th smallest key go to d_values[i]. `stage` = 0 or, for tests, the number of
+// keys a workgroup sorts in LDS at once (a power of two up to 8192).
+bool sample_sort_supported(long long n);
+size_t sample_sort_workspace_bytes();
+int sample_sort_values(uint64_t *d_keys, uint64_t *d_spare, long long n, int value_bits, int *d_values,
+                       void *workspace, size_t workspace_bytes, int stage, hipStream_t s);
+
 // Groups the points by bin for the kNN search in a handful of launches: grid from
 // the bounding box, bin of every point, bin boundary table and the inputs moved
 // into bin order (`d_sorting[i]` = original index of the i-th point). Unlike

@@ -312,6 +312,20 @@ def inverse_neighbour_index(indices):
     return offsets, slots
 
 
+def sort_distinct_keys(keys, value_bits, stage=0):
+    """Ascending order of pairwise different 64-bit keys (int64 tensor holding the
+    unsigned bit patterns): the low `value_bits` bits of the i-th smallest key."""
+    dev = require_device(keys)
+    if keys.dtype != torch.int64 or keys.dim() != 1:
+        raise ValueError("sort_distinct_keys: keys must be a 1-D int64 tensor")
+    work = keys.contiguous().clone()
+    n = work.numel()
+    values = torch.empty((n,), dtype=torch.int32, device=dev)
+    ws = workspace(lib.hgc_sort_distinct_keys_workspace_bytes(n), dev)
+    check(lib.hgc_sort_distinct_keys(p(work), n, int(value_bits), p(values), p(ws), ws.numel(), int(stage), stream()))
+    return values
+
+
 _INVERSE_CACHE = {}
 
 

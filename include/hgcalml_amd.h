@@ -388,6 +388,17 @@ int hgc_exp_neg(const float *d_distances, float *d_weights, long long n_values, 
 int hgc_exp_neg_grad(const float *d_weight_grad, const float *d_weights, float *d_distance_grad,
                      long long n_values, hgc_stream_t stream);
 
+/* Ascending sort of n 64-bit keys that differ pairwise (none of them all ones):
+ * d_values[i] = the low value_bits bits of the i-th smallest key. The order of
+ * the condensate selection (event, beta descending, position) is this sort; the
+ * reference has no counterpart (binned_assign_to_condensates_kernel.cc:187-236
+ * picks by a linear arg-max per condensation point). d_keys is overwritten.
+ * n <= 2^20. stage: 0, or the number of keys a workgroup sorts in LDS at once
+ * (a power of two up to 8192; smaller values only make it slower). */
+size_t hgc_sort_distinct_keys_workspace_bytes(long long n);
+int hgc_sort_distinct_keys(unsigned long long *d_keys, long long n, int value_bits, int *d_values,
+                           void *workspace, size_t workspace_bytes, int stage, hgc_stream_t stream);
+
 /* ------------------------------------------------------------------ */
 /* Condensate assignment                                               */
 /* ------------------------------------------------------------------ */

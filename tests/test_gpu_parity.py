@@ -1346,3 +1346,62 @@ def test_condensates_ragged_index_helpers_on_device(keep_noise):
     assert torch.equal(per_cond[ev_start[rev[:, 0].to(torch.int64)] + rev[:, 1].to(torch.int64)], a)
     if keep_noise:
         assert (a >= 0).all()
+
+
+def distinct_keys(kind, n, rng):
+    """uint64 keys with the position in the low 20 bits, so that all of them differ"""
+    pos = np.arange(n, dtype=np.uint64)
+    if kind == "random":
+        high = rng.integers(0, 1 << 43, n, dtype=np.uint64)
+    elif kind == "few_values":          # long runs of equal high parts: ties broken by position only
+        high = rng.integers(0, 5, n, dtype=np.uint64) * np.uint64(977)
+    elif kind == "one_value":
+        high = np.full(n, 12345, np.uint64)
+    elif kind == "ascending":
+        high = pos * np.uint64(3)
+    elif kind == "descending":
+        high = (np.uint64(n) - pos) * np.uint64(3)
+    elif kind == "selection":           # (event, class, beta) of a condensate call
+        ev = (pos * np.uint64(8) // np.uint64(max(n, 1))).astype(np.uint64)
+        cls = rng.choice(np.array([0, 1, 1, 1, 2, 2], np.uint64), n)
+        beta = rng.beta(0.5, 2.0, n).astype(np.float32).view(np.uint32).astype(np.uint64)
+        low = np.where(cls == 1, np.uint64(0xffffffff) - (beta | np.uint64(0x80000000)), np.uint64(0))
+        high = (ev << np.uint64(34)) | (cls << np.uint64(32)) | low
+    elif kind == "periodic":            # small keys exactly where the splitter sample looks
+        stride = max(n // 4096, 1)
+        high = np.where((pos - np.uint64(stride // 2)) % np.uint64(stride) == 0, np.uint64(1), np.uint64(1) << np.uint64(30))
+        high = high + rng.integers(0, 1 << 20, n, dtype=np.uint64)
+    return (high << np.uint64(20)) | pos
+
+
+@pytest.mark.parametrize("kind", ["random", "few_values", "one_value", "ascending", "descending", "selection", "periodic"])
+@pytest.mark.parametrize("n", [1, 2, 3, 1000, 8192, 8193, 40000, 500000, 1 << 20])
+def test_sort_distinct_keys(kind, n):
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(n % 1000 + len(kind))
+    keys = distinct_keys(kind, n, rng)
+    got = ops.sort_distinct_keys(t(keys.view(np.int64)), 20).cpu().numpy()
+    assert (got == np.argsort(keys, kind="stable").astype(np.int32)).all()
+
+
+@pytest.mark.parametrize("n,stage", [(5000, 64), (8192, 1024), (8193, 2), (40000, 128), (300000, 256)])
+def test_sort_distinct_keys_buckets_beyond_the_lds_stage(n, stage):
+    """with a small stage every bucket takes the path of sorted runs merged through global memory"""
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(n + stage)
+    for kind in ("random", "few_values", "descending"):
+        keys = distinct_keys(kind, n, rng)
+        got = ops.sort_distinct_keys(t(keys.view(np.int64)), 20, stage=stage).cpu().numpy()
+        assert (got == np.argsort(keys, kind="stable").astype(np.int32)).all()
+
+
+def test_sort_distinct_keys_refuses_what_it_cannot_do():
+    from hgcalml_amd import ops
+    keys = t(np.arange(10, dtype=np.int64))
+    with pytest.raises(Exception):
+        ops.sort_distinct_keys(keys, 0)
+    with pytest.raises(Exception):
+        ops.sort_distinct_keys(keys, 20, stage=100)          # not a power of two
+    with pytest.raises(Exception):
+        ops.sort_distinct_keys(torch.zeros((1 << 20) + 1, dtype=torch.int64, device=DEV), 21)
+    assert ops.sort_distinct_keys(keys[:0], 20).numel() == 0
