@@ -335,6 +335,47 @@ __device__ __forceinline__ int coherent_load(const int *ptr) {
     return __hip_atomic_load(ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// The event kernel's list of condensation points in LDS, by component: word w of
+// point s sits at list[w * capacity + s] (capacity a multiple of 4, the list on a
+// 16-byte boundary), so that four points are tested at a time. Word CMAX, the
+// squared radius, holds -1 for a point that claims only its own hit (its radius
+// sits in word CMAX + 3) and for the up to three slots behind the last point, so
+// that neither ever passes the sphere test. True if one of the points of the groups
+// of four that overlap [lo, hi) covers the candidate (never by the self rule; xs is
+// the candidate's position). Points before lo in the first group are tested again:
+// the candidate has been through them, none covers it.
+template <int CMAX>
+__device__ __forceinline__ bool covered_by_list(const uint32_t *list, int capacity, int lo, int hi,
+                                                const float (&xs)[CMAX], const int (&k)[kMaxBinDims]) {
+    for (int s4 = lo & ~3; s4 < hi; s4 += 4) {
+        float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+        for (int c = 0; c < CMAX; ++c) {
+            const float4 cc = *reinterpret_cast<const float4 *>(list + (size_t)c * capacity + s4);
+            float t = cc.x - xs[c];
+            d0 = d0 + t * t;
+            t = cc.y - xs[c];
+            d1 = d1 + t * t;
+            t = cc.z - xs[c];
+            d2 = d2 + t * t;
+            t = cc.w - xs[c];
+            d3 = d3 + t * t;
+        }
+        const float4 rr = *reinterpret_cast<const float4 *>(list + (size_t)CMAX * capacity + s4);
+        if (!((d0 <= rr.x) | (d1 <= rr.y) | (d2 <= rr.z) | (d3 <= rr.w))) continue;
+        uint32_t hits = (d0 <= rr.x ? 1u : 0u) | (d1 <= rr.y ? 2u : 0u) | (d2 <= rr.z ? 4u : 0u) | (d3 <= rr.w ? 8u : 0u);
+        while (hits) {
+            const int s = s4 + __builtin_ctz(hits);
+            hits &= hits - 1u;
+            uint32_t box[kMaxBinDims];
+#pragma unroll
+            for (int d = 0; d < kMaxBinDims; ++d) box[d] = list[(size_t)(CMAX + 4 + d) * capacity + s];
+            if (in_box(box, k)) return true;
+        }
+    }
+    return false;
+}
+
 // Finds the condensation points among the next `budget` candidates (all that are
 // left: budget < 0) of one event per workgroup. The walk over the sorted list
 // collects the candidates that are still open in a queue; `window` of them are
@@ -359,6 +400,25 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
     int n_alpha = launch == 0 ? 0 : p.n_alpha_at[(launch - 1) * p.num_rows + r];
     const int end = budget < 0 ? last_h : (int)min((long long)last_h, (long long)cur + budget);
     int n_list = 0;  // points of this launch, all in s_list
+    // The points go to global memory (for the grid-wide kernels) when the list is given
+    // up, not as they are found: a store in a stage would be waited for at its barrier.
+    auto flush_list = [&]() {
+        const int rank0 = n_alpha - n_list;
+        for (int i = tid; i < n_list; i += kBlock) {
+            uint32_t word[aw];
+#pragma unroll
+            for (int t = 0; t < aw; ++t) word[t] = s_list[(size_t)t * capacity + i];
+            if (word[CMAX + 1] >> 31) word[CMAX] = word[CMAX + 3], word[CMAX + 3] = 0u;
+            uint32_t *out = p.points + (size_t)(first_h + rank0 + i) * aw;
+#pragma unroll
+            for (int t = 0; t < aw; t += 4)
+                *reinterpret_cast<uint4 *>(out + t) = uint4{word[t], word[t + 1], word[t + 2], word[t + 3]};
+            const int q = (int)(word[CMAX + 1] & 0x7fffffffu);
+            p.alpha_indices[first_h + rank0 + i] = (int)word[CMAX + 2];
+            p.is_alpha_h[q] = 1;
+            p.taken_h[q] = 1;
+        }
+    };
     int n_queue = 0;
     int stopped_at = -1;
 
@@ -366,11 +426,15 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         // ---- refill the queue with the open candidates of the next windows, in order ----
         while (n_queue < window && cur < end) {
             uint64_t open_mask[kFill];
+            int is_closed[kFill];  // all loads of the step in flight together
 #pragma unroll
             for (int j = 0; j < kFill; ++j) {
                 const int pos = cur + j * kBlock + tid;
-                const bool open = pos < end && coherent_load(p.closed + pos) == 0;
-                open_mask[j] = __ballot(open);
+                is_closed[j] = pos < end ? coherent_load(p.closed + pos) : 1;
+            }
+#pragma unroll
+            for (int j = 0; j < kFill; ++j) {
+                open_mask[j] = __ballot(is_closed[j] == 0);
                 if (lane == 0) s_fill[j][wave] = __popcll(open_mask[j]);
             }
             __syncthreads();
@@ -415,14 +479,9 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
                 for (int c = 0; c < CMAX; ++c) xi[c] = __uint_as_float(ri[c]);
 #pragma unroll
                 for (int d = 0; d < kMaxBinDims; ++d) ki[d] = (int)ri[CMAX + d];
-                for (int s = 0; s < n_list; ++s) {
-                    float dsq;
-                    if (covers<CMAX>(s_list + (size_t)s * aw, xi, false, -1, ki, dsq)) {
-                        p.closed[i] = 1;
-                        break;
-                    }
-                }
+                if (covered_by_list<CMAX>(s_list, capacity, 0, n_list, xi, ki)) p.closed[i] = 1;
             }
+            flush_list();
             __threadfence();
             __syncthreads();
             n_list = 0;
@@ -457,14 +516,7 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         bool open = valid;
 
         // ---- points found earlier in this launch ----
-        if (__ballot(open && !uncoverable)) {
-            for (int s = 0; s < n_list; ++s) {
-                float dsq;
-                if (open && !uncoverable && covers<CMAX>(s_list + (size_t)s * aw, x, false, -1, k, dsq))
-                    open = false;
-                if ((s & 15) == 15 && !__ballot(open && !uncoverable)) break;
-            }
-        }
+        if (open && !uncoverable && covered_by_list<CMAX>(s_list, capacity, 0, n_list, x, k)) open = false;
         const uint64_t wave_open = __ballot(open);
         if (lane == 0) {
             s_open[wave] = wave_open != 0;
@@ -473,60 +525,69 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         __syncthreads();
 
         // ---- the window, wave after wave ----
+        // Stage w: wave w picks its condensation points one after the other (the first
+        // open lane is one, the lanes it covers close) and adds them to the list. The
+        // waves behind it test their candidates against the points of the stage before
+        // while it does so; wave w itself has done that first.
         const int n_waves = (take + kWave - 1) / kWave;
+        const uint64_t coverable_lanes = __ballot(!uncoverable);
+        int tested = n_list;  // the waves still waiting for their stage have seen the list up to here
         for (int w = 0; w < n_waves; ++w) {
             if (!s_open[w]) continue;  // uniform
+            if (wave == w) __builtin_amdgcn_s_setprio(3);  // the others wait for this wave
+            if (wave >= w && open && !uncoverable && covered_by_list<CMAX>(s_list, capacity, tested, n_list, x, k))
+                open = false;
             if (wave == w) {
-                int cnt = 0;
-                bool chosen = false;
-                while (true) {
-                    const uint64_t m = __ballot(open);
-                    if (!m) break;
-                    const int first = __builtin_ctzll(m);  // the next condensation point
-                    if (lane == first) {
-                        chosen = true;
-                        open = false;
-                    }
+                uint64_t open_lanes = __ballot(open), chosen_lanes = 0;
+                while (open_lanes) {
+                    const int first = __builtin_ctzll(open_lanes);  // the next condensation point
+                    open_lanes &= open_lanes - 1ull;
+                    chosen_lanes |= 1ull << first;
                     // the other lanes get the point from that lane's registers
-                    uint32_t head[CMAX + 2], box[kMaxBinDims];
+                    uint32_t head[CMAX + 2];
 #pragma unroll
                     for (int t = 0; t < CMAX + 2; ++t) head[t] = (uint32_t)__builtin_amdgcn_readlane((int)point[t], first);
+                    if (head[CMAX + 1] >> 31) continue;  // claims only its own hit
+                    float acc = 0.f;  // every lane, whatever its state: the masks below are scalars
 #pragma unroll
-                    for (int d = 0; d < kMaxBinDims; ++d)
-                        box[d] = (uint32_t)__builtin_amdgcn_readlane((int)point[CMAX + 4 + d], first);
-                    float dsq;
-                    if (open && !uncoverable && in_sphere<CMAX>(head, x, false, -1, dsq) && in_box(box, k)) open = false;
-                    ++cnt;
-                }
-                const uint64_t chosen_mask = __ballot(chosen);
-                if (chosen) {
-                    // for the later waves (LDS) and the grid-wide kernels (global memory)
-                    const int nth = __popcll(chosen_mask & ((1ull << lane) - 1ull));
-                    uint32_t *slot = s_list + (size_t)(n_list + nth) * aw;
-                    const int rank = n_alpha + nth;
-                    uint32_t *out = p.points + (size_t)(first_h + rank) * aw;
-#pragma unroll
-                    for (int t = 0; t < aw; t += 4) {
-                        const uint4 v{point[t], point[t + 1], point[t + 2], point[t + 3]};
-                        *reinterpret_cast<uint4 *>(slot + t) = v;
-                        *reinterpret_cast<uint4 *>(out + t) = v;
+                    for (int c = 0; c < CMAX; ++c) {
+                        const float t = __uint_as_float(head[c]) - x[c];
+                        acc = acc + t * t;
                     }
-                    const int q = (int)(point[CMAX + 1] & 0x7fffffffu);
-                    p.alpha_indices[first_h + rank] = (int)point[CMAX + 2];
-                    p.is_alpha_h[q] = 1;
-                    p.taken_h[q] = 1;
+                    uint64_t inside = __ballot(acc <= __uint_as_float(head[CMAX])) & open_lanes & coverable_lanes;
+                    if (inside) {  // the box only matters for lanes inside the sphere
+                        uint32_t box[kMaxBinDims];
+#pragma unroll
+                        for (int d = 0; d < kMaxBinDims; ++d)
+                            box[d] = (uint32_t)__builtin_amdgcn_readlane((int)point[CMAX + 4 + d], first);
+                        inside &= __ballot(in_box(box, k));
+                        open_lanes &= ~inside;
+                    }
                 }
-                if (lane == 0) s_cnt[w] = cnt;
+                open = false;  // every lane of the wave is a condensation point now, or covered by one
+                if ((chosen_lanes >> lane) & 1ull) {
+                    // for the waves behind
+                    const int nth = __popcll(chosen_lanes & ((1ull << lane) - 1ull));
+                    const bool solitary = point[CMAX + 1] >> 31;
+#pragma unroll
+                    for (int t = 0; t < aw; ++t) {
+                        uint32_t word = point[t];
+                        if (t == CMAX && solitary) word = __float_as_uint(-1.f);
+                        if (t == CMAX + 3 && solitary) word = point[CMAX];
+                        s_list[(size_t)t * capacity + n_list + nth] = word;
+                    }
+                }
+                {  // no sphere for the slots behind the last point of the list
+                    const int end_of_list = n_list + __popcll(chosen_lanes);
+                    if (lane < 3 && end_of_list + lane < capacity)
+                        s_list[(size_t)CMAX * capacity + end_of_list + lane] = __float_as_uint(-1.f);
+                }
+                if (lane == 0) s_cnt[w] = __popcll(chosen_lanes);
+                __builtin_amdgcn_s_setprio(0);
             }
             __syncthreads();
             const int added = s_cnt[w];
-            if (wave > w && __ballot(open && !uncoverable)) {
-                for (int s = n_list; s < n_list + added; ++s) {
-                    float dsq;
-                    if (open && !uncoverable && covers<CMAX>(s_list + (size_t)s * aw, x, false, -1, k, dsq))
-                        open = false;
-                }
-            }
+            tested = n_list;
             n_list += added;
             n_alpha += added;
         }
@@ -543,6 +604,7 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
         n_queue = rest;
         __syncthreads();
     }
+    flush_list();
     if (tid == 0) {
         p.cursor_at[launch * p.num_rows + r] = stopped_at >= 0 ? stopped_at : end;
         p.n_alpha_at[launch * p.num_rows + r] = n_alpha;
@@ -877,7 +939,7 @@ int run(const CondParams &p, hipStream_t s, int &last_launch) {
                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) == hipSuccess)
         list_bytes = 128 * 1024;
     (void)hipGetLastError();  // a refused grant is not an error of this call
-    const int capacity = (int)(list_bytes / point_bytes);
+    const int capacity = (int)(list_bytes / point_bytes) & ~3;  // the list is read four points at a time
     const int window = std::min(kBlock, capacity / 2 / kWave * kWave);
     // geometric shares of the sorted candidates, the last launch takes what is left;
     // n_vert_h bounds every event
