@@ -94,8 +94,8 @@ struct CondParams {
     int *pos_h;          // [n_vert_h] position of a high-beta hit among all hits, -1 unknown
     int *hit_bin;        // [n_vert] bin of a hit inside its event's grid, INT_MIN unknown
     uint32_t *cand;      // [n_vert_h] candidate records in selection order
-    int *closed;         // [n_vert_h] by selection position: never a condensation point (cannot be
-                         // picked at all, or a point of an earlier launch covers it)
+    unsigned long long *open_bits;  // one bit per selection position, 64 positions a word: still a
+                                    // candidate (it can be picked at all, and no point found so far covers it)
     uint32_t *points;    // [n_vert_h] an event's condensation points in selection order, from
                          // row_splits_h[event] on
     int *walk_end;       // [num_rows] end of the event's candidates that can be picked at all
@@ -220,14 +220,16 @@ struct Grid {
 template <int CMAX>
 __global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams p) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= p.n_vert_h) return;
+    const bool in_range = i < p.n_vert_h;
+    const int q = in_range ? p.order_h[i] : 0;
+    const bool selectable = in_range && selection_class(p, q) < 2;
+    const uint64_t open = __ballot(selectable);  // a wave holds 64 consecutive positions of one word
+    if ((threadIdx.x & (kWave - 1)) == 0 && in_range) p.open_bits[i >> 6] = open;
+    if (!in_range) return;
     constexpr int cw = cand_words(CMAX);
     const int C = p.C, B = p.B;
     Grid g;
     g.load(p);
-    const int q = p.order_h[i];
-    const bool selectable = selection_class(p, q) < 2;
-    p.closed[i] = selectable ? 0 : 1;
     if (!selectable) {
         // those that are never picked come last in an event's order: the walk ends at the first one
         const int ev = event_of(p.row_splits_h, p.num_rows, i);
@@ -331,7 +333,7 @@ __device__ __forceinline__ bool covers(const uint32_t *a, const float (&x)[CMAX]
     return in_box(box, k);
 }
 
-__device__ __forceinline__ int coherent_load(const int *ptr) {
+__device__ __forceinline__ unsigned long long coherent_load(const unsigned long long *ptr) {
     return __hip_atomic_load(ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -424,36 +426,42 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
 
     for (;;) {
         // ---- refill the queue with the open candidates of the next windows, in order ----
+        // One word of 64 positions per thread. If the open ones of all 1024 words fit
+        // into the queue they are all taken (the rule once most candidates are covered),
+        // else as many words as fit whatever they hold.
         while (n_queue < window && cur < end) {
-            uint64_t open_mask[kFill];
-            int is_closed[kFill];  // all loads of the step in flight together
-#pragma unroll
-            for (int j = 0; j < kFill; ++j) {
-                const int pos = cur + j * kBlock + tid;
-                is_closed[j] = pos < end ? coherent_load(p.closed + pos) : 1;
-            }
-#pragma unroll
-            for (int j = 0; j < kFill; ++j) {
-                open_mask[j] = __ballot(is_closed[j] == 0);
-                if (lane == 0) s_fill[j][wave] = __popcll(open_mask[j]);
-            }
+            const int word0 = cur >> 6;
+            const long long base = ((long long)word0 + tid) << 6;
+            unsigned long long bits = base < end ? coherent_load(p.open_bits + word0 + tid) : 0ull;
+            if (tid == 0) bits &= ~0ull << (cur & 63);
+            if (base + 64 > end) bits = end > base ? bits & ((1ull << (end - base)) - 1ull) : 0ull;
+            const int mine = __popcll(bits);
+            const int upto = wave_inclusive_sum(mine);
+            if (lane == kWave - 1) s_fill[0][wave] = upto;
             __syncthreads();
-            int at = n_queue, total = 0;
-            int mine[kFill];
+            int before = upto - mine, total = 0;
 #pragma unroll
-            for (int j = 0; j < kFill; ++j) {
-#pragma unroll
-                for (int w = 0; w < kWavesPerBlock; ++w) {
-                    if (w == wave) mine[j] = at + total;
-                    total += s_fill[j][w];
+            for (int w = 0; w < kWavesPerBlock; ++w) {
+                if (w < wave) before += s_fill[0][w];
+                total += s_fill[0][w];
+            }
+            const int room = kQueueCap - n_queue;
+            int words = kBlock, taken = total;
+            if (total > room) {
+                words = room >> 6;
+                if (tid == words) s_fill[1][0] = before;
+                __syncthreads();
+                taken = s_fill[1][0];
+            }
+            if (tid < words) {
+                int at = n_queue + before;
+                while (bits) {
+                    s_queue[at++] = (int)base + __builtin_ctzll(bits);
+                    bits &= bits - 1ull;
                 }
             }
-#pragma unroll
-            for (int j = 0; j < kFill; ++j)
-                if ((open_mask[j] >> lane) & 1ull)
-                    s_queue[mine[j] + __popcll(open_mask[j] & ((1ull << lane) - 1ull))] = cur + j * kBlock + tid;
-            n_queue += total;
-            cur = (int)min((long long)end, (long long)cur + kFill * kBlock);
+            n_queue += taken;
+            cur = (int)min((long long)end, ((long long)word0 + words) << 6);
             __syncthreads();
         }
         if (n_queue == 0) break;
@@ -470,7 +478,7 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
             // front of the queue
             __syncthreads();
             for (int i = front + tid; i < last_h; i += kBlock) {
-                if (coherent_load(p.closed + i)) continue;
+                if (!((coherent_load(p.open_bits + (i >> 6)) >> (i & 63)) & 1ull)) continue;
                 const uint32_t *ri = p.cand + (size_t)i * cw;
                 if (ri[CMAX + 6]) continue;
                 float xi[CMAX];
@@ -479,7 +487,8 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
                 for (int c = 0; c < CMAX; ++c) xi[c] = __uint_as_float(ri[c]);
 #pragma unroll
                 for (int d = 0; d < kMaxBinDims; ++d) ki[d] = (int)ri[CMAX + d];
-                if (covered_by_list<CMAX>(s_list, capacity, 0, n_list, xi, ki)) p.closed[i] = 1;
+                if (covered_by_list<CMAX>(s_list, capacity, 0, n_list, xi, ki))
+                    atomicAnd(p.open_bits + (i >> 6), ~(1ull << (i & 63)));
             }
             flush_list();
             __threadfence();
@@ -656,10 +665,15 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
     for (int c = 0; c < CMAX; ++c) x[c] = 0.f;
 #pragma unroll
     for (int d = 0; d < kMaxBinDims; ++d) k[d] = INT_MIN;
+    bool was_open = false;
     if (MODE == 0) {
-        if (valid) {
+        // a wave's 64 positions are one word of the bit array
+        const unsigned long long word = i_first + (tid & ~(kWave - 1)) < n_items ? p.open_bits[i >> 6] : 0ull;
+        was_open = valid && ((word >> (tid & (kWave - 1))) & 1ull);
+        alive = false;
+        if (was_open) {
             const uint32_t *rec = p.cand + (size_t)i * cw;
-            alive = p.closed[i] == 0 && i >= p.cursor_at[launch * p.num_rows + my_ev] && rec[CMAX + 6] == 0;
+            alive = i >= p.cursor_at[launch * p.num_rows + my_ev] && rec[CMAX + 6] == 0;
             if (alive) {
 #pragma unroll
                 for (int c = 0; c < CMAX; ++c) x[c] = __uint_as_float(rec[c]);
@@ -862,10 +876,13 @@ __global__ __launch_bounds__(kScanBlock) void cover_scan_kernel(const CondParams
             }
         }
     }
-    if (!valid) return;
     if (MODE == 0) {
-        if (shower >= 0) p.closed[i] = 1;
-    } else {
+        const unsigned long long still_open = __ballot(was_open && shower < 0);
+        if ((tid & (kWave - 1)) == 0 && valid) p.open_bits[i >> 6] = still_open;
+        return;
+    }
+    if (!valid) return;
+    {
         p.assignment[i] = shower;
         p.association[i] = asso;
         if (MODE == 2) p.best_dsq[i] = best;
@@ -893,7 +910,8 @@ int selection_key_bits(int num_rows) {
 
 struct Workspace {
     uint64_t *keys, *keys_sorted;
-    int *values, *order, *pos_h, *hit_bin, *closed, *walk_end, *cursor_at, *n_alpha_at;
+    int *values, *order, *pos_h, *hit_bin, *walk_end, *cursor_at, *n_alpha_at;
+    unsigned long long *open_bits;
     uint32_t *cand, *points;
     size_t used;
 };
@@ -911,7 +929,7 @@ Workspace carve_workspace(void *base, int n_vert, int n_vert_h, int num_rows, in
     w.order = carve.take<int>(nh);
     w.pos_h = carve.take<int>(nh);
     w.hit_bin = carve.take<int>(n);
-    w.closed = carve.take<int>(nh);
+    w.open_bits = carve.take<unsigned long long>(nh / 64 + 2);
     w.points = carve.take<uint32_t>(nh * (size_t)alpha_words(cmax));
     w.walk_end = carve.take<int>(rows);
     w.cursor_at = carve.take<int>(kMaxLaunches * rows);
@@ -1047,7 +1065,7 @@ int condensates_assign(int dimensions, int dimensions_binning, int *d_condensate
     p.pos_h = w.pos_h;
     p.hit_bin = w.hit_bin;
     p.cand = w.cand;
-    p.closed = w.closed;
+    p.open_bits = w.open_bits;
     p.points = w.points;
     p.walk_end = w.walk_end;
     p.cursor_at = w.cursor_at;
