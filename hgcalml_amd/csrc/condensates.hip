@@ -58,7 +58,7 @@ constexpr int kFill = 4;         // windows of the sorted list looked at per ref
 constexpr int kQueueCap = kBlock + kFill * kBlock;
 constexpr int kScanBlock = 256;  // threads of the grid-wide kernels
 constexpr int kTile = 256;       // condensation points staged in LDS at a time there (one per thread)
-constexpr int kMaxLaunches = 4;  // launches of the event kernel
+constexpr int kMaxLaunches = 3;  // launches of the event kernel (cfg5-like input: 0.47 ms with 3, 0.48 with 4, 0.55 with 2)
 
 struct CondParams {
     int C, B;
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void selection_keys_kernel(const CondParams p,
     p.is_alpha_h[q] = 0;
     p.taken_h[q] = 0;
     p.alpha_indices[q] = -1;
-    p.pos_h[q] = -1;
+    if (!p.high) p.pos_h[q] = -1;
 }
 
 // bin of every hit inside its event's grid (from the bin boundaries), and the
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(256) void hit_prepare_kernel(const CondParams p) {
     }
     p.hit_bin[i] = (cells > 0 && splits[lo] <= i && i < splits[lo + 1]) ? lo : INT_MIN;
     const int q = p.to_filtered[i];
-    if (q >= 0 && q < p.n_vert_h) p.pos_h[q] = i;
+    if (!p.high && q >= 0 && q < p.n_vert_h) p.pos_h[q] = i;
 }
 
 struct Grid {
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256) void candidate_records_kernel(const CondParams
         if (i == p.row_splits_h[ev] || selection_class(p, p.order_h[i - 1]) < 2) p.walk_end[ev] = i;
         return;  // nobody reads its record
     }
-    const int at = p.pos_h[q];
+    const int at = p.high ? q : p.pos_h[q];  // hits as their own high-beta subset: same index
     uint32_t rec[cw];
     uint32_t *point = rec + CMAX + 8;
     float centre[CMAX];
