@@ -340,10 +340,7 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
         const bool has_radius = p.radius_sq >= 0.f;
         const int kth_lane = (Kn - 1) & (kWave - 1);
         const int kth_level = (Kn - 1) >> 6;
-        // With a spare rank behind the K-th one (S*64 > K-1) a candidate that no
-        // longer beats the K-th key may be inserted anyway: it lands in the spare
-        // ranks. Then the K-th key is re-read once per batch instead of per insert.
-        const bool spare_rank = S * kWave > Kn;
+        // The K-th key is re-read once per step of 64 candidates, not per insert.
         uint64_t thr = kEmptyKey;  // current K-th key: candidates at or above it cannot enter
         // first key beyond the radius: d² <= r² <=> key < (bits(r²) + 1) << 32 for the non-negative r²
         const uint64_t radius_limit = has_radius ? (uint64_t)(__float_as_uint(p.radius_sq) + 1u) << 32 : kEmptyKey;
@@ -499,14 +496,9 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                                 const int src = __ffsll((long long)beats) - 1;
                                 beats &= beats - 1;
                                 const uint64_t cand = readlane_u64(ck, src);
-                                if (!spare_rank) {  // no spare rank: re-check against the current K-th key
-                                    uint64_t kth = kEmptyKey;
-#pragma unroll
-                                    for (int s = 0; s < S; ++s)
-                                        if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
-                                    const uint32_t ch = (uint32_t)(cand >> 32), kh = (uint32_t)(kth >> 32);
-                                    if (ch > kh || (ch == kh && (uint32_t)cand >= (uint32_t)kth)) continue;
-                                }
+                                // a candidate that an earlier insert of this step has pushed beyond the
+                                // K-th rank lands in a spare rank behind it or, in a list without one,
+                                // is larger than every key and changes nothing
                                 sorted_insert<S>(key, cand);
                             }
 #pragma unroll
