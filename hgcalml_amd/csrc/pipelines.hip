@@ -39,7 +39,10 @@ namespace {
 // four coordinates keep three binned dimensions, and their bins hold every point along the
 // others: the neighbourhood is wide in bin widths however fine the grid, so a coarser one,
 // 0.6 (points per event)^(1/3), serves better (150,000 points, K = 64, uniform / Gaussian:
-// 5-D 2.46 / 1.81 ms at 53 bins -> 1.4 / 1.8 ms at 32; 8-D 14.7 / 8.4 -> 7.9 / 8.0 ms).
+// 5-D 2.46 / 1.81 ms at 53 bins -> 1.4 / 1.8 ms at 32; 8-D 14.7 / 8.4 -> 7.9 / 8.0 ms). Small events
+// want fewer bins than one point per cell gives them (most of a small grid is boundary, and a shell
+// costs its rows whether they are inside the grid or not): 200,000 uniform 4-D points in 1000 events,
+// K = 64: 0.80 ms at 4 bins, 0.52 at 3; in 4000 events 1.07 ms at 4 bins, 0.31 at 2.
 thread_local int g_callers_knn_grid = 0;
 
 struct SearchGrid {
@@ -54,8 +57,10 @@ SearchGrid own_grid(int n_vert, int n_coords, int n_rs) {
     const int dims = n_coords <= 4 ? n_coords : 3;
     const double per_event = std::max(1.0, (double)n_vert / std::max(1, n_rs - 1));
     const double per_cell_rule = std::pow(per_event, 1.0 / std::max(dims, 1));
-    const int n_bins = (int)std::lround(n_coords <= 4 ? per_cell_rule : 0.6 * per_cell_rule);
-    return {dims, std::max(4, std::min(n_bins, dims >= 4 ? 40 : dims == 3 ? 128 : 1024))};
+    // small events: 0.75 of that up to 5,000 points per event, rising to 1 at 50,000
+    const double small = std::min(1.0, std::max(0.75, 0.75 + 0.25 * (std::log10(per_event) - 3.7)));
+    const int n_bins = (int)std::lround((n_coords <= 4 ? small : 0.6) * per_cell_rule);
+    return {dims, std::max(2, std::min(n_bins, dims >= 4 ? 40 : dims == 3 ? 128 : 1024))};
 }
 
 SearchGrid search_grid(int n_vert, int n_coords, int n_rs, int n_bins_scalar, int max_bin_dims) {

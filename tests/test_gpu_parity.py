@@ -1405,3 +1405,17 @@ def test_sort_distinct_keys_refuses_what_it_cannot_do():
     with pytest.raises(Exception):
         ops.sort_distinct_keys(torch.zeros((1 << 20) + 1, dtype=torch.int64, device=DEV), 21)
     assert ops.sort_distinct_keys(keys[:0], 20).numel() == 0
+
+
+@pytest.mark.parametrize("C,K", [(3, 16), (4, 16), (4, 64), (2, 5)])
+def test_knn_many_small_events(oracle, C, K):
+    """events of 1 to ~100 points (fewer than K in many of them): the library's own grid drops to two or
+    three bins per dimension there; same neighbours and distances as the oracle on the caller's grid"""
+    from hgcalml_amd import BinnedSelectKnn
+    rng = np.random.default_rng(900 + C + K)
+    sizes = rng.integers(1, 100, 120)
+    rs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    coords = rng.random((int(rs[-1]), C), dtype=np.float32)
+    idx, dist = BinnedSelectKnn(K, t(coords), t(rs), n_bins=6)
+    ri, rd = oracle.canonical_knn(*oracle.BinnedSelectKnn(K, coords, rs, n_bins=6))
+    assert (idx.cpu().numpy() == ri).all() and (bits(dist.cpu().numpy()) == bits(rd)).all()
