@@ -341,11 +341,11 @@ __device__ __forceinline__ unsigned long long coherent_load(const unsigned long 
 // point s sits at list[w * capacity + s] (capacity a multiple of 4, the list on a
 // 16-byte boundary), so that four points are tested at a time. Word CMAX, the
 // squared radius, holds -1 for a point that claims only its own hit (its radius
-// sits in word CMAX + 3) and for the up to three slots behind the last point, so
-// that neither ever passes the sphere test. True if one of the points of the groups
-// of four that overlap [lo, hi) covers the candidate (never by the self rule; xs is
-// the candidate's position). Points before lo in the first group are tested again:
-// the candidate has been through them, none covers it.
+// sits in word CMAX + 3), so that it never passes the sphere test. True if one of
+// the points [lo & ~3, hi) covers the candidate (never by the self rule; xs is the
+// candidate's position). Points before lo in the first group are tested again: the
+// candidate has been through them, none covers it. Slots from hi on are never
+// looked at: another wave may be writing them.
 template <int CMAX>
 __device__ __forceinline__ bool covered_by_list(const uint32_t *list, int capacity, int lo, int hi,
                                                 const float (&xs)[CMAX], const int (&k)[kMaxBinDims]) {
@@ -363,7 +363,13 @@ __device__ __forceinline__ bool covered_by_list(const uint32_t *list, int capaci
             t = cc.w - xs[c];
             d3 = d3 + t * t;
         }
-        const float4 rr = *reinterpret_cast<const float4 *>(list + (size_t)CMAX * capacity + s4);
+        float4 rr = *reinterpret_cast<const float4 *>(list + (size_t)CMAX * capacity + s4);
+        if (s4 + 4 > hi) {  // slots behind the range may be in the middle of being written
+            const int real = hi - s4;
+            rr.w = -1.f;
+            if (real < 3) rr.z = -1.f;
+            if (real < 2) rr.y = -1.f;
+        }
         if (!((d0 <= rr.x) | (d1 <= rr.y) | (d2 <= rr.z) | (d3 <= rr.w))) continue;
         uint32_t hits = (d0 <= rr.x ? 1u : 0u) | (d1 <= rr.y ? 2u : 0u) | (d2 <= rr.z ? 4u : 0u) | (d3 <= rr.w ? 8u : 0u);
         while (hits) {
@@ -585,11 +591,6 @@ __global__ __launch_bounds__(kBlock) void condensate_event_kernel(const CondPara
                         if (t == CMAX + 3 && solitary) word = point[CMAX];
                         s_list[(size_t)t * capacity + n_list + nth] = word;
                     }
-                }
-                {  // no sphere for the slots behind the last point of the list
-                    const int end_of_list = n_list + __popcll(chosen_lanes);
-                    if (lane < 3 && end_of_list + lane < capacity)
-                        s_list[(size_t)CMAX * capacity + end_of_list + lane] = __float_as_uint(-1.f);
                 }
                 if (lane == 0) s_cnt[w] = __popcll(chosen_lanes);
                 __builtin_amdgcn_s_setprio(0);
