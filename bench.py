@@ -131,10 +131,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--roofline-scale", type=float, default=1.0, help="shrink cfg4 (debugging only)")
-    ap.add_argument("--section", choices=["all", "headline", "roofline", "streams"], default="all",
+    ap.add_argument("--section", choices=["all", "headline", "roofline", "streams", "condensates"], default="all",
                     help="run only one part (for profiling); the JSON line is printed for 'all' only. 'streams': the "
                          "cfg4 gradient next to its variants without the max half and without the weight gradient, "
-                         "whose counter differences split its L2 requests by data stream")
+                         "whose counter differences split its L2 requests by data stream. 'condensates': cfg5 alone, both "
+                         "assignment modes")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets ONE GPU (no collectives, no sharding); run with --gpus 1. "
@@ -148,6 +149,14 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
 
+    if args.section == "condensates":
+        c5 = workloads.cfg5(ragged=True)
+        a5 = [torch.from_numpy(c5[k]).to(dev) for k in ("ccoords", "betas", "dist", "row_splits")]
+        for mode in (True, False):
+            m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode),
+                          args.steps, args.warmup)
+            log("bench: cfg5 condensates (%s) %.3f ms" % ("max-beta" if mode else "min-distance", m5[0]))
+        return
     # ------------------------------------------------------------------ headline: cfg2
     c2 = workloads.cfg2()
     n2, K2 = len(c2["coords"]), c2["K"]
