@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libhgcalml_amd.so")
 
-SOURCES = ["binning.hip", "knn.hip", "accumulate.hip", "accumulate_grad_fused.hip", "split_sort.hip", "sample_sort.hip", "inverse_index.hip", "neighbour_ops.hip", "condensates.hip", "pipelines.hip"]
+SOURCES = ["binning.hip", "knn.hip", "accumulate.hip", "accumulate_grad_fused.hip", "accumulate_grad_records.hip", "split_sort.hip", "sample_sort.hip", "inverse_index.hip", "neighbour_ops.hip", "condensates.hip", "pipelines.hip"]
 
 # -ffp-contract=off: distances and accumulations must be separate fp32
 #   multiplies and adds in source order to reproduce the reference bit for bit.

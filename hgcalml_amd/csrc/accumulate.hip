@@ -33,6 +33,14 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
                                  const unsigned char *maxslot, const int *inv_off, const int *inv_slots, float *gw,
                                  float *gfeat, int n_vert, int K, int F, int g_cols, bool mean_and_max, const int *idx,
                                  const int *order, float divisor, hipStream_t s);
+// accumulate_grad_records.hip: both gradients with the max part read from per-slot
+// records built in `records`; returns 1 when the shape is not covered or the storage is
+// too small (accumulate_grad_records_bytes is 0 where the path does not apply).
+size_t accumulate_grad_records_bytes(int n_vert, int K, int F);
+int launch_accumulate_grad_records(const float *g, const float *w, const float *feat, const unsigned char *maxslot,
+                                   const int *inv_off, const int *inv_slots, float *gw, float *gfeat, int n_vert, int K,
+                                   int F, const int *idx, const int *order, float divisor, void *records,
+                                   size_t records_bytes, hipStream_t s);
 
 namespace {
 
@@ -848,7 +856,8 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
                         const int *d_max_feat_indices, const unsigned char *d_max_slots, const int *d_neigh_indices,
                         const int *d_inv_offsets, const int *d_inv_slots, float *d_out_grad_distances,
                         float *d_out_grad_features, int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
-                        int mean_and_max, float divisor, const int *d_order, hgc_stream_t stream) {
+                        int mean_and_max, float divisor, const int *d_order, void *records, size_t records_bytes,
+                        hgc_stream_t stream) {
     const bool want_w = d_out_grad_distances != nullptr, want_f = d_out_grad_features != nullptr;
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_grad_from_out_feat == n_feat * (mean_and_max ? 2 : 1),
@@ -869,6 +878,13 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
     // both gradients from one gather pass where that kernel covers the shape (rows of
     // 16 to 256 features), or the mean-only feature gradient alone: the gather without
     // the dot products
+    if (fits_32bit && want_f && want_w && mean_and_max && d_max_slots && records) {
+        const int rc = launch_accumulate_grad_records(d_grad_from_out_features, d_distances, d_feat, d_max_slots,
+                                                      d_inv_offsets, d_inv_slots, d_out_grad_distances,
+                                                      d_out_grad_features, n_vert, n_neigh, n_feat, d_neigh_indices,
+                                                      d_order, divisor, records, records_bytes, s);
+        if (rc <= 0) return rc;  // 1: shape not covered
+    }
     if (fits_32bit && want_f && (want_w || !mean_and_max)) {
         const int rc = launch_accumulate_grad_fused(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices,
                                                     d_max_slots, d_inv_offsets, d_inv_slots, d_out_grad_distances,
@@ -989,7 +1005,28 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
     return accumulate_gradient(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices, d_max_slots,
                                d_neigh_indices, d_inv_offsets, d_inv_slots, d_out_grad_distances, d_out_grad_features,
                                n_vert, n_neigh, n_feat, n_grad_from_out_feat, mean_and_max, (float)n_neigh,
-                               d_vertex_order, stream);
+                               d_vertex_order, nullptr, 0, stream);
+}
+
+size_t hgc_accumulate_knn_grad_records_workspace_bytes(int n_vert, int n_neigh, int n_feat, int mean_and_max) {
+    return mean_and_max ? accumulate_grad_records_bytes(n_vert, n_neigh, n_feat) : 0;
+}
+
+int hgc_accumulate_knn_grad_records(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
+                                    const int *d_max_feat_indices, const unsigned char *d_max_slots,
+                                    const int *d_neigh_indices, const int *d_inv_offsets, const int *d_inv_slots,
+                                    const int *d_vertex_order, float *d_out_grad_distances, float *d_out_grad_features,
+                                    int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat, int n_moments,
+                                    int mean_and_max, void *workspace, size_t workspace_bytes, hgc_stream_t stream) {
+    (void)n_moments;
+    HGC_REQUIRE(n_vert <= 0 || (d_out_grad_distances && d_out_grad_features), "null pointer");
+    const size_t need = hgc_accumulate_knn_grad_records_workspace_bytes(n_vert, n_neigh, n_feat, mean_and_max);
+    if (need != 0 && d_max_slots && (!workspace || !aligned256(workspace) || workspace_bytes < need))
+        return fail(HGC_ERR_WORKSPACE, "accumulate_knn_grad_records workspace missing, misaligned or too small");
+    return accumulate_gradient(d_grad_from_out_features, d_distances, d_feat, d_max_feat_indices, d_max_slots,
+                               d_neigh_indices, d_inv_offsets, d_inv_slots, d_out_grad_distances, d_out_grad_features,
+                               n_vert, n_neigh, n_feat, n_grad_from_out_feat, mean_and_max, (float)n_neigh,
+                               d_vertex_order, need != 0 ? workspace : nullptr, workspace_bytes, stream);
 }
 
 int hgc_accumulate_knn_grad(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,

@@ -331,6 +331,12 @@ int launch_fused(const float *g, const float *w, const float *feat, const int *m
 
 }  // namespace
 
+int launch_zero_padded_weight_grad(const int *inv_off, const int *inv_slots, float *gw, int n_vert, long long total,
+                                   hipStream_t s) {
+    zero_padded_weight_grad_kernel<<<256, 256, 0, s>>>(inv_off, inv_slots, gw, n_vert, total);
+    return check_launch("zero_padded_weight_grad_kernel");
+}
+
 int launch_accumulate_grad_fused(const float *g, const float *w, const float *feat, const int *maxidx,
                                  const unsigned char *maxslot, const int *inv_off, const int *inv_slots, float *gw,
                                  float *gfeat, int n_vert, int K, int F, int g_cols, bool mean_and_max, const int *idx,
@@ -351,9 +357,7 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
     if (nb < 1 || vec * nb > 4) return 1;
 
     if (want_w) {
-        const long long total = (long long)n_vert * K;
-        zero_padded_weight_grad_kernel<<<256, 256, 0, s>>>(inv_off, inv_slots, gw, n_vert, total);
-        const int rc = check_launch("zero_padded_weight_grad_kernel");
+        const int rc = launch_zero_padded_weight_grad(inv_off, inv_slots, gw, n_vert, (long long)n_vert * K, s);
         if (rc) return rc;
     }
 #define HGC_ARGS                                                                                                   \

@@ -25,7 +25,8 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
                         const int *d_max_feat_indices, const unsigned char *d_max_slots, const int *d_neigh_indices,
                         const int *d_inv_offsets, const int *d_inv_slots, float *d_out_grad_distances,
                         float *d_out_grad_features, int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
-                        int mean_and_max, float divisor, const int *d_order, hgc_stream_t stream);
+                        int mean_and_max, float divisor, const int *d_order, void *records, size_t records_bytes,
+                        hgc_stream_t stream);
 
 namespace {
 
@@ -281,7 +282,7 @@ int hgc_push_knn(const float *d_weights, const float *d_feat, const int *d_idxs,
     // out[m, f] = sum over (v, n) naming m of feat[v, f] * w[v, n]: the mean-only
     // feature gradient of the accumulation with `feat` as upstream gradient, not divided by K
     return accumulate_gradient(d_feat, d_weights, nullptr, nullptr, nullptr, nullptr, d_inv_offsets, d_inv_slots,
-                               nullptr, d_out_feat, n_vert, n_neigh, n_feat, n_feat, 0, 1.f, nullptr, stream);
+                               nullptr, d_out_feat, n_vert, n_neigh, n_feat, n_feat, 0, 1.f, nullptr, nullptr, 0, stream);
 }
 
 int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *d_feat, const int *d_idxs,
@@ -304,7 +305,7 @@ int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *
     // w_grad[v, n] = sum_f grad[idx[v,n], f] * feat[v, f]: the weight gradient with the roles of the
     // vertex's own row (feat) and the gathered rows (grad) as in the accumulation's
     return accumulate_gradient(d_feat, nullptr, d_grad, nullptr, nullptr, d_idxs, nullptr, nullptr, d_w_grad, nullptr,
-                               n_vert, n_neigh, n_feat, n_feat, 0, 1.f, nullptr, stream);
+                               n_vert, n_neigh, n_feat, n_feat, 0, 1.f, nullptr, nullptr, 0, stream);
 }
 
 int hgc_exp_neg(const float *d_distances, float *d_weights, long long n_values, hgc_stream_t stream) {

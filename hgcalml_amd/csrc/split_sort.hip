@@ -230,9 +230,11 @@ __global__ __launch_bounds__(sort_waves(LO_BITS) * kWave) void tile_sort_kernel(
     if (wave == 0) {  // exclusive scan of the run lengths over the tile's keys
         int carry = 0;
         for (int t0 = 0; t0 < T; t0 += kWave) {
-            const int len = s_total[t0 + lane];
+            // a tile of fewer keys than the wave has lanes (T = 32): the lanes beyond it stay out of the table
+            const bool in_table = t0 + lane < T;
+            const int len = in_table ? s_total[t0 + lane] : 0;
             const int incl = wave_inclusive_sum(len);
-            s_total[t0 + lane] = carry + incl - len;
+            if (in_table) s_total[t0 + lane] = carry + incl - len;
             carry += readlane_i32(incl, kWave - 1);
         }
     }

@@ -411,6 +411,15 @@ def _accumulate_backward(grad_from_out_features, distances, features, neigh_indi
         max_slots = None
     gw = torch.empty((n, k), dtype=torch.float32, device=dev)
     gx = torch.empty((n, f), dtype=torch.float32, device=dev)
+    # with the slot table: one record per (vertex, slot) in scratch memory carries the max part to the gather
+    need = lib.hgc_accumulate_knn_grad_records_workspace_bytes(n, k, f, int(mean_and_max)) \
+        if (max_slots is not None and gl.acc_grad_hit_records) else 0
+    if need:
+        ws = workspace(need, dev)
+        check(lib.hgc_accumulate_knn_grad_records(p(g), p(w), p(x), p(mi), p(max_slots), p(idx), p(inv_offsets),
+                                                  p(inv_slots), p(vertex_order_of(neigh_indices)), p(gw), p(gx), n, k,
+                                                  f, g.shape[1], 0, int(mean_and_max), p(ws), ws.numel(), stream()))
+        return gw, gx
     check(lib.hgc_accumulate_knn_grad_slots(p(g), p(w), p(x), p(mi), p(max_slots), p(idx), p(inv_offsets),
                                             p(inv_slots), p(vertex_order_of(neigh_indices)), p(gw), p(gx), n, k, f,
                                             g.shape[1], 0, int(mean_and_max), stream()))

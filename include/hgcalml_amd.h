@@ -332,6 +332,31 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
                                   int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
                                   int n_moments, int mean_and_max, hgc_stream_t stream);
 
+/* hgc_accumulate_knn_grad_slots with scratch memory for one 32-byte record per
+ * (vertex, slot): a streaming pass over the vertices first collects, for every
+ * slot, the weight, which features have their maximum there (from d_max_slots)
+ * and their upstream gradients; the gather over the inverse index then reads
+ * one record per entry instead of a weight, a line of slot bytes and scattered
+ * pieces of the max half of the gradient row. Same results as
+ * hgc_accumulate_knn_grad_slots (feature gradient bit for bit; the weight
+ * gradient's max part is added after the mean part instead of inside it). Has
+ * no counterpart in the reference. The workspace query returns 0 for shapes the
+ * record pass does not cover (n_feat outside 16..256 or above 2*n_neigh,
+ * n_neigh > 254, gradient matrix of 4 GiB or more, !mean_and_max); the call
+ * then behaves exactly like hgc_accumulate_knn_grad_slots and accepts a NULL
+ * workspace, as it does when d_max_slots is NULL. */
+size_t hgc_accumulate_knn_grad_records_workspace_bytes(int n_vert, int n_neigh, int n_feat,
+                                                       int mean_and_max);
+int hgc_accumulate_knn_grad_records(const float *d_grad_from_out_features, const float *d_distances,
+                                    const float *d_feat, const int *d_max_feat_indices,
+                                    const unsigned char *d_max_slots, const int *d_neigh_indices,
+                                    const int *d_inv_offsets, const int *d_inv_slots,
+                                    const int *d_vertex_order,
+                                    float *d_out_grad_distances, float *d_out_grad_features,
+                                    int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
+                                    int n_moments, int mean_and_max,
+                                    void *workspace, size_t workspace_bytes, hgc_stream_t stream);
+
 /* ------------------------------------------------------------------ */
 /* Ops over the same neighbour table, either side of the accumulation  */
 /* ------------------------------------------------------------------ */
