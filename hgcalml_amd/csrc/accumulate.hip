@@ -37,6 +37,7 @@ int launch_accumulate_grad_fused(const float *g, const float *w, const float *fe
 // records built in `records`; returns 1 when the shape is not covered or the storage is
 // too small (accumulate_grad_records_bytes is 0 where the path does not apply).
 size_t accumulate_grad_records_bytes(int n_vert, int K, int F);
+bool accumulate_grad_records_pays(int n_vert, int K, int F);
 int launch_accumulate_grad_records(const float *g, const float *w, const float *feat, const unsigned char *maxslot,
                                    const int *inv_off, const int *inv_slots, float *gw, float *gfeat, int n_vert, int K,
                                    int F, const int *idx, const int *order, float divisor, void *records,
@@ -125,6 +126,13 @@ __global__ __launch_bounds__(256) void accumulate_fwd_kernel(const float *__rest
                 if (sl > 0 && arg[e] == v) {  // repeated self reference: report its first slot
                     for (int n = 0; n < sl; ++n)
                         if (irow[n] == v) {
+                            sl = n;
+                            break;
+                        }
+                }
+                if (sl < 0) {  // no maximum: index 0 is reported, the slot that names vertex 0 is credited
+                    for (int n = 0; n < K; ++n)
+                        if (irow[n] == 0) {
                             sl = n;
                             break;
                         }
@@ -288,12 +296,27 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
             store_vec_i<VEC>(out_maxidx + (size_t)v * F + fb, argidx);
             if (out_maxslot) {
                 // slot of the maximum; for a repeated self reference its first slot,
-                // which is the one the reference's gradient credits
+                // which is the one the reference's gradient credits. A feature without a
+                // maximum (slot 0 empty, every product negative) reports index 0, and the
+                // reference's gradient compares indices: it credits the slot that names
+                // vertex 0, if the row has one.
+                bool none = false;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) none = none || arg[e] < 0;
+                int first_zero = -1;
+                if (__ballot(none) != 0) {  // wave-uniform, rare
+                    for (int n0z = 0; n0z < K && first_zero < 0; n0z += kWave) {
+                        const int n = n0z + lane_id();
+                        const uint64_t zero = __ballot(n < K && irow[min(n, K - 1)] == 0);
+                        if (zero != 0) first_zero = n0z + __builtin_ctzll(zero);
+                    }
+                }
                 uint32_t packed = 0;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     int sl = arg[e];
-                    if (sl >= 0 && argidx[e] == v) sl = first_self;
+                    if (sl < 0) sl = first_zero;
+                    else if (argidx[e] == v) sl = first_self;
                     packed |= (uint32_t)(sl < 0 ? 255 : sl) << (8 * e);
                 }
                 unsigned char *dst = out_maxslot + (size_t)v * F + fb;
@@ -1010,6 +1033,10 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
 
 size_t hgc_accumulate_knn_grad_records_workspace_bytes(int n_vert, int n_neigh, int n_feat, int mean_and_max) {
     return mean_and_max ? accumulate_grad_records_bytes(n_vert, n_neigh, n_feat) : 0;
+}
+
+int hgc_accumulate_knn_grad_records_pays(int n_vert, int n_neigh, int n_feat, int mean_and_max) {
+    return mean_and_max && accumulate_grad_records_pays(n_vert, n_neigh, n_feat) ? 1 : 0;
 }
 
 int hgc_accumulate_knn_grad_records(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,

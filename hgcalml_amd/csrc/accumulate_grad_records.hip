@@ -524,6 +524,14 @@ size_t accumulate_grad_records_bytes(int n_vert, int K, int F) {
     return align_up((size_t)n_vert * K * kRecordWords * sizeof(uint32_t));
 }
 
+// Where the record pass has measured faster than the gather with the slot table (MI355X; kNN
+// tables of 150 k vertices and banded tables of 1 M, K = 16..64, F = 32..128): slots that hold
+// two hits or fewer on average, and gathered rows that add up to more than the L2 caches keep
+// (below that the streaming pass costs more than the gather saves).
+bool accumulate_grad_records_pays(int n_vert, int K, int F) {
+    return accumulate_grad_records_bytes(n_vert, K, F) != 0 && F <= 2 * K && (long long)n_vert * F >= (12ll << 20);
+}
+
 // Returns 1 when the shape is not covered (the caller then takes another path).
 int launch_accumulate_grad_records(const float *g, const float *w, const float *feat, const unsigned char *maxslot,
                                    const int *inv_off, const int *inv_slots, float *gw, float *gfeat, int n_vert, int K,

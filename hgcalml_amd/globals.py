@@ -20,12 +20,14 @@ not depend on it, the run time does); when set, the search bins exactly as the
 reference would: `n_bins` (or its default formula, which reads the first event's
 size) over `max_bin_dims` dimensions.
 
-`acc_grad_hit_records` (no counterpart): the accumulation's gradient first builds
-one 32-byte record per (vertex, slot) in scratch memory (N*K*32 bytes) that hands
-the max part to the gather pass. Switch it off to save that memory; the results
+`acc_grad_hit_records` (no counterpart): the accumulation's gradient can first
+build one 32-byte record per (vertex, slot) in scratch memory (N*K*32 bytes) that
+hands the max part to the gather pass. None: where the library says it pays (wide
+rows of large tables); True: wherever the shape allows; False: never. The results
 are the same (the weight gradient to the last bits of its tolerance)."""
+
 knn_ops_use_tf_gradients = False
 acc_ops_use_tf_gradients = False
 debug_checks = False
 knn_callers_grid = False
-acc_grad_hit_records = True
+acc_grad_hit_records = None

@@ -412,8 +412,10 @@ def _accumulate_backward(grad_from_out_features, distances, features, neigh_indi
     gw = torch.empty((n, k), dtype=torch.float32, device=dev)
     gx = torch.empty((n, f), dtype=torch.float32, device=dev)
     # with the slot table: one record per (vertex, slot) in scratch memory carries the max part to the gather
-    need = lib.hgc_accumulate_knn_grad_records_workspace_bytes(n, k, f, int(mean_and_max)) \
-        if (max_slots is not None and gl.acc_grad_hit_records) else 0
+    need = 0
+    if max_slots is not None and gl.acc_grad_hit_records is not False:
+        if gl.acc_grad_hit_records or lib.hgc_accumulate_knn_grad_records_pays(n, k, f, int(mean_and_max)):
+            need = lib.hgc_accumulate_knn_grad_records_workspace_bytes(n, k, f, int(mean_and_max))
     if need:
         ws = workspace(need, dev)
         check(lib.hgc_accumulate_knn_grad_records(p(g), p(w), p(x), p(mi), p(max_slots), p(idx), p(inv_offsets),

@@ -259,9 +259,11 @@ int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int 
                        int n_moments, int mean_and_max, hgc_stream_t stream);
 
 /* hgc_accumulate_knn that also reports, as one byte per (vertex, feature), the
- * neighbour SLOT that attained the maximum (255: none; for a repeated self
- * reference the first slot naming the vertex, which is the one the reference's
- * gradient credits). Has no counterpart in the reference, which re-derives the
+ * neighbour SLOT that attained the maximum (for a repeated self reference the
+ * first slot naming the vertex, which is the one the reference's gradient
+ * credits; where no slot attained it -- slot 0 empty and every product
+ * negative -- the reference reports index 0 and its gradient credits the slot
+ * that names vertex 0, so that slot is reported, 255 if the row has none). Has no counterpart in the reference, which re-derives the
  * slot in the gradient by comparing indices; it exists so that the gradient
  * gathers 1 byte instead of 4 per (neighbour, feature). Needs n_neigh <= 254
  * and, like the reference, indices that are unique in a row apart from
@@ -341,12 +343,16 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
  * hgc_accumulate_knn_grad_slots (feature gradient bit for bit; the weight
  * gradient's max part is added after the mean part instead of inside it). Has
  * no counterpart in the reference. The workspace query returns 0 for shapes the
- * record pass does not cover (n_feat outside 16..256 or above 2*n_neigh,
- * n_neigh > 254, gradient matrix of 4 GiB or more, !mean_and_max); the call
- * then behaves exactly like hgc_accumulate_knn_grad_slots and accepts a NULL
- * workspace, as it does when d_max_slots is NULL. */
+ * record pass does not cover (n_feat outside 16..128, n_neigh > 254, gradient
+ * matrix of 4 GiB or more, !mean_and_max); the call then behaves exactly like
+ * hgc_accumulate_knn_grad_slots and accepts a NULL workspace, as it does when
+ * d_max_slots is NULL. hgc_accumulate_knn_grad_records_pays says where the
+ * record pass has measured faster (n_feat <= 2 n_neigh and n_vert * n_feat of
+ * 12 Mi elements or more: cfg4 5.8 -> 5.2 ms); elsewhere
+ * hgc_accumulate_knn_grad_slots is the better call. */
 size_t hgc_accumulate_knn_grad_records_workspace_bytes(int n_vert, int n_neigh, int n_feat,
                                                        int mean_and_max);
+int hgc_accumulate_knn_grad_records_pays(int n_vert, int n_neigh, int n_feat, int mean_and_max);
 int hgc_accumulate_knn_grad_records(const float *d_grad_from_out_features, const float *d_distances,
                                     const float *d_feat, const int *d_max_feat_indices,
                                     const unsigned char *d_max_slots, const int *d_neigh_indices,

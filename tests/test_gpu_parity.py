@@ -7,6 +7,8 @@ gradient bit-exact (same fp32 operation order); the weight gradient within
 1e-5 relative to the magnitude of the summed terms (its dot products are
 reduced in a different order than the oracle's serial loop).
 """
+import contextlib
+
 import numpy as np
 import pytest
 import torch
@@ -305,6 +307,18 @@ def test_knn_result_does_not_depend_on_the_grid(oracle, C, K, n_events):
 
 # ------------------------------------------------------------------ accumulate
 
+@contextlib.contextmanager
+def hit_records(on):
+    """forces the record pass of the accumulation's gradient on or off (the default decides by shape)"""
+    import hgcalml_amd.globals as gl
+    before = gl.acc_grad_hit_records
+    gl.acc_grad_hit_records = on
+    try:
+        yield
+    finally:
+        gl.acc_grad_hit_records = before
+
+
 def make_acc_case(rng, n, K, F, holes=True):
     x = rng.standard_normal((n, F)).astype(np.float32)
     idx = np.stack([np.concatenate([[v], rng.permutation(np.delete(np.arange(n), v))[:K - 1]])
@@ -406,14 +420,110 @@ def test_accumulate_slot_table_path(oracle, K, F):
     assert (sl[n // 2 + 2] == 255).all()      # a row without any neighbour
     rgw, rgx = oracle.accumulate_knn_grad_kernel(g, w, x, idx, rarg)
     inv = ops.inverse_neighbour_index(t(idx))
-    gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(g), t(w), t(x), t(idx), arg, slots, *inv)
     gw0, gx0 = torch.ops.hgcalml.accumulate_knn_grad(t(g), t(w), t(x), t(idx), arg, *inv)
-    assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
-    assert torch.equal(gx, gx0)
-    # the two paths reduce the weight gradient's dot products in different orders
     tol = grad_tolerance(g, x, idx, w, K)
-    assert (np.abs(gw.cpu().numpy() - rgw) <= tol).all() and (np.abs(gw0.cpu().numpy() - rgw) <= tol).all()
-    assert (gw.cpu().numpy()[idx < 0] == 0).all()
+    assert (np.abs(gw0.cpu().numpy() - rgw) <= tol).all()
+    # with the slot table: the gather that compares slot bytes, and the one that reads per-slot hit records
+    for records in (False, True):
+        with hit_records(records):
+            gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(g), t(w), t(x), t(idx), arg, slots, *inv)
+        assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
+        assert torch.equal(gx, gx0)
+        # the paths reduce the weight gradient's dot products in different orders
+        assert (np.abs(gw.cpu().numpy() - rgw) <= tol).all()
+        assert (gw.cpu().numpy()[idx < 0] == 0).all()
+
+
+@pytest.mark.parametrize("K,F", [(64, 128), (64, 64), (6, 128), (8, 64), (20, 100), (254, 96), (33, 17), (12, 48), (3, 16)])
+def test_accumulate_gradient_hit_records(oracle, K, F):
+    """The gradient whose max part travels in per-slot records, on the cases that decide which kind of
+    record a slot gets: slots with exactly five and six hits (listed / one bit per feature), a slot
+    that holds every maximum of its vertex, a vertex without any, repeated self references whose first
+    slot is of either kind, -1 tails, a missing slot 0, rows of fewer features than a wave has lanes,
+    K that is no power of two. Feature gradient bitwise, weight gradient within the stated tolerance,
+    against the oracle and against the slot-byte gather."""
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(700 + K + F)
+    n = 260
+    d, x, idx = make_acc_case(rng, n, K, F)
+    w = np.exp(-d).astype(np.float32)
+    x = np.abs(x) + np.float32(0.1)            # all positive: a slot's weight decides where the maxima go
+    # vertex 3: slot 1 takes every maximum; vertex 4: slot 2 takes exactly five, slot 1 six (if there are enough features)
+    w[3, :] = 1e-6
+    w[3, min(1, K - 1)] = 1e9
+    if K >= 3 and F >= 12:
+        w[4, :] = 1e-9
+        w[4, 1:3] = 1.0
+        x[idx[4, 2], :5] = 1e12                 # slot 2 wins features 0..4
+        x[idx[4, 1], 5:11] = 1e12               # slot 1 wins features 5..10
+    # vertex 5: repeated self references, self wins everything (first self slot: all hits, one bit per feature)
+    idx[5, K // 2:] = 5
+    x[5] = 1e4
+    # vertex 6: repeated self references, self wins two features only (listed record)
+    idx[6, 1:1 + max(1, K // 3)] = 6
+    x[6] = 1e-3
+    x[6, :2] = 2e4
+    # vertex 8: nothing wins (slot 0 missing, every product negative)
+    idx[8, 0] = -1
+    w[8, :] = -1.0
+    x_neg = x
+    out, arg, slots = torch.ops.hgcalml.accumulate_knn_slots(t(w), t(x_neg), t(idx), 0, True)
+    ref, rarg = oracle.AccumulateLinKnn(w, x_neg, idx)
+    assert (bits(out.cpu().numpy()) == bits(ref)).all() and (arg.cpu().numpy() == rarg).all()
+    sl = slots.cpu().numpy()
+    assert (sl[3] == min(1, K - 1)).all()
+    # nothing wins in row 8: index 0 is reported and the slot that names vertex 0 (if any) is credited
+    names_zero = np.nonzero(idx[8] == 0)[0]
+    assert (rarg[8] == 0).all() and (sl[8] == (names_zero[0] if len(names_zero) else 255)).all()
+    if K >= 3 and F >= 12:
+        assert (sl[4, :5] == 2).all() and (sl[4, 5:11] == 1).all()
+    g = rng.standard_normal((n, 2 * F)).astype(np.float32)
+    rgw, rgx = oracle.accumulate_knn_grad_kernel(g, w, x_neg, idx, rarg)
+    inv = ops.inverse_neighbour_index(t(idx))
+    tol = grad_tolerance(g, x_neg, idx, w, K)
+    with hit_records(False):
+        gw0, gx0 = torch.ops.hgcalml.accumulate_knn_grad_slots(t(g), t(w), t(x_neg), t(idx), arg, slots, *inv)
+    for _ in range(2):      # twice: the scratch records of the first call are overwritten by the second
+        with hit_records(True):
+            gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(g), t(w), t(x_neg), t(idx), arg, slots, *inv)
+        assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
+        assert torch.equal(gx, gx0)
+        assert (np.abs(gw.cpu().numpy() - rgw) <= tol).all()
+        assert (gw.cpu().numpy()[idx < 0] == 0).all()
+
+
+def test_accumulate_gradient_hit_records_workspace_rules():
+    """the C entry point: workspace sizes, where the record pass applies and where it pays, refusal of a
+    workspace that is too small, and the fall-back to the slot-byte gather where it does not apply"""
+    from hgcalml_amd._lib import lib
+    assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 64, 128, 1) == 1000 * 64 * 32
+    assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 64, 128, 0) == 0      # mean only: nothing to record
+    assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 255, 128, 1) == 0     # slots are bytes
+    assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 64, 192, 1) == 0      # rows beyond 128 features
+    assert lib.hgc_accumulate_knn_grad_records_pays(1000000, 64, 128, 1) == 1
+    assert lib.hgc_accumulate_knn_grad_records_pays(150000, 64, 64, 1) == 0
+    assert lib.hgc_accumulate_knn_grad_records_pays(1000000, 16, 128, 1) == 0
+    from hgcalml_amd import ops
+    from hgcalml_amd._lib import p, stream
+    rng = np.random.default_rng(5)
+    n, K, F = 200, 16, 32
+    d, x, idx = make_acc_case(rng, n, K, F)
+    w = np.exp(-d).astype(np.float32)
+    g = t(rng.standard_normal((n, 2 * F)).astype(np.float32))
+    tw, tx, ti = t(w), t(x), t(idx)
+    out, arg, slots = torch.ops.hgcalml.accumulate_knn_slots(tw, tx, ti, 0, True)
+    inv = ops.inverse_neighbour_index(ti)
+    gw, gx = torch.empty((n, K), device="cuda"), torch.empty((n, F), device="cuda")
+    small = torch.empty(256, dtype=torch.uint8, device="cuda")
+    rc = lib.hgc_accumulate_knn_grad_records(p(g), p(tw), p(tx), p(arg), p(slots), p(ti), p(inv[0]), p(inv[1]), None, p(gw),
+                                             p(gx), n, K, F, 2 * F, 0, 1, p(small), small.numel(), stream())
+    assert rc == -2 and b"workspace" in lib.hgc_last_error()
+    # without a slot table there is nothing to build records from: same call as hgc_accumulate_knn_grad
+    rc = lib.hgc_accumulate_knn_grad_records(p(g), p(tw), p(tx), p(arg), None, p(ti), p(inv[0]), p(inv[1]), None, p(gw),
+                                             p(gx), n, K, F, 2 * F, 0, 1, None, 0, stream())
+    assert rc == 0
+    gw0, gx0 = torch.ops.hgcalml.accumulate_knn_grad(g, tw, tx, ti, arg, *inv)
+    assert torch.equal(gx, gx0) and torch.equal(gw, gw0)
 
 
 def test_inverse_neighbour_index_is_ordered():
@@ -617,6 +727,41 @@ def test_accumulate_cfg4_full_size_slot_kernels_vs_oracle(oracle, capsys):
         print("\ncfg4 N=1M weight gradient, 32000 rows x 64 slots: worst |error| / sum|terms| = %.2e, "
               "worst |error| / |value| (|value| > 1e-3) = %.2e" % (worst_scaled, worst_rel))
     assert worst_rel < 1e-3
+
+
+def test_accumulate_cfg4_full_size_all_rows_vs_oracle(oracle, capsys):
+    """cfg4 at its full size, every one of the 1,000,000 rows against the oracle: forward (with the arg-max
+    slot table) and arg-max indices bitwise; the gradient through both gathers that use the slot table
+    (slot-byte compares; per-slot hit records, the one bench.py times): feature gradient bitwise, weight
+    gradient within 1e-5 of the sum of the magnitudes of its terms."""
+    from hgcalml_amd import ops
+    c = workloads.cfg4()
+    n, K, F = len(c["indices"]), c["K"], c["F"]
+    w = np.exp(-c["distsq"]).astype(np.float32)
+    ref, rarg = oracle.accumulate_knn_kernel(w, c["features"], c["indices"])
+    rgw, rgx = oracle.accumulate_knn_grad_kernel(c["grad_out"], w, c["features"], c["indices"], rarg)
+    tw, tx, ti, tg = t(w), t(c["features"]), t(c["indices"]), t(c["grad_out"])
+    out, arg, slots = torch.ops.hgcalml.accumulate_knn_slots(tw, tx, ti, 0, True)
+    assert (bits(out.cpu().numpy()) == bits(ref)).all()
+    assert (arg.cpu().numpy() == rarg).all()
+    del out, ref
+    inv = ops.inverse_neighbour_index(ti)
+    # tolerance of the weight gradient, in blocks (the gathered |features| of all rows at once would be 32 GB)
+    tol = np.empty((n, K), np.float32)
+    for s0 in range(0, n, 50000):
+        s1 = min(n, s0 + 50000)
+        tol[s0:s1] = grad_tolerance(c["grad_out"][s0:s1], c["features"], c["indices"][s0:s1], w[s0:s1], K)
+    worst = {}
+    for records in (False, True):
+        with hit_records(records):
+            gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(tg, tw, tx, ti, arg, slots, *inv)
+        assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
+        err = np.abs(gw.cpu().numpy() - rgw)
+        assert (err <= tol).all()
+        worst[records] = float((err / tol).max()) * 1e-5
+    with capsys.disabled():
+        print("\ncfg4 N=1M, all rows: weight gradient worst |error| / sum|terms| = %.2e (slot-byte gather), %.2e "
+              "(hit records)" % (worst[False], worst[True]))
 
 
 def test_cfg2_full_size_accumulate_in_bin_order_vs_oracle(oracle):

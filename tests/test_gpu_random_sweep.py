@@ -65,7 +65,13 @@ def test_random_configuration(oracle, seed):
                 assert (arg.cpu().numpy() == ra).all()
             gg = g if mm else g[:, :F].copy()
             rgw, rgx = oracle.accumulate_knn_grad_kernel(gg, w, x, gi, ra)
-            gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(gg), t(w), t(x), idx, arg, slots, *inv)
+            # the gather fed by per-slot hit records in half of the configurations (it applies up to 128 features)
+            import hgcalml_amd.globals as gl
+            gl.acc_grad_hit_records = bool(seed % 2)
+            try:
+                gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(t(gg), t(w), t(x), idx, arg, slots, *inv)
+            finally:
+                gl.acc_grad_hit_records = None
             assert (bits(gx.cpu().numpy()) == bits(rgx)).all()
             gm = np.abs(gg[:, :F]) / K + (np.abs(gg[:, F:]) if mm else 0)
             scale = (np.abs(x[np.maximum(gi, 0)]) * gm[:, None, :]).sum(-1)
