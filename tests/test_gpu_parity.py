@@ -199,6 +199,16 @@ def test_knn_cfg3_full_size_properties(oracle):
     assert check_knn_rows(oracle, i, d, c["coords"], c["row_splits"], c["K"], rows, radius=c["max_radius"]) == 0
 
 
+def test_knn_cfg3_full_size_all_rows_vs_oracle(oracle):
+    """cfg3 at its full size (16 ragged events, ~1.14 M points, K=32, radius 0.1): every row against the
+    oracle's binned search followed by the radius rule -- indices and distances bitwise in canonical order;
+    a row that differs must be an exact tie at the K-th boundary and a valid neighbour set (one row of
+    the 1.14 M is: two candidates at bitwise the same distance, the oracle keeps the one its walk meets
+    first, the library the lower index)"""
+    c = workloads.cfg3()
+    run_knn_case(oracle, c["coords"], c["row_splits"], c["K"], c["n_bins"], max_radius=c["max_radius"], max_ties=4)
+
+
 @pytest.mark.parametrize("C,B", [(2, 2), (3, 3), (3, 2), (4, 3), (5, 3), (6, 3), (7, 3), (8, 3), (9, 3), (6, 4), (5, 5)])
 def test_knn_dimensions(oracle, C, B):
     from hgcalml_amd import BinnedSelectKnn
