@@ -21,6 +21,7 @@ _SIGNATURES = {
     "hgc_version": (_c_int, []),
     "hgc_last_error": (ctypes.c_char_p, []),
     "hgc_set_status_word": (_c_int, [_ptr]),
+    "hgc_get_status_word": (_ptr, []),
     "hgc_bin_by_coordinates_total_bins": (_c_int, [_ptr, _c_int, _c_int, _ptr]),
     "hgc_bin_by_coordinates": (_c_int, [_ptr] * 7 + [_c_int] * 5 + [_ptr]),
     "hgc_bin_by_coordinates_strided": (_c_int, [_ptr, _c_int] + [_ptr] * 8 + [_c_int] * 5 + [_ptr]),
@@ -32,6 +33,7 @@ _SIGNATURES = {
     "hgc_binned_select_knn": (_c_int, [_ptr] * 9 + [_c_int] * 7 + [_ptr]),
     "hgc_binned_select_knn_fused": (_c_int, [_ptr] * 9 + [_c_float] + [_ptr] * 2 + [_c_int] * 7 + [_ptr]),
     "hgc_set_knn_grid": (_c_int, [_c_int]),
+    "hgc_get_knn_grid": (_c_int, []),
     "hgc_sort_distinct_keys_workspace_bytes": (_c_size, [ctypes.c_longlong]),
     "hgc_sort_distinct_keys": (_c_int, [_ptr, ctypes.c_longlong, _c_int, _ptr, _ptr, _c_size, _c_int, _ptr]),
     "hgc_binned_select_knn_pipeline_workspace_bytes": (_c_size, [_c_int] * 6),

@@ -513,6 +513,8 @@ int hgc_set_status_word(int *d_word) {
     return HGC_OK;
 }
 
+int *hgc_get_status_word(void) { return hgc::g_status_word; }
+
 const char *hgc_last_error(void) { return hgc::last_error_buffer(); }
 
 int hgc_bin_by_coordinates_total_bins(const int *h_n_bins, int n_nbins, int n_rs, int *h_out_total_bins) {

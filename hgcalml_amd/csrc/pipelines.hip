@@ -398,6 +398,8 @@ int hgc_set_knn_grid(int use_callers_grid) {
     return HGC_OK;
 }
 
+int hgc_get_knn_grid(void) { return g_callers_knn_grid; }
+
 size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, int n_rs, int n_bins_scalar,
                                                       int max_bin_dims, int use_direction) {
     const SearchGrid asked = callers_grid(n_coords, n_bins_scalar, max_bin_dims);

@@ -609,3 +609,95 @@ def exp_neg_grad(weight_grad, weights):
     check(lib.hgc_exp_neg_grad(p(g), p(w), p(out), w.numel(), stream()))
     return out
 
+
+# --------------------------------------------------------------------------- shapes without data
+
+# Fake ("meta") implementations: output shapes and dtypes from input shapes alone, so that
+# torch.compile / torch.export can trace through the ops without running a kernel.
+
+def _i32_like(shape, ref):
+    return ref.new_empty(shape, dtype=torch.int32)
+
+
+def _f32_like(shape, ref):
+    return ref.new_empty(shape, dtype=torch.float32)
+
+
+@bin_by_coordinates.register_fake
+def _(coordinates, row_splits, bin_width, nbins, n_total_bins, calc_n_per_bin):
+    n, c = coordinates.shape
+    return _i32_like((n, c + 1), coordinates), _i32_like((n,), coordinates), _i32_like((n_total_bins,), coordinates)
+
+
+@binned_select_knn.register_fake
+def _(coords, bin_idx, dim_bin_idx, bin_boundaries, n_bins, bin_width, direction, n_neighbours, tf_compatible,
+      use_direction):
+    n = coords.shape[0]
+    return _i32_like((n, n_neighbours), coords), _f32_like((n, n_neighbours), coords)
+
+
+@index_replacer.register_fake
+def _(to_be_replaced, replacements):
+    return _i32_like(to_be_replaced.shape, to_be_replaced)
+
+
+def _accumulate_shapes(features, indices, mean_and_max):
+    n, f = features.shape
+    return _f32_like((n, 2 * f if mean_and_max else f), features), _i32_like((n, f), features)
+
+
+@accumulate_knn.register_fake
+def _(distances, features, indices, n_moments, mean_and_max):
+    return _accumulate_shapes(features, indices, mean_and_max)
+
+
+@accumulate_knn_slots.register_fake
+def _(distances, features, indices, n_moments, mean_and_max):
+    out, maxidx = _accumulate_shapes(features, indices, mean_and_max)
+    n, f = features.shape
+    with_slots = mean_and_max and indices.shape[1] <= 254
+    return out, maxidx, features.new_empty((n, f) if with_slots else (0,), dtype=torch.uint8)
+
+
+def _accumulate_grad_shapes(features, neigh_indices):
+    return _f32_like(neigh_indices.shape, features), _f32_like(features.shape, features)
+
+
+@accumulate_knn_grad.register_fake
+def _(grad_from_out_features, distances, features, neigh_indices, max_feat_indices, inv_offsets, inv_slots):
+    return _accumulate_grad_shapes(features, neigh_indices)
+
+
+@accumulate_knn_grad_slots.register_fake
+def _(grad_from_out_features, distances, features, neigh_indices, max_feat_indices, max_slots, inv_offsets,
+      inv_slots):
+    return _accumulate_grad_shapes(features, neigh_indices)
+
+
+@select_knn_grad.register_fake
+def _(grad_distances, indices, distances, coordinates):
+    return _f32_like(coordinates.shape, coordinates)
+
+
+@local_distance.register_fake
+def _(coordinates, neighbour_idxs):
+    return _f32_like(neighbour_idxs.shape, coordinates)
+
+
+@push_knn.register_fake
+def _(weights, features, indices):
+    return _f32_like(features.shape, features)
+
+
+@push_knn_grad.register_fake
+def _(grad, weights, features, indices):
+    return _f32_like(weights.shape, features), _f32_like(features.shape, features)
+
+
+@binned_assign_to_condensates.register_fake
+def _(ccoords, dist, beta, no_condensation_mask, bins_flat, bin_splits, indices_to_filtered, original_indices,
+      row_splits, n_bins, bin_widths, ccoords_h, dist_h, beta_h, no_condensation_mask_h, row_splits_h, beta_threshold,
+      assign_by_max_beta):
+    n, nh, rows = ccoords.shape[0], beta_h.numel(), row_splits.numel() - 1
+    return (_i32_like((nh,), ccoords), _i32_like((n,), ccoords), _i32_like((nh,), ccoords), _i32_like((n,), ccoords),
+            _i32_like((rows + 1,), ccoords))

@@ -13,8 +13,14 @@
  *     work is enqueued on it; no call synchronises the device.
  *   - Return value: 0 on success, a negative hgc_status otherwise. Argument
  *     errors are detected on the host before anything is launched.
- *   - The library is stateless and re-entrant; calls that share output or
- *     workspace buffers must be ordered by the caller.
+ *   - The library keeps no state between calls except three per-THREAD
+ *     settings: the text of the last error (hgc_last_error), the device status
+ *     word (hgc_set_status_word) and the choice of the kNN search grid
+ *     (hgc_set_knn_grid). A setting made on one thread is not seen by calls made
+ *     on another (e.g. by an autograd engine's backward threads): set it on the
+ *     thread that makes the call, as the Python wrappers do right before each
+ *     call. Calls are re-entrant; calls that share output or workspace buffers
+ *     must be ordered by the caller.
  *
  * Each entry point names the reference interface it replaces (paths relative
  * to the HGCalML tree). The reference boundary is the functor
@@ -68,6 +74,8 @@ enum hgc_data_flag {
                                              ((2d+1)^(n_bin_dim-1) at shell distance d) and ended there */
 };
 int hgc_set_status_word(int *d_word);
+/* The calling thread's status word (NULL: none registered on this thread). */
+int *hgc_get_status_word(void);
 
 /* ------------------------------------------------------------------ */
 /* Spatial binning                                                     */
@@ -205,6 +213,8 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
  * (n_bins_scalar bins over min(max_bin_dims, n_coords) dimensions),
  * hgc_set_knn_grid(0) returns to the default. The workspace query covers both. */
 int hgc_set_knn_grid(int use_callers_grid);
+/* The calling thread's setting (0: the library's own grid, the initial state). */
+int hgc_get_knn_grid(void);
 size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, int n_rs,
                                                       int n_bins_scalar, int max_bin_dims,
                                                       int use_direction);

@@ -5,8 +5,9 @@
 The expected outputs come from the CPU oracle (``oracle/``), whose functions are pinned by
 tests/test_oracle_pins.py against brute force, closed forms and float64 autograd. The reference's own
 kernels cannot be built in this image (they need the TensorFlow and CUDA runtime headers) and its test
-tree holds no numeric vectors for these ops, so these files are a frozen copy of a pinned oracle: they
-catch drift of the oracle and give the GPU tests data that does not depend on it. Seeds are fixed; the
+tree holds no numeric vectors for these ops, so these files are a frozen copy of this repository's own
+oracle: regression fixtures. They pin nothing independently of the oracle (tests/test_oracle_pins.py does
+that); they catch drift of the oracle and of the GPU path between commits. Seeds are fixed; the
 arrays of a second run are identical.
 """
 import os

@@ -99,6 +99,38 @@ def test_host_side_argument_checks(capi):
     assert h(one, 10, 10, one, one, null, 0, null) == -2
 
 
+def test_settings_are_per_thread(capi):
+    """the status word, the choice of the kNN grid and the last error text belong to the thread that set
+    them: another thread sees the initial state, and what it sets does not leak back"""
+    import threading
+    capi.hgc_get_status_word.restype = ctypes.c_void_p
+    capi.hgc_set_status_word.argtypes = [ctypes.c_void_p]
+    capi.hgc_last_error.restype = ctypes.c_char_p
+    assert capi.hgc_set_knn_grid(1) == 0 and capi.hgc_get_knn_grid() == 1
+    assert capi.hgc_set_status_word(ctypes.c_void_p(4096)) == 0 and capi.hgc_get_status_word() == 4096
+    nb = (ctypes.c_int * 1)(0)
+    out = ctypes.c_int(0)
+    assert capi.hgc_bin_by_coordinates_total_bins(nb, 1, 2, ctypes.byref(out)) == -1
+    mine = capi.hgc_last_error()
+    assert mine
+    seen = {}
+
+    def other():
+        seen["grid"] = capi.hgc_get_knn_grid()
+        seen["word"] = capi.hgc_get_status_word()
+        seen["error"] = capi.hgc_last_error()
+        capi.hgc_set_knn_grid(0)
+        capi.hgc_set_status_word(ctypes.c_void_p(8192))
+
+    th = threading.Thread(target=other)
+    th.start()
+    th.join()
+    assert seen == {"grid": 0, "word": None, "error": b""}
+    assert capi.hgc_get_knn_grid() == 1 and capi.hgc_get_status_word() == 4096 and capi.hgc_last_error() == mine
+    capi.hgc_set_knn_grid(0)
+    capi.hgc_set_status_word(None)
+
+
 def test_package_refuses_cpu_tensors(capi):
     import torch
     from hgcalml_amd import AccumulateLinKnn
