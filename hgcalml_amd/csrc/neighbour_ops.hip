@@ -243,9 +243,141 @@ __global__ __launch_bounds__(256) void exp_neg_grad_kernel(const float *__restri
     }
 }
 
+
+// ---- feature-weighted moments of the neighbours' coordinates ----------------------
+//
+// modules/neighbour_covariance_op.py:8-62 builds, with w = exp(-distsq) and a = the
+// (activated) features,
+//   S[v,f]       = sum_n w[v,n] a[j,f]
+//   mean[v,f,c]  = sum_n w[v,n] a[j,f] x[j,c] / (S[v,f] + 1e-3)
+//   cov[v,f,c,d] = sum_n w[v,n] a[j,f] (x[j,c] - mean[j,f,c]) (x[j,d] - mean[j,f,d]) / (S[v,f] + 1e-3)
+// (j = idx[v,n]; every neighbour is centred on ITS OWN mean) out of three mean-only
+// accumulations over matrices of F, F*C and F*C*C columns that it materialises first.
+// Here two passes over the neighbour table do it, one thread per (vertex, feature): the
+// first gathers a[j,f] and x[j,:], the second a[j,f], x[j,:] and mean[j,f,:] and forms the
+// C*C products in registers. The sums run over the slots in order and every term is formed
+// as the composition forms it -- ((x*a)*w, ((cen_c*cen_d)*a)*w, the sum divided by K and
+// multiplied by K again as the accumulation's mean is) -- so the results are its bits.
+
+__device__ __forceinline__ float divide_no_nan(float a, float b) { return b == 0.f ? 0.f : a / b; }
+
+template <int C>
+__global__ __launch_bounds__(256) void neighbour_means_kernel(const float *__restrict__ coords,
+                                                              const float *__restrict__ weights,
+                                                              const float *__restrict__ feats, const int *__restrict__ idx,
+                                                              float *__restrict__ sumw, float *__restrict__ means,
+                                                              const int *__restrict__ order, int n_vert, int n_feat,
+                                                              int n_neigh) {
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int i = (int)(t / n_feat);
+    if (i >= n_vert) return;
+    const int f = (int)(t - (long long)i * n_feat);
+    const int v = order ? order[i] : i;  // processing order with locality: results do not depend on it
+    if ((unsigned)v >= (unsigned)n_vert) return;
+    const float kf = (float)n_neigh;
+    float s = 0.f, sc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) sc[c] = 0.f;
+    for (int n = 0; n < n_neigh; ++n) {
+        const int j = idx[(size_t)v * n_neigh + n];
+        if ((unsigned)j >= (unsigned)n_vert) continue;
+        const float w = weights[(size_t)v * n_neigh + n];
+        const float a = feats[(size_t)j * n_feat + f];
+        s = s + a * w;
+#pragma unroll
+        for (int c = 0; c < C; ++c) sc[c] = sc[c] + (coords[(size_t)j * C + c] * a) * w;
+    }
+    const float S = (s / kf) * kf;
+    sumw[(size_t)v * n_feat + f] = S;
+#pragma unroll
+    for (int c = 0; c < C; ++c) means[((size_t)v * n_feat + f) * C + c] = divide_no_nan((sc[c] / kf) * kf, S + 1e-3f);
+}
+
+template <int C>
+__global__ __launch_bounds__(256) void neighbour_covariance_kernel(const float *__restrict__ coords,
+                                                                   const float *__restrict__ weights,
+                                                                   const float *__restrict__ feats,
+                                                                   const int *__restrict__ idx,
+                                                                   const float *__restrict__ sumw,
+                                                                   const float *__restrict__ means, float *__restrict__ cov,
+                                                                   const int *__restrict__ order, int n_vert, int n_feat,
+                                                                   int n_neigh) {
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int i = (int)(t / n_feat);
+    if (i >= n_vert) return;
+    const int f = (int)(t - (long long)i * n_feat);
+    const int v = order ? order[i] : i;
+    if ((unsigned)v >= (unsigned)n_vert) return;
+    const float kf = (float)n_neigh;
+    float acc[C][C];  // the lower triangle is accumulated, the products are symmetric bit for bit
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int d = 0; d < C; ++d) acc[c][d] = 0.f;
+    for (int n = 0; n < n_neigh; ++n) {
+        const int j = idx[(size_t)v * n_neigh + n];
+        if ((unsigned)j >= (unsigned)n_vert) continue;
+        const float w = weights[(size_t)v * n_neigh + n];
+        const float a = feats[(size_t)j * n_feat + f];
+        float cen[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) cen[c] = coords[(size_t)j * C + c] - means[((size_t)j * n_feat + f) * C + c];
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int d = 0; d <= c; ++d) acc[c][d] = acc[c][d] + ((cen[c] * cen[d]) * a) * w;
+    }
+    const float den = sumw[(size_t)v * n_feat + f] + 1e-3f;
+    float *out = cov + ((size_t)v * n_feat + f) * C * C;
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int d = 0; d < C; ++d) out[c * C + d] = divide_no_nan((acc[c > d ? c : d][c > d ? d : c] / kf) * kf, den);
+}
+
+template <int C>
+int launch_neighbour_covariance(const float *coords, const float *weights, const float *feats, const int *idx, float *cov,
+                                float *means, float *sumw, const int *order, int n_vert, int n_feat, int n_neigh,
+                                hipStream_t s) {
+    const int blocks = ceil_div((long long)n_vert * n_feat, 256);
+    neighbour_means_kernel<C><<<blocks, 256, 0, s>>>(coords, weights, feats, idx, sumw, means, order, n_vert, n_feat,
+                                                     n_neigh);
+    int rc = check_launch("neighbour_means_kernel");
+    if (rc) return rc;
+    neighbour_covariance_kernel<C><<<blocks, 256, 0, s>>>(coords, weights, feats, idx, sumw, means, cov, order, n_vert,
+                                                          n_feat, n_neigh);
+    return check_launch("neighbour_covariance_kernel");
+}
+
 }  // namespace
 
 extern "C" {
+
+int hgc_neighbour_covariance(const float *d_coords, const float *d_weights, const float *d_feats, const int *d_n_idxs,
+                             const int *d_vertex_order, float *d_covariance, float *d_means, float *d_sum_weights,
+                             int n_vert, int n_coords, int n_feat, int n_neigh, hgc_stream_t stream) {
+    HGC_REQUIRE(n_vert >= 0 && n_coords >= 1 && n_feat >= 1 && n_neigh >= 1, "bad sizes");
+    if (n_coords > 6) return fail(HGC_ERR_UNSUPPORTED, "neighbour covariance is built for up to 6 coordinates");
+    HGC_REQUIRE((long long)n_vert * std::max(n_neigh, n_feat * n_coords * n_coords) < (1ll << 31),
+                "tensor too large for int32 indexing");
+    if (n_vert == 0) return HGC_OK;
+    HGC_REQUIRE(d_coords && d_weights && d_feats && d_n_idxs && d_covariance && d_means && d_sum_weights, "null pointer");
+    hipStream_t s = as_stream(stream);
+#define HGC_COV(C)                                                                                                  \
+    case C:                                                                                                         \
+        return launch_neighbour_covariance<C>(d_coords, d_weights, d_feats, d_n_idxs, d_covariance, d_means,        \
+                                              d_sum_weights, d_vertex_order, n_vert, n_feat, n_neigh, s)
+    switch (n_coords) {
+        HGC_COV(1);
+        HGC_COV(2);
+        HGC_COV(3);
+        HGC_COV(4);
+        HGC_COV(5);
+        HGC_COV(6);
+    }
+#undef HGC_COV
+    return HGC_ERR_UNSUPPORTED;
+}
 
 int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const float *d_dist, const float *d_coord,
                         const int *d_inv_offsets, const int *d_inv_slots, float *d_grad_coord, int n_vert, int n_neigh,

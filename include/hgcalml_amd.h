@@ -403,6 +403,31 @@ int hgc_local_distance(const int *d_neigh_idxs, const float *d_coords, float *d_
                        int n_coords, int n_in_vert, int n_out_vert, int n_neigh,
                        hgc_stream_t stream);
 
+/* Feature-weighted mean and covariance of the neighbours' coordinates, as the
+ * wrapper modules/neighbour_covariance_op.py:8-62 composes them from three
+ * mean-only accumulations over matrices of F, F*C and F*C*C columns: with
+ * j = idx[v,n],
+ *   S[v,f]       = sum_n w[v,n] a[j,f]
+ *   mean[v,f,c]  = sum_n w[v,n] a[j,f] x[j,c] / (S[v,f] + 1e-3)
+ *   cov[v,f,c,d] = sum_n w[v,n] a[j,f] (x[j,c] - mean[j,f,c]) (x[j,d] - mean[j,f,d]) / (S[v,f] + 1e-3)
+ * (every neighbour centred on its own mean; sums in slot order, divided and
+ * multiplied by K as the accumulation's mean is; a zero denominator gives 0).
+ * Two passes over the table, nothing of F*C*C columns is materialised as
+ * input. d_weights are exp(-distsq) and d_feats the activated features
+ * (sigmoid + 1e-3), both formed by the caller. The compiled
+ * NeighbourCovarianceOpFunctor of the reference
+ * (modules/compiled/neighbour_covariance_kernel.h: unweighted, lower triangle,
+ * centred on the accumulating vertex) is not what that wrapper calls and is not
+ * built. n_coords <= 6.
+ *   d_coords [n_vert, n_coords], d_weights, d_n_idxs [n_vert, n_neigh],
+ *   d_feats [n_vert, n_feat]; outputs d_covariance [n_vert, n_feat, n_coords^2],
+ *   d_means [n_vert, n_feat, n_coords], d_sum_weights [n_vert, n_feat] (S).
+ *   d_vertex_order (may be NULL): as for hgc_accumulate_knn_slots. */
+int hgc_neighbour_covariance(const float *d_coords, const float *d_weights, const float *d_feats,
+                             const int *d_n_idxs, const int *d_vertex_order, float *d_covariance,
+                             float *d_means, float *d_sum_weights, int n_vert, int n_coords, int n_feat,
+                             int n_neigh, hgc_stream_t stream);
+
 /* out[m,f] = sum over (v,n) with idx[v,n] == m of feat[v,f] * w[v,n]
  * (idx < 0: no neighbour). Replaces PushKnnOpFunctor
  * (modules/compiled/push_knn_kernel.h, _kernel.cc:40-62); the additions of

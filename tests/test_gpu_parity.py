@@ -1073,6 +1073,47 @@ def test_neighbour_covariance(oracle):
     # exp and sigmoid come from different libraries: 1e-5 relative to the largest entry
     assert np.abs(mean.cpu().numpy() - rmean).max() <= 1e-5 * np.abs(rmean).max()
     assert np.abs(cov.cpu().numpy() - rcov).max() <= 1e-5 * np.abs(rcov).max()
+    # the two kernels form every term and every sum as the route through the accumulation op does
+    from hgcalml_amd.neighbour_covariance_op import _moments_by_accumulation
+    cov2, mean2 = _moments_by_accumulation(t(x), t(d2), t(feat), t(idx))
+    assert torch.equal(mean, mean2) and torch.equal(cov, cov2)
+
+
+@pytest.mark.parametrize("C,F,K", [(4, 16, 12), (2, 5, 7), (6, 3, 9), (7, 4, 5)])
+def test_neighbour_covariance_shapes_and_gradients(C, F, K):
+    """other coordinate and feature counts (seven coordinates take the route through the accumulation op),
+    and the gradients w.r.t. coordinates, distances and features against float64 autograd of the formulas"""
+    from hgcalml_amd import NeighbourCovariance
+    rng = np.random.default_rng(83 + C + F)
+    n = 400
+    x = rng.standard_normal((n, C)).astype(np.float32)
+    feat = rng.standard_normal((n, F)).astype(np.float32)
+    idx = np.stack([np.concatenate([[v], rng.choice(np.delete(np.arange(n), v), K - 1, replace=False)])
+                    for v in range(n)]).astype(np.int32)
+    idx[5:50, K // 2:] = -1
+    d2 = rng.random((n, K), dtype=np.float32)
+    gc = rng.standard_normal((n, F, C * C)).astype(np.float32)
+    gm = rng.standard_normal((n, F, C)).astype(np.float32)
+
+    def formulas(xx, dd, ff, ii):
+        a = torch.sigmoid(ff) + 1e-3
+        w = torch.where(ii >= 0, torch.exp(-dd), torch.zeros_like(dd))
+        j = ii.clamp(min=0).long()
+        total = (w[:, :, None] * a[j]).sum(1)[:, :, None] + 1e-3
+        mean = (w[:, :, None, None] * a[j][:, :, :, None] * xx[j][:, :, None, :]).sum(1) / total
+        cen = xx[:, None, :] - mean
+        outer = (cen[:, :, :, None] * cen[:, :, None, :]).reshape(n, F, C * C) * a[:, :, None]
+        return (w[:, :, None, None] * outer[j]).sum(1) / total, mean
+
+    tx, td, tf = (t(v_).requires_grad_(True) for v_ in (x, d2, feat))
+    cov, mean = NeighbourCovariance(tx, td, tf, t(idx))
+    ((cov * t(gc)).sum() + (mean * t(gm)).sum()).backward()
+    rx, rd, rf = (t(v_).double().requires_grad_(True) for v_ in (x, d2, feat))
+    rcov, rmean = formulas(rx, rd, rf, t(idx))
+    ((rcov * t(gc).double()).sum() + (rmean * t(gm).double()).sum()).backward()
+    assert torch.allclose(cov.double(), rcov, rtol=1e-4, atol=1e-5) and torch.allclose(mean.double(), rmean, rtol=1e-4, atol=1e-5)
+    for got, want in ((tx.grad, rx.grad), (td.grad, rd.grad), (tf.grad, rf.grad)):
+        assert (got.double() - want).abs().max() <= 1e-4 * want.abs().max()
 
 
 @pytest.mark.parametrize("case", ["clusters", "one_bin", "ragged"])
