@@ -764,7 +764,9 @@ int accumulate_forward(const float *d_distances, const float *d_feat, const int 
                        int n_out_feat, int mean_and_max, float divisor, const int *d_order, hgc_stream_t stream) {
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_out_feat == n_feat * (mean_and_max ? 2 : 1), "n_out_feat must be n_feat * (mean_and_max ? 2 : 1)");
-    HGC_REQUIRE((long long)n_vert * std::max(n_neigh, 2 * n_feat) < (1ll << 31), "tensor too large for int32 indexing");
+    // slots are numbered with 32 bits; matrices of any size (beyond 4 GiB: the thread-per-element kernels with
+    // 64-bit offsets)
+    HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neigh must stay below 2^31");
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_distances && d_feat && d_idxs && d_out_feat, "null pointer");
     HGC_REQUIRE(!mean_and_max || d_out_maxidxs, "mean_and_max needs d_out_maxidxs");
@@ -885,7 +887,7 @@ int accumulate_gradient(const float *d_grad_from_out_features, const float *d_di
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_grad_from_out_feat == n_feat * (mean_and_max ? 2 : 1),
                 "gradient width must be n_feat * (mean_and_max ? 2 : 1)");
-    HGC_REQUIRE((long long)n_vert * std::max(n_neigh, 2 * n_feat) < (1ll << 31), "tensor too large for int32 indexing");
+    HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neigh must stay below 2^31");
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_grad_from_out_features && (want_w || want_f), "null pointer");
     HGC_REQUIRE(!want_w || (d_feat && d_neigh_indices), "null pointer");

@@ -54,6 +54,7 @@ struct KnnParams {
     float radius_sq;  // < 0: no radius
     int n_vert, K, n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction;
     int boundary_shift;  // the boundary of bin b sits at bin_boundaries[b << boundary_shift]
+    int rank_base;       // WINDOW kernels: the neighbour ranks below this one are in the output already
 };
 
 template <int C>
@@ -262,7 +263,12 @@ __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, 
 // C: coordinates per point, NB: binned dimensions (0 for either: taken from the
 // arguments), S: registers of the sorted list per lane, MAPPED: results in the
 // index space and at the positions of `sorting`.
-template <int C, int NB, int S, bool MAPPED>
+// WINDOW: more neighbours are asked for than the registers hold (64 S). The search then runs
+// once per window of 64 S ranks: launch t finds the 64 S smallest keys ABOVE the last key of
+// launch t-1 (read back from the output row) and writes them behind it. Every launch walks
+// the shells from the query's bin again and stops by the same rule on its own list, so each
+// window is exact; slow (the walk is repeated) but without a bound on K.
+template <int C, int NB, int S, bool MAPPED, bool WINDOW = false>
 __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(const KnnParams p) {
     constexpr int kDims = NB > 0 ? NB : kMaxBinDims;  // array extents
     __shared__ __attribute__((aligned(8))) uint8_t mark_strips[kQueriesPerBlock][kMarkCap];
@@ -275,12 +281,20 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
     if (q >= p.n_vert) return;
 
     const int K = p.K;
-    const int Kn = K - 1;  // neighbours besides the point itself
+    const int rank_base = WINDOW ? p.rank_base : 0;
+    const int Kn = WINDOW ? min(K - 1 - rank_base, S * kWave) : K - 1;  // neighbours (besides the point itself) to find
     const int self_id = MAPPED ? p.sorting[q] : q;
     const size_t out_row = (size_t)self_id * K;
     const int pad_idx = p.tf_compat ? self_id : -1;
 
     bool searching = Kn > 0;
+    uint64_t floor_key = 0;  // WINDOW: only keys above this one are candidates
+    if (WINDOW && rank_base > 0) {
+        const int last_idx = p.out_idx[out_row + rank_base];
+        const float last_dist = p.out_dist[out_row + rank_base];
+        if (last_idx == pad_idx) searching = false;  // the windows before found fewer points than they had room for
+        floor_key = ((uint64_t)__float_as_uint(last_dist) << 32) | (uint32_t)last_idx;
+    }
     if (p.use_direction) {
         const int dq = p.direction[q];
         if (dq == 0 || dq == 2) searching = false;  // may not have neighbours
@@ -483,6 +497,7 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                             valid &= ~__builtin_amdgcn_ballot_w64(dj == 1 || dj == 2);  // may not be a neighbour
                         }
                         const uint64_t ck = ((uint64_t)__float_as_uint(dsq) << 32) | id;
+                        if (WINDOW) valid &= __builtin_amdgcn_ballot_w64(ck > floor_key);
                         // below the K-th key and (keys compare like distances) within the radius
                         uint64_t beats = valid & __builtin_amdgcn_ballot_w64(ck < cut);
                         if (beats) {
@@ -527,7 +542,7 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
     }
 
     // ---- write the row: slot 0 = self, then ascending (distance, index) ----
-    if (lane == 0) {
+    if (lane == 0 && rank_base == 0) {
         p.out_idx[out_row] = self_id;
         p.out_dist[out_row] = 0.f;
     }
@@ -536,8 +551,8 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
         const int rank = s * kWave + lane;
         if (rank < Kn) {
             const bool filled = key[s] != kEmptyKey;
-            p.out_idx[out_row + 1 + rank] = filled ? (int)(uint32_t)key[s] : pad_idx;
-            p.out_dist[out_row + 1 + rank] = filled ? __uint_as_float((uint32_t)(key[s] >> 32)) : 0.f;
+            p.out_idx[out_row + 1 + rank_base + rank] = filled ? (int)(uint32_t)key[s] : pad_idx;
+            p.out_dist[out_row + 1 + rank_base + rank] = filled ? __uint_as_float((uint32_t)(key[s] >> 32)) : 0.f;
         }
     }
 }
@@ -546,6 +561,15 @@ template <int C, int NB, bool MAPPED>
 int launch_levels(const KnnParams &p, hipStream_t s) {
     const int levels = std::max(1, ceil_div(p.K - 1, kWave));
     const dim3 grid(ceil_div(p.n_vert, kQueriesPerBlock)), block(kQueriesPerBlock * kWave);
+    if (levels > kBulkInsertMaxRuns) {  // more neighbours than the registers hold: one launch per window of ranks
+        KnnParams window = p;
+        for (window.rank_base = 0; window.rank_base < p.K - 1; window.rank_base += kBulkInsertMaxRuns * kWave) {
+            knn_wave_kernel<C, NB, kBulkInsertMaxRuns, MAPPED, true><<<grid, block, 0, s>>>(window);
+            const int rc = check_launch("knn_wave_kernel (window of ranks)");
+            if (rc) return rc;
+        }
+        return HGC_OK;
+    }
     switch (levels) {
         case 1: knn_wave_kernel<C, NB, 1, MAPPED><<<grid, block, 0, s>>>(p); break;
         case 2: knn_wave_kernel<C, NB, 2, MAPPED><<<grid, block, 0, s>>>(p); break;
@@ -585,7 +609,7 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
     HGC_REQUIRE(n_coords > 1, "BinnedSelectKnnOp expects at least 2 dimensions.");
     HGC_REQUIRE(n_coords >= n_bin_dim, "fewer coordinates than binning dimensions");
     HGC_REQUIRE(n_vert >= 0, "negative number of points");
-    HGC_REQUIRE(n_neigh >= 1 && n_neigh <= 8 * kWave + 1, "1 <= n_neighbours <= %d", 8 * kWave + 1);
+    HGC_REQUIRE(n_neigh >= 1, "n_neighbours must be positive");
     HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neighbours overflows int32");
     // candidate rows are addressed by 32-bit byte offsets
     HGC_REQUIRE((unsigned long long)n_vert * (unsigned long long)n_coords * sizeof(float) < (1ull << 32),
@@ -624,6 +648,7 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
     p.tf_compat = tf_compat;
     p.use_direction = use_direction;
     p.boundary_shift = boundary_shift;
+    p.rank_base = 0;
     return d_sorting ? launch_coords<true>(p, s) : launch_coords<false>(p, s);
 }
 

@@ -421,7 +421,7 @@ int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *
                       float *d_feat_grad, float *d_w_grad, int n_vert, int n_neigh, int n_feat, hgc_stream_t stream) {
     HGC_REQUIRE(n_vert <= 0 || (d_feat_grad && d_w_grad), "null pointer");
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
-    HGC_REQUIRE((long long)n_vert * std::max(n_neigh, n_feat) < (1ll << 31), "tensor too large for int32 indexing");
+    HGC_REQUIRE((long long)n_vert * n_neigh < (1ll << 31), "n_vert * n_neigh must stay below 2^31");
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_grad && d_weights && d_feat && d_idxs, "null pointer");
     {

@@ -160,9 +160,10 @@ int hgc_gather_rows(const void *d_in, const int *d_rows, void *d_out, int n_rows
  * (or (self, 0.0) if tf_compat) at the tail. The reference leaves the slots in
  * fill/replacement order; the neighbour SET is the same except where the K-th
  * and (K+1)-th distances are exactly equal, where the lower index is kept.
- * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, 1 <= n_neigh <= 513 (the
- * reference has no limit on n_neigh), n_vert * n_neigh < 2^31, coordinate matrix
- * below 4 GiB. A shell at distance d is walked as (2d+1)^(n_bin_dim-1) rows of
+ * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, n_neigh >= 1 without an upper
+ * bound (up to 513 the sorted list lives in registers; beyond that the search
+ * runs once per window of 512 ranks and is correspondingly slow),
+ * n_vert * n_neigh < 2^31, coordinate matrix below 4 GiB. A shell at distance d is walked as (2d+1)^(n_bin_dim-1) rows of
  * bins; a query whose walk would reach a shell of 2^24 rows or more (grids far
  * finer than the points are dense, e.g. 5 binned dimensions with more than 30
  * bins each) ends there and sets HGC_FLAG_SHELL_TOO_WIDE in the status word;

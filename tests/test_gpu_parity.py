@@ -228,6 +228,20 @@ def test_knn_neighbour_counts(oracle, K):
     run_knn_case(oracle, coords, rs, K, 7)
 
 
+@pytest.mark.parametrize("K,radius,tf_compatible", [(514, None, False), (700, None, False), (1300, None, True),
+                                                     (1100, 0.3, False), (1026, 0.25, True)])
+def test_knn_more_neighbours_than_the_registers_hold(oracle, K, radius, tf_compatible):
+    """K beyond 513 (the reference has no bound): the search runs once per window of 512 ranks. Two events, one of
+    them smaller than K (its rows end in padding inside a later window, or before it), with and without a radius
+    that leaves some rows short"""
+    rng = np.random.default_rng(170 + K)
+    coords = rng.random((2400, 3), dtype=np.float32)
+    rs = np.array([0, 900, 2400], np.int32)
+    # with ~1500 candidate distances per row an exact tie at the K-th boundary does occur (one row at K = 514);
+    # compare_knn proves every such row a tie and a valid neighbour set
+    run_knn_case(oracle, coords, rs, K, 6, max_radius=radius, tf_compatible=tf_compatible, max_ties=3)
+
+
 @pytest.mark.parametrize("C,n_bins", [(3, 4), (4, 12), (2, 5)])
 def test_knn_dense_bins_long_candidate_lists(oracle, C, n_bins):
     """thousands of points in a few bins: the candidate list of a batch of
@@ -836,6 +850,33 @@ def test_accumulate_matrices_beyond_4_gib():
         assert torch.equal(gx[lo:hi].view(torch.int32), gx_s.view(torch.int32))
         tol = grad_tolerance(gs.cpu().numpy(), xs.cpu().numpy(), ids.cpu().numpy(), ws.cpu().numpy(), K)
         assert (np.abs(gw[lo:hi].cpu().numpy() - gw_s.cpu().numpy()) <= 2 * tol).all()
+
+
+def test_push_knn_matrices_beyond_2_to_31_elements():
+    """PushKnn and its gradient on a feature matrix of more than 2^31 elements (9 GB): the thread-per-element
+    kernels address it with 64-bit offsets (the reference indexes with size_t, modules/compiled/push_knn_kernel.cc:40-62);
+    only the slot numbers n_vert * n_neigh have to fit 31 bits. Closed blocks of the table, run alone through the wave
+    kernels (pinned against the oracle elsewhere), must give the same rows bit for bit (weight gradient: tolerance)."""
+    from hgcalml_amd import ops
+    n, F, K, blk = 4_400_000, 512, 4, 3000
+    assert n * F >= 1 << 31 and n * K < 1 << 31
+    gen = torch.Generator(device=DEV).manual_seed(78)
+    x = torch.randn(n, F, generator=gen, device=DEV)
+    w, idx = blocked_neighbour_table(n, K, blk, gen)
+    out = torch.ops.hgcalml.push_knn(w, x, idx)
+    tail = (n // blk - 1) * blk
+    for lo, hi in ((0, blk), (tail, n)):
+        xs, ws, ids = x[lo:hi].contiguous(), w[lo:hi].contiguous(), (idx[lo:hi] - lo).contiguous()
+        assert torch.equal(out[lo:hi].view(torch.int32), torch.ops.hgcalml.push_knn(ws, xs, ids).view(torch.int32))
+    g = out      # any matrix of the same shape serves as upstream gradient
+    wgrad, fgrad = torch.ops.hgcalml.push_knn_grad(g, w, x, idx)
+    for lo, hi in ((0, blk), (tail, n)):
+        xs, ws, gs, ids = (x[lo:hi].contiguous(), w[lo:hi].contiguous(), g[lo:hi].contiguous(),
+                           (idx[lo:hi] - lo).contiguous())
+        wgrad_s, fgrad_s = torch.ops.hgcalml.push_knn_grad(gs, ws, xs, ids)
+        assert torch.equal(fgrad[lo:hi].view(torch.int32), fgrad_s.view(torch.int32))
+        scale = (gs[ids.long()].abs() * xs[:, None, :].abs()).sum(-1)
+        assert ((wgrad[lo:hi] - wgrad_s).abs() <= 2e-5 * scale + 1e-30).all()
 
 
 # ------------------------------------------------------------------ ops next to the accumulation
