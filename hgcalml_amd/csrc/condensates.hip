@@ -365,6 +365,10 @@ __device__ __forceinline__ bool covered_by_list(const uint32_t *list, int capaci
         }
         float4 rr = *reinterpret_cast<const float4 *>(list + (size_t)CMAX * capacity + s4);
         if (s4 + 4 > hi) {  // slots behind the range may be in the middle of being written
+            // Invariant: nothing read from a slot >= hi may reach `hits`. The distances d0..d3 of such
+            // slots are sums of squares of whatever the slot held -- non-negative, infinite or NaN --
+            // and their radius is forced to -1 here, so `d <= rr` is false for every one of them;
+            // the box words of a slot are only read for a set bit of `hits`.
             const int real = hi - s4;
             rr.w = -1.f;
             if (real < 3) rr.z = -1.f;

@@ -167,7 +167,9 @@ int hgc_gather_rows(const void *d_in, const int *d_rows, void *d_out, int n_rows
  * bins; a query whose walk would reach a shell of 2^24 rows or more (grids far
  * finer than the points are dense, e.g. 5 binned dimensions with more than 30
  * bins each) ends there and sets HGC_FLAG_SHELL_TOO_WIDE in the status word;
- * hgc_binned_select_knn_pipeline refuses such grids on the host instead. */
+ * without a registered status word that is silent and the rows of such queries
+ * can miss neighbours (hgc_binned_select_knn_pipeline refuses such grids on the
+ * host instead, whatever the status word). */
 int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int *d_direction,
                           const int *d_dim_bin_idx, const int *d_bin_boundaries,
                           const int *d_n_bins, const float *d_bin_width,
@@ -236,7 +238,9 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
  * HGC_STATIC_SCRATCH_BYTES is refused with HGC_ERR_WORKSPACE (N = 150,000 points
  * with 4 coordinates, one event and n_bins = 30 need 19.3 MiB). All calls on
  * one GPU share that GPU's array: calls that overlap on one GPU (different
- * streams or threads) race and must be ordered by the caller. */
+ * streams or threads) race and must be ordered by the caller. The first call on
+ * a device looks the array's address up (hipGetSymbolAddress, under a lock):
+ * make it outside a stream capture. */
 #define HGC_STATIC_SCRATCH_BYTES (32u << 20)
 int hgc_binned_select_knn_pipeline_static(const float *d_coords, const int *d_row_splits,
                                           const int *d_direction, int n_vert, int n_coords, int n_rs,
@@ -456,7 +460,10 @@ int hgc_exp_neg_grad(const float *d_weight_grad, const float *d_weights, float *
                      long long n_values, hgc_stream_t stream);
 
 /* Ascending sort of n 64-bit keys that differ pairwise (none of them all ones):
- * d_values[i] = the low value_bits bits of the i-th smallest key. The order of
+ * d_values[i] = the low value_bits bits of the i-th smallest key. The keys are
+ * not checked: equal keys come out in an unspecified order relative to each
+ * other (every value still appears exactly once, nothing faults), and a key of
+ * all ones is taken for padding and may lose its place to real keys. The order of
  * the condensate selection (event, beta descending, position) is this sort; the
  * reference has no counterpart (binned_assign_to_condensates_kernel.cc:187-236
  * picks by a linear arg-max per condensation point). d_keys is overwritten.

@@ -1632,6 +1632,20 @@ def test_sort_distinct_keys_buckets_beyond_the_lds_stage(n, stage):
         assert (got == np.argsort(keys, kind="stable").astype(np.int32)).all()
 
 
+def test_sort_distinct_keys_with_equal_keys_still_permutes():
+    """equal keys are outside the contract (their mutual order is unspecified): every value still comes out once
+    and the keys come out ascending"""
+    from hgcalml_amd import ops
+    rng = np.random.default_rng(3)
+    n = 50000
+    high = rng.integers(0, 40, n).astype(np.uint64) << np.uint64(20)     # ~1250 copies of each key ...
+    keys = high | np.arange(n, dtype=np.uint64)                          # ... told apart by the value bits only
+    dup = keys.copy()
+    dup[1::2] = (dup[1::2] & ~np.uint64((1 << 20) - 1)) | (dup[0:-1:2] & np.uint64((1 << 20) - 1))   # pairs of equal keys
+    got = ops.sort_distinct_keys(t(dup.view(np.int64)), 20).cpu().numpy()
+    assert len(got) == n and (np.sort(got) == np.sort((dup & np.uint64((1 << 20) - 1)).astype(np.int32))).all()
+
+
 def test_sort_distinct_keys_refuses_what_it_cannot_do():
     from hgcalml_amd import ops
     keys = t(np.arange(10, dtype=np.int64))
