@@ -17,10 +17,17 @@ into a HIP graph (same kernels, same buffers); the faster of the two is reported
 
 The `roofline` object is measured in a second timed loop of the same run (also
 K iterations, HIP events on the stream the kernels are launched on) at cfg4
-(N=1,000,000, K=64, F=128, banded neighbour table): the dominant kernel, one
-launch of the accumulate_knn gradient (algorithmic bytes 4*N*(3K+5F)), with
-the forward launch (4*N*(2K+4F)), the forward+gradient pair and the pair plus
-one build of the inverse neighbour index next to it, against the 8 TB/s HBM peak.
+(N=1,000,000, K=64, F=128, banded neighbour table): the dominant piece, one call
+of the accumulate_knn gradient (algorithmic bytes 4*N*(3K+5F); two kernels: the
+streaming pass that builds the per-slot hit records and the gather over the
+inverse index), with the forward launch (4*N*(2K+4F)), the forward+gradient pair
+and the pair plus one build of the inverse neighbour index next to it, against
+the 8 TB/s HBM peak. Next to the fraction of the HBM roofline it states two
+floors of what this formulation can reach on this memory system: the same
+K-fold gather of 512-byte rows with one multiply-add per element and nothing
+else (`l2_gather_floor_ms`: PushKnn over the same table, timed in the same run),
+and the issue time of the gradient's vector instructions alone (`valu_floor_ms`,
+from the committed counter summary).
 
 `cpu_baseline` times the CPU oracle (a single-threaded C restatement of the
 reference CPU kernels) on this box's host: the binned kNN kernel over the full
@@ -48,6 +55,21 @@ HBM_PEAK_GBS = 8000.0
 # carries what the committed summary profiles/accumulate_knn_cfg4_hbm_counters.txt holds
 # (its "bench.py reads" line, stamped with the commit it was measured at), or null.
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "accumulate_knn_cfg4_hbm_counters.txt")
+COUNTER_SUMMARY = os.path.join(ROOT, "profiles", "accumulate_knn_cfg4_sq_tcc_counters.txt")
+
+
+def measured_valu_floor():
+    """{'ms': issue time of the gradient's vector instructions, 'measured_at': commit} from the committed
+    counter summary (its "bench.py reads" line), or None"""
+    try:
+        with open(COUNTER_SUMMARY) as f:
+            for line in f:
+                if line.startswith("bench.py reads:"):
+                    fields = dict(kv.split("=", 1) for kv in line.split(":", 1)[1].split())
+                    return {"ms": float(fields["gradient_valu_floor_ms"]), "measured_at": fields.get("measured_at", "unknown")}
+    except (OSError, KeyError, ValueError):
+        pass
+    return None
 
 
 def measured_traffic():
@@ -245,13 +267,21 @@ def main():
     _, arg4, slots4 = torch.ops.hgcalml.accumulate_knn_slots(w4, x4, i4, 0, True)
     inv_ms = event_ms(lambda: ops.inverse_neighbour_index(i4), 3, 1)
     inv = ops.inverse_neighbour_index(i4)
+    import hgcalml_amd.globals as gl
     grad_ms = event_ms(lambda: torch.ops.hgcalml.accumulate_knn_grad_slots(g4, w4, x4, i4, arg4, slots4, *inv),
                        args.steps, args.warmup)
+    # the same gradient through the gather that compares slot bytes (no records, no streaming pass)
+    gl.acc_grad_hit_records = False
+    grad_slots_ms = event_ms(lambda: torch.ops.hgcalml.accumulate_knn_grad_slots(g4, w4, x4, i4, arg4, slots4, *inv),
+                             max(3, args.steps // 2), 2)
+    gl.acc_grad_hit_records = None
+    # the K-fold gather of this table with one multiply-add per gathered element and nothing else
+    push_ms = event_ms(lambda: torch.ops.hgcalml.push_knn(w4, x4, i4), max(3, args.steps // 2), 2)
     bytes_fwd = 4.0 * n4 * (2 * K4 + 4 * F4)
     bytes_bwd = 4.0 * n4 * (3 * K4 + 5 * F4)
     achieved = (bytes_fwd + bytes_bwd) / ((fwd_ms[0] + grad_ms[0]) * 1e-3) / 1e9
-    log("bench: cfg4 fwd %.3f ms, grad %.3f ms, inverse index (one-off) %.3f ms -> %.1f GB/s" %
-        (fwd_ms[0], grad_ms[0], inv_ms[0], achieved))
+    log("bench: cfg4 fwd %.3f ms, grad %.3f ms (slot-byte gather %.3f ms, bare ordered gather %.3f ms), inverse index "
+        "(one-off) %.3f ms -> %.1f GB/s" % (fwd_ms[0], grad_ms[0], grad_slots_ms[0], push_ms[0], inv_ms[0], achieved))
 
     if args.section == "streams":
         # same table, same inputs: the gradient without the max half (no slot bytes, no max-half loads), and the
@@ -337,6 +367,8 @@ def main():
         log("bench: CPU oracle kNN %.0f queries/s (%.1f s)" % (qps, secs))
 
     traffic = measured_traffic() if args.roofline_scale == 1.0 else None
+    valu_floor = measured_valu_floor() if args.roofline_scale == 1.0 else None
+    floors_ms = [push_ms[0]] + ([valu_floor["ms"]] if valu_floor else [])
     with_build = (bytes_fwd + bytes_bwd) / ((fwd_ms[0] + grad_ms[0] + inv_ms[0]) * 1e-3) / 1e9
     line = {
         "metric": "kNN queries/s at N=150k,4D,K=64; accumulate_knn fwd+grad achieved HBM GB/s",
@@ -359,13 +391,22 @@ def main():
         "accumulate_fwd_grad_GBps": round(achieved, 1),
         # the dominant kernel of the graded path: one launch of the one-pass gradient kernel
         "roofline": {"bound": "hbm",
-                     "kernel": "accumulate_grad_fused_kernel: accumulate_knn gradient (weights + features), cfg4 "
-                               "(N=%d, K=%d, F=%d), one launch" % (n4, K4, F4),
+                     "kernel": "hit_records_kernel + accumulate_grad_records_kernel: one call of the accumulate_knn "
+                               "gradient (weights + features), cfg4 (N=%d, K=%d, F=%d)" % (n4, K4, F4),
                      "achieved": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": traffic["gradient"] if traffic else None,
                      "traffic_measured_at": traffic["measured_at"] if traffic else None,
                      "algorithmic_bytes": bytes_bwd, "launch_ms": round(grad_ms[0], 4),
+                     # the same call through the gather that compares slot bytes (one kernel, no records)
+                     "launch_ms_slot_byte_gather": round(grad_slots_ms[0], 4),
+                     # floors of this formulation on this memory system: the bare K-fold gather of the same rows
+                     # (PushKnn, timed above), the issue time of the gradient's vector instructions (counters)
+                     "l2_gather_floor_ms": round(push_ms[0], 4),
+                     "valu_floor_ms": valu_floor["ms"] if valu_floor else None,
+                     "valu_floor_from": "profiles/accumulate_knn_cfg4_sq_tcc_counters.txt @ %s" %
+                                        valu_floor["measured_at"] if valu_floor else None,
+                     "frac_of_achievable": round(max(floors_ms) / grad_ms[0], 4),
                      "forward": {"kernel": "accumulate_fwd_wave_kernel, same workload, one launch",
                                  "achieved": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9, 1),
                                  "frac": round(bytes_fwd / (fwd_ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
