@@ -311,7 +311,7 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
     const int *__restrict__ row_splits, int n_vert, int n_dims, int n_rs, int n_bins_scalar,
     float *__restrict__ shift_out, float *__restrict__ bin_width_out, int *__restrict__ n_bins_out,
     int *__restrict__ binass, int *__restrict__ flat, int *__restrict__ rank, int *__restrict__ counts,
-    int n_bins_bound, int sub_shift, int *__restrict__ status) {
+    int n_bins_bound, int sub_shift, int spatial, int *__restrict__ status) {
     __shared__ float s_lo[4][kMaxBinDims], s_hi[4][kMaxBinDims];
     __shared__ float s_shift[kMaxBinDims], s_bw;
     __shared__ int s_nb[kMaxBinDims];
@@ -350,16 +350,19 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
     __syncthreads();
     const float bw = s_bw;
     for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < n_vert; p += gridDim.x * blockDim.x) {
-        int mul = 1, cell = 0, flags = 0;
+        int mul = 1, cell = 0, flags = 0, half = 0;
         for (int c = n_dims - 1; c >= 0; --c) {
             const float raw = coords[(size_t)p * stride + c];
             if (!isfinite(raw)) flags |= HGC_FLAG_COORDINATE_NOT_FINITE;
             const float x = raw - s_shift[c];
-            int k = (int)(x / bw);
+            const float in_bins = x / bw;
+            int k = (int)in_bins;
             const int nb = s_nb[c];
             if (k < 0 || k >= nb) {
                 k = 0;
                 flags |= HGC_FLAG_COORDINATE_OUT_OF_GRID;
+            } else if (in_bins - (float)k >= 0.5f) {
+                half |= 1 << (n_dims - 1 - c);  // upper half of the bin in this dimension (last dimension: bit 0)
             }
             binass[(size_t)p * (n_dims + 1) + c + 1] = k;
             cell += k * mul;
@@ -378,10 +381,14 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
         if (flags && status) atomicOr(status, flags);
         cell = min(cell, n_bins_bound - 1);  // no effect for row splits that end at n_vert
         binass[(size_t)p * (n_dims + 1)] = ev;
-        flat[p] = cell;
-        // every bin has 2^sub_shift counters, a point takes the one its index names:
-        // the increments of a crowded bin queue up on several addresses instead of one
-        rank[p] = atomicAdd(&counts[((size_t)cell << sub_shift) | (p & ((1 << sub_shift) - 1))], 1);
+        // Every bin has 2^sub_shift counters, so that the increments of a crowded bin queue up on
+        // several addresses instead of one. spatial (sub_shift = n_dims): the counter is the half of
+        // the bin the point lies in, per dimension -- the bin's points then come grouped by these
+        // 2^n_dims sub-cells, a grid of half the bin width nested in the bins, and the flat index
+        // names the sub-cell. Otherwise a point takes the counter its index names.
+        const int counter = (cell << sub_shift) | (spatial ? half : (p & ((1 << sub_shift) - 1)));
+        flat[p] = spatial ? counter : cell;
+        rank[p] = atomicAdd(&counts[counter], 1);
     }
 }
 
@@ -390,12 +397,17 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
 __global__ __launch_bounds__(256) void move_to_bin_order_kernel(
     const float *__restrict__ coords, const int *__restrict__ binass, const int *__restrict__ flat,
     const int *__restrict__ rank, const int *__restrict__ direction, const int *__restrict__ boundaries, int n_vert,
-    int n_coords, int n_dims, int sub_shift, int rows_aligned, int *__restrict__ sorting,
-    float *__restrict__ scoords, int *__restrict__ sflat, int *__restrict__ sbinass, int *__restrict__ sdir) {
+    int n_coords, int n_dims, int sub_shift, int spatial, int rows_aligned, int *__restrict__ sorting,
+    float *__restrict__ scoords, int *__restrict__ sflat, int *__restrict__ sbinass, int *__restrict__ sdir,
+    int *__restrict__ bin_starts, int n_bins_bound) {
     const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    // the boundary of every bin once more without the stride of the counters: the table the search reads most
+    if (bin_starts)
+        for (int b = p; b <= n_bins_bound; b += gridDim.x * blockDim.x)
+            bin_starts[b] = boundaries[(size_t)b << sub_shift];
     if (p >= n_vert) return;
-    const int cell = flat[p];
-    const int at = boundaries[((size_t)cell << sub_shift) | (p & ((1 << sub_shift) - 1))] + rank[p];
+    const int cell = flat[p];  // spatial: the sub-cell, which is its own counter
+    const int at = boundaries[spatial ? (size_t)cell : ((size_t)cell << sub_shift) | (p & ((1 << sub_shift) - 1))] + rank[p];
     sorting[at] = p;
     sflat[at] = cell;
     if (n_coords == 4 && rows_aligned) {
@@ -442,37 +454,46 @@ int launch_fill_i32(int *p, int value, long long n, hipStream_t s) {
 // results again), many assign the bins
 static int grouping_blocks(int n_vert) { return std::max(1, std::min(128, ceil_div(n_vert, 1024))); }
 
-int bin_grouping_sub_shift(int n_bins_bound) {
+bool bin_grouping_spatial(int n_bins_bound, int n_bin_dims) {
+    return n_bin_dims >= 2 && n_bin_dims <= 4 && (((size_t)n_bins_bound << n_bin_dims) + 1) <= ((size_t)1 << 22);
+}
+
+int bin_grouping_sub_shift(int n_bins_bound, int n_bin_dims, bool spatial) {
+    if (spatial && bin_grouping_spatial(n_bins_bound, n_bin_dims)) return n_bin_dims;
     int shift = 0;
     while (shift < 5 && (((size_t)n_bins_bound << (shift + 1)) + 1) <= ((size_t)1 << 20)) ++shift;
     return shift;
 }
 
-static size_t grouping_counters(int n_bins_bound) {
-    return ((size_t)n_bins_bound << bin_grouping_sub_shift(n_bins_bound)) + 1;
+static size_t grouping_counters(int n_bins_bound, int n_bin_dims, bool spatial) {
+    return ((size_t)n_bins_bound << bin_grouping_sub_shift(n_bins_bound, n_bin_dims, spatial)) + 1;
 }
 
-size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound) {
+size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound, int n_bin_dims, bool spatial) {
     size_t temp = 0;
     (void)rocprim::exclusive_scan(nullptr, temp, (const int *)nullptr, (int *)nullptr, 0,
-                                  grouping_counters(n_bins_bound), rocprim::plus<int>(), (hipStream_t) nullptr);
+                                  grouping_counters(n_bins_bound, n_bin_dims, spatial), rocprim::plus<int>(),
+                                  (hipStream_t) nullptr);
     const size_t n = std::max(n_vert, 1);
     return align_up(temp) + align_up((size_t)grouping_blocks(n_vert) * 2 * kMaxBinDims * sizeof(float)) +
-           align_up(grouping_counters(n_bins_bound) * sizeof(int)) + 2 * align_up(n * sizeof(int)) +
+           align_up(grouping_counters(n_bins_bound, n_bin_dims, spatial) * sizeof(int)) + 2 * align_up(n * sizeof(int)) +
            align_up(n * (kMaxBinDims + 1) * sizeof(int));
 }
 
 int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_direction, int n_vert, int n_coords,
                  int n_bin_dims, int n_rs, int n_bins_scalar, int n_bins_bound, float *d_shift, float *d_bin_width,
                  int *d_n_bins, int *d_boundaries, int *d_sorting, float *d_scoords, int *d_sflat, int *d_sbinass,
-                 int *d_sdir, void *workspace, size_t workspace_bytes, hipStream_t s) {
-    if (!workspace || !aligned256(workspace) || workspace_bytes < bin_grouping_workspace_bytes(n_vert, n_bins_bound))
+                 int *d_sdir, bool spatial, int *d_bin_starts, void *workspace, size_t workspace_bytes,
+                 hipStream_t s) {
+    spatial = spatial && bin_grouping_spatial(n_bins_bound, n_bin_dims);
+    if (!workspace || !aligned256(workspace) ||
+        workspace_bytes < bin_grouping_workspace_bytes(n_vert, n_bins_bound, n_bin_dims, spatial))
         return fail(HGC_ERR_WORKSPACE, "bin grouping workspace missing, misaligned or too small");
     const int blocks = grouping_blocks(n_vert);
     Carver carve(workspace);
     float *partial = carve.take<float>((size_t)blocks * 2 * kMaxBinDims);
-    const int sub_shift = bin_grouping_sub_shift(n_bins_bound);
-    const size_t n_counters = grouping_counters(n_bins_bound);
+    const int sub_shift = bin_grouping_sub_shift(n_bins_bound, n_bin_dims, spatial);
+    const size_t n_counters = grouping_counters(n_bins_bound, n_bin_dims, spatial);
     int *counts = carve.take<int>(n_counters);
     int *flat = carve.take<int>(n_vert);
     int *rank = carve.take<int>(n_vert);
@@ -486,7 +507,7 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
     bin_points_ranked_kernel<<<std::min(4096, ceil_div(n_vert, 256)), 256, 0, s>>>(d_coords, n_coords, partial, blocks, d_row_splits, n_vert,
                                                     n_bin_dims, n_rs, n_bins_scalar, d_shift, d_bin_width, d_n_bins,
                                                     binass, flat, rank, counts, n_bins_bound, sub_shift,
-                                                    status_word());
+                                                    spatial ? 1 : 0, status_word());
     rc = check_launch("bin_points_ranked");
     if (rc) return rc;
     // boundaries[b << sub_shift] = number of points in bins below b
@@ -495,8 +516,9 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
         ((reinterpret_cast<uintptr_t>(d_coords) | reinterpret_cast<uintptr_t>(d_scoords)) & 15u) == 0;
     move_to_bin_order_kernel<<<ceil_div(n_vert, 256), 256, 0, s>>>(d_coords, binass, flat, rank, d_direction,
                                                                    d_boundaries, n_vert, n_coords, n_bin_dims,
-                                                                   sub_shift, rows_aligned, d_sorting, d_scoords,
-                                                                   d_sflat, d_sbinass, d_sdir);
+                                                                   sub_shift, spatial ? 1 : 0, rows_aligned, d_sorting,
+                                                                   d_scoords, d_sflat, d_sbinass, d_sdir, d_bin_starts,
+                                                                   n_bins_bound);
     return check_launch("move_to_bin_order");
 }
 

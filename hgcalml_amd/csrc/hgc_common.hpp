@@ -84,14 +84,22 @@ int sample_sort_values(uint64_t *d_keys, uint64_t *d_spare, long long n, int val
 // into bin order (`d_sorting[i]` = original index of the i-th point). Unlike
 // hgc_sort_by_bin the order inside a bin is not specified (it can differ from
 // run to run). `n_bins_bound` bounds the number of bins of all events. The
-// boundary of bin b is d_boundaries[b << bin_grouping_sub_shift(n_bins_bound)];
-// the table has (n_bins_bound << shift) + 1 entries.
-int bin_grouping_sub_shift(int n_bins_bound);
-size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound);
+// boundary of bin b is d_boundaries[b << shift] with shift =
+// bin_grouping_sub_shift(...); the table has (n_bins_bound << shift) + 1 entries.
+// spatial (granted where bin_grouping_spatial says so: 2 to 4 binned dimensions, table
+// within bounds): shift = n_bin_dims, the points of a bin come grouped by the half of the
+// bin they lie in per dimension (sub-cell bits: dimension i at bit n_bin_dims - 1 - i),
+// every table entry is the boundary of such a sub-cell, and d_sflat holds sub-cell indices
+// (bin << n_bin_dims | bits) instead of bin indices.
+// d_bin_starts (may be null): n_bins_bound + 1 entries, the boundary of every bin without a stride.
+bool bin_grouping_spatial(int n_bins_bound, int n_bin_dims);
+int bin_grouping_sub_shift(int n_bins_bound, int n_bin_dims, bool spatial);
+size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound, int n_bin_dims, bool spatial);
 int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_direction, int n_vert, int n_coords,
                  int n_bin_dims, int n_rs, int n_bins_scalar, int n_bins_bound, float *d_shift, float *d_bin_width,
                  int *d_n_bins, int *d_boundaries, int *d_sorting, float *d_scoords, int *d_sflat, int *d_sbinass,
-                 int *d_sdir, void *workspace, size_t workspace_bytes, hipStream_t s);
+                 int *d_sdir, bool spatial, int *d_bin_starts, void *workspace, size_t workspace_bytes,
+                 hipStream_t s);
 
 int launch_fill_i32(int *p, int value, long long n, hipStream_t s);
 
@@ -115,13 +123,18 @@ size_t stable_key_sort_workspace_bytes(long long total, int n_keys, int per_key_
 int stable_key_sort(const int *d_keys, const int *d_values, long long total, int n_keys, int per_key_hint,
                     int *d_offsets, int *d_order, void *workspace, size_t workspace_bytes, hipStream_t s);
 
-// hgc_binned_select_knn_fused over a boundary table with stride 2^boundary_shift
+// hgc_binned_select_knn_fused over a boundary table with stride 2^boundary_shift.
+// fine_bits > 0 (= n_bin_dim): d_bin_idx holds the half-bin cells of bin_grouping's spatial mode
+// and d_cell_boundaries is that mode's table (one entry per cell); a query whose bin holds more
+// than fine_min_population points then walks the nested grid of half the bin width instead of
+// the bins.
 int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const int *d_direction,
                               const int *d_dim_bin_idx, const int *d_bin_boundaries, int boundary_shift,
                               const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
                               const float *d_shift, float max_radius, int *d_indices, float *d_dist, int n_vert,
                               int n_neigh, int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
-                              int use_direction, hipStream_t s);
+                              int use_direction, const int *d_cell_boundaries, int fine_bits,
+                              int fine_min_population, hipStream_t s);
 
 // hgc_binned_assign_to_condensates with two more arguments: with d_high set, the *_h
 // arrays are the arrays of all hits themselves (n_vert_h == n_vert, d_indices_to_filtered[i]

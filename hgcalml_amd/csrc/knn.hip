@@ -44,6 +44,7 @@ struct KnnParams {
     const int *direction;
     const int *dim_bin_idx;
     const int *bin_boundaries;
+    const int *cell_boundaries;  // NESTED kernels: one entry per half-bin cell
     const int *n_bins;
     const float *bin_width;
     const int *sorting;  // may be null
@@ -55,6 +56,11 @@ struct KnnParams {
     int n_vert, K, n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction;
     int boundary_shift;  // the boundary of bin b sits at bin_boundaries[b << boundary_shift]
     int rank_base;       // WINDOW kernels: the neighbour ranks below this one are in the output already
+    // fine_bits = n_bin_dim: bin_idx is that of the spatial grouping, bin_idx[q] = bin << fine_bits |
+    // half-bin bits, and the points of a bin are grouped by these cells. NESTED kernels: a query
+    // whose bin holds more than fine_min_population points walks the nested grid of half the bin
+    // width over cell_boundaries.
+    int fine_bits, fine_min_population;
 };
 
 template <int C>
@@ -98,6 +104,16 @@ __device__ __forceinline__ float dist_sq(const float (&q)[C > 0 ? C : 1], const 
         }
     }
     return acc;
+}
+
+// A value that is the same in every lane, told to the compiler: what is computed from it
+// then sits in scalar registers. (Loads through pointers the compiler cannot prove read-only
+// are vector loads even at a wave-uniform address.) Not everything gains by it: a vector
+// instruction takes one scalar operand only, so values that meet in one instruction, like
+// the two edge distances of a dimension, are better left in vector registers.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float uniform(float v) {
+    return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v)));
 }
 
 extern "C" __device__ int __llvm_amdgcn_writelane(int, int, int) __asm("llvm.amdgcn.writelane");
@@ -250,8 +266,9 @@ constexpr int kMarkCap = 2048;
 // against 0.78 ms with 4 and 0.95 ms with 8).
 constexpr int kQueriesPerBlock = 1;
 
-// q = x / w, r = x % w for 0 <= x < 2^24 and w < 2^13, without an integer divide:
-// the float quotient is off by at most one, the remainder says which way
+// q = x / w, r = x % w for 0 <= x < 2^22 and w < 2^13, without an integer divide: with inv_w
+// within an ulp of 1 / w (the hardware's approximate reciprocal will do) the float quotient is
+// off by at most one, the remainder says which way
 __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, int &r) {
     q = (int)((float)x * inv_w);
     r = x - q * w;
@@ -260,51 +277,25 @@ __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, 
     r -= fix * w;
 }
 
-// C: coordinates per point, NB: binned dimensions (0 for either: taken from the
-// arguments), S: registers of the sorted list per lane, MAPPED: results in the
-// index space and at the positions of `sorting`.
-// WINDOW: more neighbours are asked for than the registers hold (64 S). The search then runs
-// once per window of 64 S ranks: launch t finds the 64 S smallest keys ABOVE the last key of
-// launch t-1 (read back from the output row) and writes them behind it. Every launch walks
-// the shells from the query's bin again and stops by the same rule on its own list, so each
-// window is exact; slow (the walk is repeated) but without a bound on K.
-template <int C, int NB, int S, bool MAPPED, bool WINDOW = false>
-__global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(const KnnParams p) {
+// The walk over the shells of bins around query q (one wave), which leaves the Kn smallest keys
+// in `key`. FINE: the walk runs on the nested grid of half the bin width (see KnnParams::fine_bits).
+// Its cells are numbered 2 k + h per dimension (bin k, half h); the points of a bin come grouped
+// by half-bin cell with the LAST dimension's half as the lowest bit, so a run of cells along the
+// last dimension is contiguous inside a bin and falls into one piece per bin it touches: a row of
+// the shell at distance d takes up to d + 1 segments instead of one. Any grid gives the same
+// result, the K smallest keys: the choice is one of cost only.
+//
+// A walk on the nested grid gives up (returns false, the list is to be discarded) when it has not
+// ended after shell kFineMaxShell: its shells have 2^(B-1) times the rows of the bins' shells
+// and more segments per row, which pays only while few of them are needed. All coordinates
+// being binned, that is the rule where the bin's neighbourhood is about as crowded as the bin.
+constexpr int kFineMaxShell = 3;
+
+template <int C, int NB, int S, bool MAPPED, bool WINDOW, bool FINE>
+__device__ __forceinline__ bool walk_shells(const KnnParams &p, const int q, const int lane, uint8_t *const marks,
+                                            const int Kn, const uint64_t floor_key, uint64_t (&key)[S]) {
     constexpr int kDims = NB > 0 ? NB : kMaxBinDims;  // array extents
-    __shared__ __attribute__((aligned(8))) uint8_t mark_strips[kQueriesPerBlock][kMarkCap];
-    const int lane = lane_id();
-    // queries come in bin order and differ a lot in cost from region to region:
-    // chunks of 512 of them are dealt to the XCDs in turn
-    const int tile = xcd_chunked_block<512>(blockIdx.x, gridDim.x);
-    const int q = tile * kQueriesPerBlock + (threadIdx.x >> 6);  // one query per wave
-    uint8_t *const marks = mark_strips[threadIdx.x >> 6];
-    if (q >= p.n_vert) return;
-
-    const int K = p.K;
-    const int rank_base = WINDOW ? p.rank_base : 0;
-    const int Kn = WINDOW ? min(K - 1 - rank_base, S * kWave) : K - 1;  // neighbours (besides the point itself) to find
-    const int self_id = MAPPED ? p.sorting[q] : q;
-    const size_t out_row = (size_t)self_id * K;
-    const int pad_idx = p.tf_compat ? self_id : -1;
-
-    bool searching = Kn > 0;
-    uint64_t floor_key = 0;  // WINDOW: only keys above this one are candidates
-    if (WINDOW && rank_base > 0) {
-        const int last_idx = p.out_idx[out_row + rank_base];
-        const float last_dist = p.out_dist[out_row + rank_base];
-        if (last_idx == pad_idx) searching = false;  // the windows before found fewer points than they had room for
-        floor_key = ((uint64_t)__float_as_uint(last_dist) << 32) | (uint32_t)last_idx;
-    }
-    if (p.use_direction) {
-        const int dq = p.direction[q];
-        if (dq == 0 || dq == 2) searching = false;  // may not have neighbours
-    }
-
-    uint64_t key[S];
-#pragma unroll
-    for (int s = 0; s < S; ++s) key[s] = kEmptyKey;
-
-    if (searching) {
+    {
         // query coordinates (wave-uniform)
         float qc[C > 0 ? C : 1];
         const float *qrow = p.coord + (size_t)q * p.n_coords;
@@ -314,6 +305,8 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
         }
 
         const int B = NB > 0 ? NB : p.n_bin_dim;
+        const int own_cell = uniform(p.bin_idx[q]);   // with fine_bits: bin and half-bin bits
+        const int own_bin = own_cell >> p.fine_bits;
         int nb[kDims], qb[kDims];
         int cells_per_event = 1;
         int reach_max = 0;  // beyond this shell distance no bin is inside the grid
@@ -322,15 +315,20 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
             nb[i] = 1;
             qb[i] = 0;
             if (i < B) {
-                nb[i] = p.n_bins[i];
-                qb[i] = p.dim_bin_idx[(size_t)q * (B + 1) + 1 + i];
+                nb[i] = uniform(p.n_bins[i]);
+                qb[i] = uniform(p.dim_bin_idx[(size_t)q * (B + 1) + 1 + i]);
                 cells_per_event *= nb[i];
+                if (FINE) {
+                    nb[i] *= 2;
+                    qb[i] = 2 * qb[i] + ((own_cell >> (B - 1 - i)) & 1);
+                }
                 reach_max = max(reach_max, max(qb[i], nb[i] - 1 - qb[i]));
             }
         }
-        const int event_base = cells_per_event * (p.bin_idx[q] / cells_per_event);
+        const int event_base = cells_per_event * (own_bin / cells_per_event);
         const int nb_last = nb[B - 1], qb_last = qb[B - 1];
-        const float bw = p.bin_width[0];
+        const int bins_last = FINE ? nb_last >> 1 : nb_last;  // bins (not cells) along the last dimension
+        const float bw = FINE ? 0.5f * p.bin_width[0] : p.bin_width[0];
         const float inv_bw = 1.f / bw;
         const float bins_per_unit = 1.001f * inv_bw;  // generous by 0.1 %, for the pruning bound only
 
@@ -362,30 +360,97 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
         const uint64_t radius_limit = has_radius ? (uint64_t)(__float_as_uint(p.radius_sq) + 1u) << 32 : kEmptyKey;
         uint64_t cut = radius_limit;  // min(thr, radius_limit): what a candidate's key has to stay below
 
+        // Row and slot numbers of a shell are divided as floats (divmod_small), which is exact below
+        // 2^22 for divisors below 2^13: no shell has more rows than the grid, times the pieces of
+        // a row on the nested grid.
+        {
+            long long grid_rows = FINE ? nb_last / 2 + 2 : 2;
+            bool rows_fit = true;
+            for (int i = 0; i < B - 1; ++i) {
+                grid_rows = min(grid_rows * nb[i], 1ll << 40);
+                rows_fit = rows_fit && nb[i] < (1 << 13);
+            }
+            if (!rows_fit || grid_rows >= (1ll << 22)) {
+                if (FINE) return false;  // the grid of bins may do
+                if (p.status && lane == 0) atomicOr(p.status, HGC_FLAG_SHELL_TOO_WIDE);
+                return true;  // the list stays empty
+            }
+        }
+        // the first shell whose slots need more than one batch of 64 (walked whole: (2d+1)^(B-1)
+        // rows and (2d-1)^(B-1) inner rows; on the nested grid d + 1 pieces per row)
+        const int first_cut_shell = FINE ? (B == 2 ? 5 : B == 3 ? 2 : B == 4 ? 2 : 1) : (B == 2 ? 17 : B == 3 ? 3 : B == 4 ? 2 : 1);
+
         // Shell 0 (the query's own bin) never ends the search. When it cannot fill
         // the list either (so that it cannot prune shell 1), it is walked together
         // with shell 1: every row of that shell then takes its whole run of the last
         // dimension, and the run of the centre row contains the own bin.
         bool with_own_bin = false;
-        {
-            const int own = p.bin_idx[q];
-            if (reach_max > 0 && own + 1 < p.n_bboundaries)
-                with_own_bin = p.bin_boundaries[(size_t)(own + 1) << p.boundary_shift] -
-                                   p.bin_boundaries[(size_t)own << p.boundary_shift] <= Kn;
+        if (reach_max > 0 && own_bin + 1 < p.n_bboundaries) {
+            if (FINE)
+                with_own_bin = p.cell_boundaries[own_cell + 1] - p.cell_boundaries[own_cell] <= Kn;
+            else
+                with_own_bin = p.bin_boundaries[(size_t)(own_bin + 1) << p.boundary_shift] -
+                                   p.bin_boundaries[(size_t)own_bin << p.boundary_shift] <= Kn;
         }
-        for (int d = with_own_bin ? 1 : 0; d <= reach_max; ++d) {
-            // a shell is walked as W^(B-1) rows of bins; the row number has to stay exact as a float
-            // (divmod_small) and 2 * rows inside an int
-            long long rows64 = d < (1 << 12) ? 1 : 1ll << 24;
-            for (int i = 0; i < B - 1; ++i) rows64 = min(rows64 * (2 * min(d, 1 << 12) + 1), 1ll << 24);
-            if (rows64 >= 1ll << 24) {
-                if (p.status && lane == 0) atomicOr(p.status, HGC_FLAG_SHELL_TOO_WIDE);
-                break;
+        for (int d = uniform(with_own_bin ? 1 : 0); d <= reach_max; ++d) {
+            if (FINE && d > kFineMaxShell) return false;
+            // The shell is walked as rows of bins (cells) along the last dimension. Only rows inside
+            // the grid and within reach of the search are numbered: per leading dimension the
+            // offsets -below[i] .. -below[i] + width[i] - 1, where an offset o is within reach when
+            // (|o| - 1 + distance to the facing edge of the own bin) bin widths do not exceed the
+            // K-th distance (the radius) as it is when the shell begins, generously rounded.
+            // (A shell whose slots fit one batch anyway is cut to the grid only.)
+            const bool cut_to_reach = d >= first_cut_shell;
+            float reach_bins = 3.0e9f;
+            if (cut_to_reach) {
+                float reach2_shell = thr == kEmptyKey ? 3.0e38f : __uint_as_float((uint32_t)(thr >> 32));
+                if (has_radius) reach2_shell = fminf(reach2_shell, p.radius_sq);
+                if (reach2_shell < 1.0e37f) reach_bins = __builtin_amdgcn_sqrtf(reach2_shell) * bins_per_unit + 1.001f;
             }
-            const int W = 2 * d + 1;
-            const float inv_W = 1.f / (float)W;
-            const int n_rows = (int)rows64;
-            const int n_slots = d == 0 ? 1 : 2 * n_rows;
+            int below[kDims], width[kDims], below_in[kDims], width_in[kDims];
+            float inv_width[kDims], inv_width_in[kDims];
+            int n_rows = 1;
+            int n_inner = 1;  // rows with every leading offset inside +-(d - 1): they contribute end caps only
+#pragma unroll
+            for (int i = 0; i < kDims - 1; ++i) {
+                below[i] = below_in[i] = 0;
+                width[i] = width_in[i] = 1;
+                inv_width[i] = inv_width_in[i] = 1.f;
+                if (i < B - 1) {
+                    int lo_i = min(d, qb[i]), hi_i = min(d, nb[i] - 1 - qb[i]);
+                    if (cut_to_reach) {
+                        lo_i = min(lo_i, uniform((int)fminf(reach_bins - to_lower[i], 1.0e9f)));
+                        hi_i = min(hi_i, uniform((int)fminf(reach_bins - to_upper[i], 1.0e9f)));
+                    }
+                    below[i] = lo_i;
+                    width[i] = lo_i + hi_i + 1;
+                    below_in[i] = min(lo_i, max(d - 1, 0));
+                    width_in[i] = below_in[i] + min(hi_i, max(d - 1, 0)) + 1;
+                    if (i > 0) {  // the leading digit of a row number is what the divisions leave
+                        inv_width[i] = __builtin_amdgcn_rcpf((float)width[i]);
+                        inv_width_in[i] = __builtin_amdgcn_rcpf((float)width_in[i]);
+                    }
+                    n_rows *= width[i];  // at most the rows of the grid: see rows_fit
+                    n_inner *= width_in[i];
+                }
+            }
+            // the last dimension: are the end caps (offsets -d and +d) inside the grid and within reach?
+            int lo_last = min(d, qb_last), hi_last = min(d, nb_last - 1 - qb_last);
+            if (cut_to_reach) {
+                lo_last = min(lo_last, uniform((int)fminf(reach_bins - tl_last, 1.0e9f)));
+                hi_last = min(hi_last, uniform((int)fminf(reach_bins - tu_last, 1.0e9f)));
+            }
+            const bool low_caps = lo_last == d, high_caps = hi_last == d;
+            // Segments per row on the nested grid: a run falls into one piece per bin it touches
+            // (an inner row uses two of them for its end caps).
+            const int P = FINE ? max(2, ((qb_last + hi_last) >> 1) - ((qb_last - lo_last) >> 1) + 1) : 1;
+            const float inv_P = __builtin_amdgcn_rcpf((float)P);
+            // Slots of the shell. Grid of bins: one per row (the run of a row on a face of the
+            // shell, one end cap of an inner row) and, when both end caps are in reach, one more per
+            // inner row. When the own bin is walked with shell 1 every row is a run. Nested grid:
+            // P per row.
+            const bool runs_only = d == 0 || (d == 1 && with_own_bin);
+            const int n_slots = d == 0 ? 1 : FINE ? n_rows * P : (!runs_only && low_caps && high_caps) ? n_rows + n_inner : n_rows;
 
             for (int slot0 = 0; slot0 < n_slots; slot0 += kWave) {
                 // ---- each lane resolves one segment of the shell ----
@@ -398,22 +463,33 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                 float reach2 = thr == kEmptyKey ? 3.0e38f : __uint_as_float((uint32_t)(thr >> 32));
                 if (has_radius) reach2 = fminf(reach2, p.radius_sq);
                 if (slot < n_slots) {
-                    int row = slot >> 1;
-                    const bool second = slot & 1;
-                    bool inside = true, on_face = d == 0 || (d == 1 && with_own_bin);
-                    int cell = 0;
+                    int row, piece;
+                    bool inner = false;  // numbered among the inner rows
+                    if (FINE) {
+                        divmod_small(slot, P, inv_P, row, piece);
+                    } else {
+                        inner = slot >= n_rows;
+                        row = inner ? slot - n_rows : slot;
+                        piece = (inner || !low_caps) ? 1 : 0;  // the end cap an inner row takes in this slot
+                    }
+                    const bool second = piece == 1;
+                    bool on_face = runs_only;
+                    int cell = 0, halves = 0;
                     float gap2 = 0.f;  // squared lower bound of the distance to this row of bins
                     int off[kDims];
 #pragma unroll
                     for (int i = kDims - 2; i >= 0; --i) {
                         off[i] = 0;
                         if (i < B - 1) {
+                            // digits of the row number: offsets of the leading dimensions
+                            const int below_i = inner ? below_in[i] : below[i];
                             if (i > 0) {
                                 int digit;
-                                divmod_small(row, W, inv_W, row, digit);
-                                off[i] = digit - d;
+                                divmod_small(row, inner ? width_in[i] : width[i], inner ? inv_width_in[i] : inv_width[i],
+                                             row, digit);
+                                off[i] = digit - below_i;
                             } else {
-                                off[i] = row - d;  // what is left is the leading digit
+                                off[i] = row - below_i;  // what is left is the leading digit
                             }
                         }
                     }
@@ -421,17 +497,21 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                     for (int i = 0; i < kDims - 1; ++i) {
                         if (i < B - 1) {
                             const int o = off[i];
-                            const int k = qb[i] + o;
-                            inside = inside && (uint32_t)k < (uint32_t)nb[i];
+                            const int k = qb[i] + o;  // inside the grid: the numbered rows all are
                             on_face = on_face || o == d || o == -d;
-                            cell = cell * nb[i] + k;
+                            if (FINE) {
+                                cell = cell * (nb[i] >> 1) + (k >> 1);
+                                halves = (halves << 1) | (k & 1);
+                            } else {
+                                cell = cell * nb[i] + k;
+                            }
                             const float edge = o > 0 ? to_upper[i] : to_lower[i];
                             const float g = o == 0 ? 0.f : ((float)(abs(o) - 1) + edge) * bw;
                             gap2 += g * g;
                         }
                     }
-                    // a whole run of the last dimension (rows on a face of the shell; the
-                    // second slot of such a row is unused), or one of the two end caps
+                    // a whole run of the last dimension (rows on a face of the shell), or one of the
+                    // two end caps
                     const float cap_gap = ((float)(d - 1) + (second ? tu_last : tl_last)) * bw;
                     const float cap2 = gap2 + cap_gap * cap_gap;
                     // bins of a run that are provably too far are cut off (bound
@@ -443,17 +523,40 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                     const int cap = second ? qb_last + d : qb_last - d;
                     int lo = on_face ? run_lo : cap;
                     int hi = on_face ? run_hi : cap;
-                    const bool too_far = on_face ? (second || 0.999f * gap2 > reach2) : 0.999f * cap2 > reach2;
+                    bool too_far = on_face ? 0.999f * gap2 > reach2 : (piece > 1 || 0.999f * cap2 > reach2);
                     lo = max(lo, 0);
                     hi = min(hi, nb_last - 1);
-                    if (inside && !too_far && lo <= hi) {
-                        const int first = event_base + cell * nb_last + lo;
-                        const int last = event_base + cell * nb_last + hi + 1;
-                        if (last < p.n_bboundaries) {
-                            seg_start = p.bin_boundaries[(size_t)first << p.boundary_shift];
-                            seg_len = p.bin_boundaries[(size_t)last << p.boundary_shift] - seg_start;
-                        } else if (p.status) {  // the reference prints "idx out of range" and skips the bin
-                            atomicOr(p.status, HGC_FLAG_BIN_BEYOND_TABLE);
+                    if (FINE) {
+                        if (on_face) {
+                            // piece number `piece` of the run: the part inside one bin, counted from the
+                            // first bin any run of this shell can touch (not from this row's own first
+                            // bin: the run shrinks with the K-th distance while the row's slots may lie
+                            // in two batches)
+                            const int bin = ((qb_last - lo_last) >> 1) + piece;
+                            lo = max(lo, 2 * bin);
+                            hi = min(hi, 2 * bin + 1);
+                        }
+                    }
+                    if (!too_far && lo <= hi) {
+                        if (FINE) {
+                            const int bin = event_base + cell * bins_last + (lo >> 1);
+                            if (bin + 1 < p.n_bboundaries) {
+                                const int first = (((bin << (B - 1)) | halves) << 1) | (lo & 1);
+                                const int last = ((((bin << (B - 1)) | halves) << 1) | (hi & 1)) + 1;
+                                seg_start = p.cell_boundaries[first];
+                                seg_len = p.cell_boundaries[last] - seg_start;
+                            } else if (p.status) {
+                                atomicOr(p.status, HGC_FLAG_BIN_BEYOND_TABLE);
+                            }
+                        } else {
+                            const int first = event_base + cell * nb_last + lo;
+                            const int last = event_base + cell * nb_last + hi + 1;
+                            if (last < p.n_bboundaries) {
+                                seg_start = p.bin_boundaries[(size_t)first << p.boundary_shift];
+                                seg_len = p.bin_boundaries[(size_t)last << p.boundary_shift] - seg_start;
+                            } else if (p.status) {  // the reference prints "idx out of range" and skips the bin
+                                atomicOr(p.status, HGC_FLAG_BIN_BEYOND_TABLE);
+                            }
                         }
                     }
                 }
@@ -528,16 +631,89 @@ __global__ __launch_bounds__(kQueriesPerBlock * kWave) void knn_wave_kernel(cons
                 }
             }
 
-            // stop rule (fp32, evaluated left to right)
+            // stop rule (fp32, evaluated left to right); on the nested grid, which the reference does
+            // not have, with a margin for points that rounding has put into the neighbouring cell
             float reach = bw * (float)d;
             reach = reach * bw;
             reach = reach * (float)d;
+            if (FINE) reach *= 0.998f;
             uint64_t kth = kEmptyKey;
 #pragma unroll
             for (int s = 0; s < S; ++s)
                 if (s == kth_level) kth = readlane_u64(key[s], kth_lane);
             if (kth != kEmptyKey && reach > __uint_as_float((uint32_t)(kth >> 32))) break;
             if (has_radius && reach > p.radius_sq) break;
+        }
+    }
+    return true;
+}
+
+// C: coordinates per point, NB: binned dimensions (0 for either: taken from the
+// arguments), S: registers of the sorted list per lane, MAPPED: results in the
+// index space and at the positions of `sorting`.
+// WINDOW: more neighbours are asked for than the registers hold (64 S). The search then runs
+// once per window of 64 S ranks: launch t finds the 64 S smallest keys ABOVE the last key of
+// launch t-1 (read back from the output row) and writes them behind it. Every launch walks
+// the shells from the query's bin again and stops by the same rule on its own list, so each
+// window is exact; slow (the walk is repeated) but without a bound on K.
+// NESTED: the search runs over a nested grid (see KnnParams::fine_bits): a query whose bin holds more
+// than fine_min_population points walks the nested grid (and the grid of bins after all when that
+// walk gives up), the others the grid of bins.
+template <int C, int NB, int S, bool MAPPED, bool WINDOW = false, bool NESTED = false>
+__global__ __launch_bounds__(kQueriesPerBlock * kWave)
+__attribute__((amdgpu_waves_per_eu((NESTED && S == 1) ? 8 : 1, 8)))
+void knn_wave_kernel(const KnnParams p) {
+    __shared__ __attribute__((aligned(8))) uint8_t mark_strips[kQueriesPerBlock][kMarkCap];
+    const int lane = lane_id();
+    // queries come in bin order and differ a lot in cost from region to region:
+    // chunks of 512 of them are dealt to the XCDs in turn
+    const int tile = xcd_chunked_block<512>(blockIdx.x, gridDim.x);
+    const int q = tile * kQueriesPerBlock + (threadIdx.x >> 6);  // one query per wave
+    uint8_t *const marks = mark_strips[threadIdx.x >> 6];
+    if (q >= p.n_vert) return;
+    bool crowded = false;
+    if constexpr (NESTED) {
+        const int own_bin = uniform(p.bin_idx[q]) >> p.fine_bits;
+        if (own_bin + 1 < p.n_bboundaries)
+            crowded = p.bin_boundaries[(size_t)(own_bin + 1) << p.boundary_shift] -
+                          p.bin_boundaries[(size_t)own_bin << p.boundary_shift] > p.fine_min_population;
+    }
+
+    const int K = p.K;
+    const int rank_base = WINDOW ? p.rank_base : 0;
+    const int Kn = WINDOW ? min(K - 1 - rank_base, S * kWave) : K - 1;  // neighbours (besides the point itself) to find
+    const int self_id = MAPPED ? p.sorting[q] : q;
+    const size_t out_row = (size_t)self_id * K;
+    const int pad_idx = p.tf_compat ? self_id : -1;
+
+    bool searching = Kn > 0;
+    uint64_t floor_key = 0;  // WINDOW: only keys above this one are candidates
+    if (WINDOW && rank_base > 0) {
+        const int last_idx = p.out_idx[out_row + rank_base];
+        const float last_dist = p.out_dist[out_row + rank_base];
+        if (last_idx == pad_idx) searching = false;  // the windows before found fewer points than they had room for
+        floor_key = ((uint64_t)__float_as_uint(last_dist) << 32) | (uint32_t)last_idx;
+    }
+    if (p.use_direction) {
+        const int dq = p.direction[q];
+        if (dq == 0 || dq == 2) searching = false;  // may not have neighbours
+    }
+
+    uint64_t key[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) key[s] = kEmptyKey;
+
+    if (searching) {
+        if constexpr (NESTED) {
+            if (!crowded) {
+                walk_shells<C, NB, S, MAPPED, WINDOW, false>(p, q, lane, marks, Kn, floor_key, key);
+            } else if (!walk_shells<C, NB, S, MAPPED, WINDOW, true>(p, q, lane, marks, Kn, floor_key, key)) {
+#pragma unroll
+                for (int s = 0; s < S; ++s) key[s] = kEmptyKey;
+                walk_shells<C, NB, S, MAPPED, WINDOW, false>(p, q, lane, marks, Kn, floor_key, key);
+            }
+        } else {
+            walk_shells<C, NB, S, MAPPED, WINDOW, false>(p, q, lane, marks, Kn, floor_key, key);
         }
     }
 
@@ -569,6 +745,18 @@ int launch_levels(const KnnParams &p, hipStream_t s) {
             if (rc) return rc;
         }
         return HGC_OK;
+    }
+    if constexpr (MAPPED && C == NB && NB >= 2 && NB <= 4) {  // all coordinates binned: a crowded bin has its neighbours close by
+        if (p.fine_bits > 0 && p.cell_boundaries) {
+            switch (levels) {
+                case 1: knn_wave_kernel<C, NB, 1, MAPPED, false, true><<<grid, block, 0, s>>>(p); break;
+                case 2: knn_wave_kernel<C, NB, 2, MAPPED, false, true><<<grid, block, 0, s>>>(p); break;
+                case 3:
+                case 4: knn_wave_kernel<C, NB, 4, MAPPED, false, true><<<grid, block, 0, s>>>(p); break;
+                default: knn_wave_kernel<C, NB, 8, MAPPED, false, true><<<grid, block, 0, s>>>(p); break;
+            }
+            return check_launch("knn_wave_kernel (nested grid)");
+        }
     }
     switch (levels) {
         case 1: knn_wave_kernel<C, NB, 1, MAPPED><<<grid, block, 0, s>>>(p); break;
@@ -602,7 +790,8 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
                               const int *d_n_bins, const float *d_bin_width, const int *d_sorting,
                               const float *d_shift, float max_radius, int *d_indices, float *d_dist, int n_vert,
                               int n_neigh, int n_coords, int n_bin_dim, int n_bboundaries, int tf_compat,
-                              int use_direction, hipStream_t s) {
+                              int use_direction, const int *d_cell_boundaries, int fine_bits,
+                              int fine_min_population, hipStream_t s) {
     // same conditions as the reference op (binned_select_knn_kernel.cc:336-352)
     HGC_REQUIRE(n_bin_dim > 1, "BinnedSelectKnnOp expects at least 2 binning dimensions.");
     HGC_REQUIRE(n_bin_dim < 6, "BinnedSelectKnnOp expects maximum 5 binning dimensions.");
@@ -616,6 +805,8 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
                 "coordinate matrix must stay below 4 GiB");
     HGC_REQUIRE(n_bboundaries >= 2, "bin boundary table too short");
     HGC_REQUIRE(boundary_shift >= 0 && boundary_shift < 8, "bad boundary stride");
+    HGC_REQUIRE(fine_bits == 0 || (fine_bits == n_bin_dim && fine_bits <= 4),
+                "a nested grid has one bit per binned dimension, four at most");
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_coord && d_bin_idx && d_dim_bin_idx && d_bin_boundaries && d_n_bins && d_bin_width &&
                     d_indices && d_dist,
@@ -649,6 +840,9 @@ int binned_select_knn_strided(const float *d_coord, const int *d_bin_idx, const 
     p.use_direction = use_direction;
     p.boundary_shift = boundary_shift;
     p.rank_base = 0;
+    p.cell_boundaries = d_cell_boundaries;
+    p.fine_bits = fine_bits;
+    p.fine_min_population = fine_min_population;
     return d_sorting ? launch_coords<true>(p, s) : launch_coords<false>(p, s);
 }
 
@@ -666,7 +860,8 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
                                 int use_direction, hgc_stream_t stream) {
     return binned_select_knn_strided(d_coord, d_bin_idx, d_direction, d_dim_bin_idx, d_bin_boundaries, 0, d_n_bins,
                                      d_bin_width, d_sorting, d_shift, max_radius, d_indices, d_dist, n_vert, n_neigh,
-                                     n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction, as_stream(stream));
+                                     n_coords, n_bin_dim, n_bboundaries, tf_compat, use_direction, nullptr, 0, 0,
+                                     as_stream(stream));
 }
 
 int hgc_binned_select_knn(const float *d_coord, const int *d_bin_idx, const int *d_direction,

@@ -30,44 +30,65 @@ namespace {
 
 // The grid the kNN pipeline searches on. The neighbour sets do not depend on it (the search is
 // exact), only the run time does, so by default the pipeline does not take the caller's grid
-// (the reference wrapper's n_bins over min(3, C) dimensions) but its own: up to four binned
-// dimensions -- binning the fourth coordinate of 4-D points too removes the candidates that
-// are close in three coordinates and far in the fourth -- and about one point per cell,
-// n_bins = (points per event)^(1/dimensions). Measured on one event of 150,000 points, K = 64,
-// against n_bins = 30 over three dimensions: clusters + noise in 4-D 0.65 -> 0.53 ms, a Gaussian
-// blob in 4-D 1.33 -> 0.89 ms, clusters + noise in 3-D 0.45 -> 0.37 ms. Points with more than
-// four coordinates keep three binned dimensions, and their bins hold every point along the
-// others: the neighbourhood is wide in bin widths however fine the grid, so a coarser one,
-// 0.6 (points per event)^(1/3), serves better (150,000 points, K = 64, uniform / Gaussian:
-// 5-D 2.46 / 1.81 ms at 53 bins -> 1.4 / 1.8 ms at 32; 8-D 14.7 / 8.4 -> 7.9 / 8.0 ms). Small events
-// want fewer bins than one point per cell gives them (most of a small grid is boundary, and a shell
-// costs its rows whether they are inside the grid or not): 200,000 uniform 4-D points in 1000 events,
-// K = 64: 0.80 ms at 4 bins, 0.52 at 3; in 4000 events 1.07 ms at 4 bins, 0.31 at 2.
+// (the reference wrapper's n_bins over min(3, C) dimensions) but its own.
+//   * Up to four binned dimensions: binning the fourth coordinate of 4-D points too removes the
+//     candidates that are close in three coordinates and far in the fourth.
+//   * n_bins = 0.9 (points per event * 64 / K)^(1/dimensions) with K taken inside 32 .. 64: a bit
+//     more than one point per bin at K = 64, and finer for fewer neighbours (16 events of 20,000 to
+//     120,000 3-D points, K = 32, radius 0.1: 1.72 ms -> 1.59 ms). For more than 64 neighbours a
+//     coarser grid did not pay (150,000 clustered 4-D points, K = 129 / 257: 0.96 / 2.23 ms on the
+//     grid for 64, 1.02 / 2.49 ms on one scaled further).
+//   * Where every coordinate is binned (2 to 4 of them) and the table stays small, a nested grid of
+//     half the bin width for the queries of crowded bins (bin_grouping's spatial mode,
+//     KnnParams::fine_bits): with it the bins themselves can be wider than a single grid would
+//     want them, which is what sparse regions like (their shells are mostly empty bins). Measured
+//     kernel times, 150,000 points in 4-D, K = 64, single grid of 20 bins -> nested grid on 18 bins:
+//     clusters + noise 450 -> 425 us, Gaussian blob 825 -> 515 us, uniform 418 -> 351 us.
+//   * Points with more than four coordinates keep three binned dimensions, and their bins hold
+//     every point along the others: the neighbourhood is wide in bin widths however fine the
+//     grid, so a coarser one, 0.6 (points per event)^(1/3), serves better (150,000 points,
+//     K = 64, uniform / Gaussian: 5-D 2.46 / 1.81 ms at 53 bins -> 1.4 / 1.8 ms at 32; 8-D 14.7 /
+//     8.4 -> 7.9 / 8.0 ms).
+//   * Small events want fewer bins than that (most of a small grid is boundary): 200,000 uniform
+//     4-D points in 1000 events, K = 64: 0.80 ms at 4 bins, 0.52 at 3; in 4000 events 1.07 ms at
+//     4 bins, 0.31 at 2.
 thread_local int g_callers_knn_grid = 0;
 
 struct SearchGrid {
     int n_bin_dims, n_bins;
+    bool nested;  // ask for the nested grid of half the bin width (granted where the boundary table stays small)
 };
 
 SearchGrid callers_grid(int n_coords, int n_bins_scalar, int max_bin_dims) {
-    return {std::min(max_bin_dims, n_coords), n_bins_scalar};
+    return {std::min(max_bin_dims, n_coords), n_bins_scalar, false};
 }
 
-SearchGrid own_grid(int n_vert, int n_coords, int n_rs) {
+// kSmallestGridK: the grid for this many neighbours or fewer is the finest one (it sizes the workspace)
+constexpr int kSmallestGridK = 32, kLargestGridK = 64;
+// a bin with more than (K - 1) / kCrowdedBinFraction points sends its queries to the nested grid
+constexpr int kCrowdedBinFraction = 4;
+
+SearchGrid own_grid(int n_vert, int n_coords, int n_rs, int n_neigh) {
     const int dims = n_coords <= 4 ? n_coords : 3;
     const double per_event = std::max(1.0, (double)n_vert / std::max(1, n_rs - 1));
-    const double per_cell_rule = std::pow(per_event, 1.0 / std::max(dims, 1));
-    // small events: 0.75 of that up to 5,000 points per event, rising to 1 at 50,000
+    // small events: 0.75 of the rule up to 5,000 points per event, rising to 1 at 50,000
     const double small = std::min(1.0, std::max(0.75, 0.75 + 0.25 * (std::log10(per_event) - 3.7)));
-    const int n_bins = (int)std::lround((n_coords <= 4 ? small : 0.6) * per_cell_rule);
-    return {dims, std::max(2, std::min(n_bins, dims >= 4 ? 40 : dims == 3 ? 128 : 1024))};
+    double n_bins;
+    if (n_coords <= 4) {
+        const double k = std::min(std::max(n_neigh, kSmallestGridK), kLargestGridK);
+        n_bins = 0.9 * small * std::pow(per_event * 64.0 / k, 1.0 / dims);
+    } else {
+        n_bins = 0.6 * std::pow(per_event, 1.0 / dims);
+    }
+    return {dims, std::max(2, std::min((int)std::lround(n_bins), dims >= 4 ? 40 : dims == 3 ? 128 : 1024)),
+            dims == n_coords};
 }
 
-SearchGrid search_grid(int n_vert, int n_coords, int n_rs, int n_bins_scalar, int max_bin_dims) {
+SearchGrid search_grid(int n_vert, int n_coords, int n_rs, int n_neigh, int n_bins_scalar, int max_bin_dims) {
     const SearchGrid asked = callers_grid(n_coords, n_bins_scalar, max_bin_dims);
     // a request the reference op refuses stays refused
     if (g_callers_knn_grid || asked.n_bin_dims < 2 || asked.n_bin_dims > 5 || n_bins_scalar < 1) return asked;
-    return own_grid(n_vert, n_coords, n_rs);
+    return own_grid(n_vert, n_coords, n_rs, n_neigh);
 }
 
 constexpr int kMaxDevices = 64;
@@ -92,16 +113,21 @@ int static_scratch(void **out) {
 }
 
 struct KnnPipelineLayout {
-    size_t shift, bin_width, n_bins, sorting, bounds, scoords, sflat, sbinass, sdir, grouping_ws, total;
+    size_t shift, bin_width, n_bins, sorting, bounds, bin_starts, scoords, sflat, sbinass, sdir, grouping_ws, total;
     int total_bins_bound;
+    bool nested;
+    int boundary_shift;
 };
 
-KnnPipelineLayout knn_layout(int n_vert, int n_coords, int n_bin_dims, int n_rs, int n_bins_scalar, int use_direction) {
+KnnPipelineLayout knn_layout(int n_vert, int n_coords, const SearchGrid &grid, int n_rs, int use_direction) {
     KnnPipelineLayout L{};
+    const int n_bin_dims = grid.n_bin_dims, n_bins_scalar = grid.n_bins;
     // every per-dimension bin count is at most n_bins_scalar + 1
     long long bound = n_rs - 1;
     for (int i = 0; i < n_bin_dims; ++i) bound = std::min<long long>(bound * (n_bins_scalar + 1), 1ll << 40);
     L.total_bins_bound = (int)std::min<long long>(bound, (1ll << 31) - 2);
+    L.nested = grid.nested && bin_grouping_spatial(L.total_bins_bound, n_bin_dims);
+    L.boundary_shift = bin_grouping_sub_shift(L.total_bins_bound, n_bin_dims, L.nested);
     const size_t n = std::max(n_vert, 1);
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -113,12 +139,13 @@ KnnPipelineLayout knn_layout(int n_vert, int n_coords, int n_bin_dims, int n_rs,
     L.bin_width = take(sizeof(float));
     L.n_bins = take(8 * sizeof(int));
     L.sorting = take(n * sizeof(int));
-    L.bounds = take((((size_t)L.total_bins_bound << bin_grouping_sub_shift(L.total_bins_bound)) + 1) * sizeof(int));
+    L.bounds = take((((size_t)L.total_bins_bound << L.boundary_shift) + 1) * sizeof(int));
+    L.bin_starts = take(((size_t)L.total_bins_bound + 1) * sizeof(int));
     L.scoords = take(n * n_coords * sizeof(float));
     L.sflat = take(n * sizeof(int));
     L.sbinass = take(n * (n_bin_dims + 1) * sizeof(int));
     L.sdir = take(use_direction ? n * sizeof(int) : 0);
-    L.grouping_ws = take(bin_grouping_workspace_bytes(n_vert, L.total_bins_bound));
+    L.grouping_ws = take(bin_grouping_workspace_bytes(n_vert, L.total_bins_bound, n_bin_dims, L.nested));
     L.total = off;
     return L;
 }
@@ -405,10 +432,13 @@ size_t hgc_binned_select_knn_pipeline_workspace_bytes(int n_vert, int n_coords, 
     const SearchGrid asked = callers_grid(n_coords, n_bins_scalar, max_bin_dims);
     if (n_vert < 0 || n_coords < 1 || n_rs < 2 || n_bins_scalar < 1 || asked.n_bin_dims < 1 || asked.n_bin_dims > 5)
         return 0;
-    // enough for either grid, whichever hgc_set_knn_grid selects at the time of the call
-    const SearchGrid own = own_grid(n_vert, n_coords, n_rs);
-    return std::max(knn_layout(n_vert, n_coords, asked.n_bin_dims, n_rs, asked.n_bins, use_direction).total,
-                    knn_layout(n_vert, n_coords, own.n_bin_dims, n_rs, own.n_bins, use_direction).total);
+    // enough for either grid, whichever hgc_set_knn_grid selects at the time of the call, and for
+    // the library's own grid at any number of neighbours (the coarser grids of larger numbers can be
+    // nested ones where the finest is not)
+    size_t bytes = knn_layout(n_vert, n_coords, asked, n_rs, use_direction).total;
+    for (int k = kSmallestGridK; k <= kLargestGridK; k *= 2)
+        bytes = std::max(bytes, knn_layout(n_vert, n_coords, own_grid(n_vert, n_coords, n_rs, k), n_rs, use_direction).total);
+    return bytes;
 }
 
 int hgc_binned_select_knn_pipeline_static(const float *d_coords, const int *d_row_splits, const int *d_direction,
@@ -438,19 +468,19 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
     HGC_REQUIRE(n_bins_scalar >= 1, "n_bins must be positive");
     HGC_REQUIRE(std::min(max_bin_dims, n_coords) > 1, "BinnedSelectKnnOp expects at least 2 binning dimensions.");
     HGC_REQUIRE(std::min(max_bin_dims, n_coords) < 6, "BinnedSelectKnnOp expects maximum 5 binning dimensions.");
-    const SearchGrid grid = search_grid(n_vert, n_coords, n_rs, n_bins_scalar, max_bin_dims);
+    const SearchGrid grid = search_grid(n_vert, n_coords, n_rs, n_neigh, n_bins_scalar, max_bin_dims);
     const int n_bin_dims = grid.n_bin_dims;
     n_bins_scalar = grid.n_bins;
-    {   // the widest shell a query can reach, (2 (n_bins + 1) + 1)^(B - 1) rows of bins, has to stay below 2^24
+    {   // the rows of bins of the grid (all dimensions but the last), which bound the rows of a shell, stay below 2^22
         long long rows = 1;
-        for (int i = 0; i < n_bin_dims - 1; ++i) rows = std::min(rows * (2ll * (n_bins_scalar + 1) + 1), 1ll << 40);
-        HGC_REQUIRE(rows < (1ll << 24), "n_bins = %d is too fine for %d binned dimensions (a shell of the walk would "
-                    "have %lld rows of bins, the limit is 2^24)", n_bins_scalar, n_bin_dims, rows);
+        for (int i = 0; i < n_bin_dims - 1; ++i) rows = std::min(rows * (n_bins_scalar + 1ll), 1ll << 40);
+        HGC_REQUIRE(rows < (1ll << 22), "n_bins = %d is too fine for %d binned dimensions (the grid would have %lld "
+                    "rows of bins, the limit is 2^22)", n_bins_scalar, n_bin_dims, rows);
     }
     if (n_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_coords && d_row_splits && d_indices && d_dist, "null pointer");
     const int use_direction = d_direction != nullptr;
-    const KnnPipelineLayout L = knn_layout(n_vert, n_coords, n_bin_dims, n_rs, n_bins_scalar, use_direction);
+    const KnnPipelineLayout L = knn_layout(n_vert, n_coords, grid, n_rs, use_direction);
     HGC_REQUIRE(L.total_bins_bound < (1ll << 31) - 2, "bin table overflows int32: fewer bins or events per call");
     if (!workspace || !aligned256(workspace) || workspace_bytes < L.total)
         return fail(HGC_ERR_WORKSPACE, "kNN pipeline workspace missing, misaligned or too small");
@@ -460,6 +490,7 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
     int *n_bins = reinterpret_cast<int *>(ws + L.n_bins);
     int *sorting = d_out_sorting ? d_out_sorting : reinterpret_cast<int *>(ws + L.sorting);
     int *bounds = reinterpret_cast<int *>(ws + L.bounds);
+    int *bin_starts = reinterpret_cast<int *>(ws + L.bin_starts);
     float *scoords = reinterpret_cast<float *>(ws + L.scoords);
     int *sflat = reinterpret_cast<int *>(ws + L.sflat);
     int *sbinass = reinterpret_cast<int *>(ws + L.sbinass);
@@ -469,11 +500,12 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
     // bin: its results are in the caller's index space and in canonical order.
     const int rc = bin_grouping(d_coords, d_row_splits, d_direction, n_vert, n_coords, n_bin_dims, n_rs, n_bins_scalar,
                                 L.total_bins_bound, shift, bin_width, n_bins, bounds, sorting, scoords, sflat, sbinass,
-                                sdir, ws + L.grouping_ws, L.total - L.grouping_ws, as_stream(stream));
+                                sdir, L.nested, bin_starts, ws + L.grouping_ws, L.total - L.grouping_ws, as_stream(stream));
     if (rc) return rc;
-    return binned_select_knn_strided(scoords, sflat, sdir, sbinass, bounds, bin_grouping_sub_shift(L.total_bins_bound),
-                                     n_bins, bin_width, sorting, shift, max_radius, d_indices, d_dist, n_vert, n_neigh,
-                                     n_coords, n_bin_dims, L.total_bins_bound + 1, tf_compat, use_direction,
+    return binned_select_knn_strided(scoords, sflat, sdir, sbinass, bin_starts, 0, n_bins, bin_width,
+                                     sorting, shift, max_radius, d_indices, d_dist, n_vert, n_neigh, n_coords,
+                                     n_bin_dims, L.total_bins_bound + 1, tf_compat, use_direction,
+                                     L.nested ? bounds : nullptr, L.nested ? n_bin_dims : 0, std::max(n_neigh - 1, 1) / kCrowdedBinFraction,
                                      as_stream(stream));
 }
 

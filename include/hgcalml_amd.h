@@ -70,8 +70,8 @@ enum hgc_data_flag {
     HGC_FLAG_COORDINATE_NOT_FINITE = 2,   /* NaN or Inf among the binned coordinates */
     HGC_FLAG_BIN_BEYOND_TABLE = 4,        /* kNN: a bin of the walk lies beyond d_bin_boundaries: skipped */
     HGC_FLAG_REPLACEMENT_OUT_OF_RANGE = 8, /* index replacer: entry >= n_replacements: left untouched */
-    HGC_FLAG_SHELL_TOO_WIDE = 16          /* kNN: a query's walk reached a shell of 2^24 or more rows of bins
-                                             ((2d+1)^(n_bin_dim-1) at shell distance d) and ended there */
+    HGC_FLAG_SHELL_TOO_WIDE = 16          /* kNN: a query's walk reached a shell of 2^22 or more rows of bins
+                                             inside the grid and within reach, and ended there */
 };
 int hgc_set_status_word(int *d_word);
 /* The calling thread's status word (NULL: none registered on this thread). */
@@ -163,10 +163,11 @@ int hgc_gather_rows(const void *d_in, const int *d_rows, void *d_out, int n_rows
  * Supported: 2 <= n_bin_dim <= 5, n_coords >= 2, n_neigh >= 1 without an upper
  * bound (up to 513 the sorted list lives in registers; beyond that the search
  * runs once per window of 512 ranks and is correspondingly slow),
- * n_vert * n_neigh < 2^31, coordinate matrix below 4 GiB. A shell at distance d is walked as (2d+1)^(n_bin_dim-1) rows of
- * bins; a query whose walk would reach a shell of 2^24 rows or more (grids far
- * finer than the points are dense, e.g. 5 binned dimensions with more than 30
- * bins each) ends there and sets HGC_FLAG_SHELL_TOO_WIDE in the status word;
+ * n_vert * n_neigh < 2^31, coordinate matrix below 4 GiB. A shell at distance d is walked as rows of
+ * bins along the last binned dimension, those of its (2d+1)^(n_bin_dim-1) rows that are inside
+ * the grid and within reach of the search; a query whose walk would reach a shell of 2^22 such
+ * rows or more (grids far finer than the points are dense, e.g. 5 binned dimensions with more
+ * than 45 bins each) ends there and sets HGC_FLAG_SHELL_TOO_WIDE in the status word;
  * without a registered status word that is silent and the rows of such queries
  * can miss neighbours (hgc_binned_select_knn_pipeline refuses such grids on the
  * host instead, whatever the status word). */
@@ -210,11 +211,14 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
  *
  * The neighbour sets of an exact search do not depend on the grid it walks, so
  * by default the pipeline searches on a grid of its own choice (up to four
- * binned dimensions, about one point per cell) and takes n_bins_scalar and
+ * binned dimensions, about one point per bin at 64 neighbours and finer for
+ * fewer; where every coordinate is binned, a second grid of half the bin width
+ * nested inside for the queries of crowded bins) and takes n_bins_scalar and
  * max_bin_dims only for the reference's argument checks; hgc_set_knn_grid(1)
  * makes the calling thread's later calls bin exactly as asked
  * (n_bins_scalar bins over min(max_bin_dims, n_coords) dimensions),
- * hgc_set_knn_grid(0) returns to the default. The workspace query covers both. */
+ * hgc_set_knn_grid(0) returns to the default. The workspace query covers both,
+ * for any number of neighbours. */
 int hgc_set_knn_grid(int use_callers_grid);
 /* The calling thread's setting (0: the library's own grid, the initial state). */
 int hgc_get_knn_grid(void);
@@ -236,12 +240,12 @@ int hgc_binned_select_knn_pipeline(const float *d_coords, const int *d_row_split
  * The call allocates and frees nothing. A problem whose
  * hgc_binned_select_knn_pipeline_workspace_bytes(...) exceeds
  * HGC_STATIC_SCRATCH_BYTES is refused with HGC_ERR_WORKSPACE (N = 150,000 points
- * with 4 coordinates, one event and n_bins = 30 need 19.3 MiB). All calls on
+ * with 4 coordinates, one event and n_bins = 30 need 42.1 MiB). All calls on
  * one GPU share that GPU's array: calls that overlap on one GPU (different
  * streams or threads) race and must be ordered by the caller. The first call on
  * a device looks the array's address up (hipGetSymbolAddress, under a lock):
  * make it outside a stream capture. */
-#define HGC_STATIC_SCRATCH_BYTES (32u << 20)
+#define HGC_STATIC_SCRATCH_BYTES (64u << 20)
 int hgc_binned_select_knn_pipeline_static(const float *d_coords, const int *d_row_splits,
                                           const int *d_direction, int n_vert, int n_coords, int n_rs,
                                           int n_neigh, int n_bins_scalar, int max_bin_dims, int tf_compat,

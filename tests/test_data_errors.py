@@ -177,7 +177,7 @@ def test_replacement_out_of_range_is_flagged_and_left_alone(debug_checks):
 
 @pytest.mark.gpu
 def test_too_fine_grid_is_refused_or_flagged():
-    """5 binned dimensions, 40 bins each: a shell of the walk would have (2*41+1)^4 > 2^24 rows"""
+    """5 binned dimensions, 48 bins each: the grid has 49^4 > 2^22 rows of bins, more than a shell of the walk may have"""
     from hgcalml_amd import BinnedSelectKnn
     from hgcalml_amd import globals as gl
     x = torch.rand((200, 5), device=DEV)
@@ -185,11 +185,11 @@ def test_too_fine_grid_is_refused_or_flagged():
     gl.knn_callers_grid = True          # bin exactly as asked
     try:
         with pytest.raises(ValueError, match="too fine"):
-            BinnedSelectKnn(4, x, rs, n_bins=40, max_bin_dims=5)
+            BinnedSelectKnn(4, x, rs, n_bins=48, max_bin_dims=5)
         idx, _ = BinnedSelectKnn(4, x, rs, n_bins=20, max_bin_dims=5)
     finally:
         gl.knn_callers_grid = False
     assert (idx[:, 0].cpu() == torch.arange(200)).all() and (idx >= 0).all()
     # on the library's own grid the same request is simply answered
-    idx2, _ = BinnedSelectKnn(4, x, rs, n_bins=40, max_bin_dims=5)
+    idx2, _ = BinnedSelectKnn(4, x, rs, n_bins=48, max_bin_dims=5)
     assert torch.equal(idx, idx2)
