@@ -255,6 +255,42 @@ def test_knn_dense_bins_long_candidate_lists(oracle, C, n_bins):
     run_knn_case(oracle, coords, rs, 20, n_bins)
 
 
+@pytest.mark.parametrize("case", ["blob4", "blob3", "blob2", "uniform4", "clumps", "clumps_radius", "edge"])
+def test_knn_nested_grid_cases(oracle, case):
+    """the library's own grid with every coordinate binned carries a nested grid of half the bin
+    width for the queries of crowded bins (more than (K-1)/4 points):
+    blob*: most queries walk it; uniform4: bins just above the threshold, shells of several
+    batches of segments while the list fills; clumps: tight groups of 20 points far from
+    everything else -- their walk on the nested grid gives up after a few shells and starts
+    again on the grid of bins; edge: crowded bins on the border of the grid"""
+    rng = np.random.default_rng({"blob4": 1, "blob3": 2, "blob2": 3, "uniform4": 4, "clumps": 5, "clumps_radius": 5,
+                                 "edge": 6}[case])
+    kw = {}
+    if case.startswith("blob"):
+        C = int(case[-1])
+        n, K = 30000, {4: 40, 3: 24, 2: 16}[C]
+        coords = rng.standard_normal((n, C)).astype(np.float32)
+    elif case == "uniform4":
+        n, K = 40000, 16
+        coords = rng.random((n, 4), dtype=np.float32)
+    elif case in ("clumps", "clumps_radius"):
+        centres = rng.random((30, 4), dtype=np.float32)
+        clumps = (centres[:, None, :] + 1e-3 * rng.standard_normal((30, 20, 4))).reshape(-1, 4).astype(np.float32)
+        coords = np.concatenate([clumps, rng.random((3000, 4), dtype=np.float32)])
+        coords = coords[rng.permutation(len(coords))]
+        n, K = len(coords), 64
+        if case == "clumps_radius":
+            kw = dict(max_radius=0.2, tf_compatible=True)
+    else:
+        corner = (1e-2 * rng.random((3000, 3))).astype(np.float32)                     # crowded bins at the lower corner
+        far = (1.0 - 1e-2 * rng.random((3000, 3))).astype(np.float32)                  # ... and at the upper one
+        coords = np.concatenate([corner, far, rng.random((6000, 3), dtype=np.float32)])
+        coords = coords[rng.permutation(len(coords))]
+        n, K = len(coords), 32
+    rs = np.array([0, n], np.int32) if case != "blob3" else np.array([0, 9000, 9000, n], np.int32)
+    run_knn_case(oracle, np.ascontiguousarray(coords), rs, K, 10, max_ties=1, **kw)
+
+
 def test_knn_small_events_direction_tf_compat(oracle):
     rng = np.random.default_rng(18)
     coords = rng.standard_normal((330, 3)).astype(np.float32)
