@@ -351,6 +351,7 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
     const float bw = s_bw;
     for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < n_vert; p += gridDim.x * blockDim.x) {
         int mul = 1, cell = 0, flags = 0, half = 0;
+        int ks[kMaxBinDims];
         for (int c = n_dims - 1; c >= 0; --c) {
             const float raw = coords[(size_t)p * stride + c];
             if (!isfinite(raw)) flags |= HGC_FLAG_COORDINATE_NOT_FINITE;
@@ -364,7 +365,7 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
             } else if (in_bins - (float)k >= 0.5f) {
                 half |= 1 << (n_dims - 1 - c);  // upper half of the bin in this dimension (last dimension: bit 0)
             }
-            binass[(size_t)p * (n_dims + 1) + c + 1] = k;
+            ks[c] = k;
             cell += k * mul;
             mul *= nb;
         }
@@ -380,7 +381,12 @@ __global__ __launch_bounds__(256) void bin_points_ranked_kernel(
         cell += ev * mul;
         if (flags && status) atomicOr(status, flags);
         cell = min(cell, n_bins_bound - 1);  // no effect for row splits that end at n_vert
-        binass[(size_t)p * (n_dims + 1)] = ev;
+        if (n_dims == 3) {  // one 16-byte row (the workspace is aligned)
+            reinterpret_cast<int4 *>(binass)[p] = make_int4(ev, ks[0], ks[1], ks[2]);
+        } else {
+            binass[(size_t)p * (n_dims + 1)] = ev;
+            for (int c = 0; c < n_dims; ++c) binass[(size_t)p * (n_dims + 1) + c + 1] = ks[c];
+        }
         // Every bin has 2^sub_shift counters, so that the increments of a crowded bin queue up on
         // several addresses instead of one. spatial (sub_shift = n_dims): the counter is the half of
         // the bin the point lies in, per dimension -- the bin's points then come grouped by these
@@ -412,10 +418,17 @@ __global__ __launch_bounds__(256) void move_to_bin_order_kernel(
     sflat[at] = cell;
     if (n_coords == 4 && rows_aligned) {
         reinterpret_cast<float4 *>(scoords)[at] = reinterpret_cast<const float4 *>(coords)[p];
+    } else if (n_coords == 3) {  // one 12-byte store per row instead of three of 4 bytes to a scattered address
+        struct __attribute__((packed, aligned(4))) Row3 { float v[3]; };
+        reinterpret_cast<Row3 *>(scoords)[at] = reinterpret_cast<const Row3 *>(coords)[p];
     } else {
         for (int c = 0; c < n_coords; ++c) scoords[(size_t)at * n_coords + c] = coords[(size_t)p * n_coords + c];
     }
-    for (int c = 0; c <= n_dims; ++c) sbinass[(size_t)at * (n_dims + 1) + c] = binass[(size_t)p * (n_dims + 1) + c];
+    if (n_dims == 3) {
+        reinterpret_cast<int4 *>(sbinass)[at] = reinterpret_cast<const int4 *>(binass)[p];
+    } else {
+        for (int c = 0; c <= n_dims; ++c) sbinass[(size_t)at * (n_dims + 1) + c] = binass[(size_t)p * (n_dims + 1) + c];
+    }
     if (direction) sdir[at] = direction[p];
 }
 
