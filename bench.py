@@ -153,11 +153,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--roofline-scale", type=float, default=1.0, help="shrink cfg4 (debugging only)")
-    ap.add_argument("--section", choices=["all", "headline", "roofline", "streams", "condensates"], default="all",
+    ap.add_argument("--section", choices=["all", "headline", "roofline", "streams", "condensates", "blob"], default="all",
                     help="run only one part (for profiling); the JSON line is printed for 'all' only. 'streams': the "
                          "cfg4 gradient next to its variants without the max half and without the weight gradient, "
                          "whose counter differences split its L2 requests by data stream. 'condensates': cfg5 alone, both "
-                         "assignment modes")
+                         "assignment modes. 'blob': the kNN search over the 4-D Gaussian blob alone")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build targets ONE GPU (no collectives, no sharding); run with --gpus 1. "
@@ -178,6 +178,12 @@ def main():
             m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode),
                           args.steps, args.warmup)
             log("bench: cfg5 condensates (%s) %.3f ms" % ("max-beta" if mode else "min-distance", m5[0]))
+        return
+    if args.section == "blob":
+        blob = torch.from_numpy(np.random.default_rng(5).standard_normal((150000, 4)).astype(np.float32)).to(dev)
+        rs_blob = torch.tensor([0, 150000], dtype=torch.int32, device=dev)
+        mb = event_ms(lambda: BinnedSelectKnn(65, blob, rs_blob, n_bins=30), args.steps, args.warmup)
+        log("bench: kNN over a 4-D Gaussian blob, N=150000, K=65: %.3f ms" % mb[0])
         return
     # ------------------------------------------------------------------ headline: cfg2
     c2 = workloads.cfg2()
