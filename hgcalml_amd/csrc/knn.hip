@@ -661,7 +661,7 @@ __device__ __forceinline__ bool walk_shells(const KnnParams &p, const int q, con
 // walk gives up), the others the grid of bins.
 template <int C, int NB, int S, bool MAPPED, bool WINDOW = false, bool NESTED = false>
 __global__ __launch_bounds__(kQueriesPerBlock * kWave)
-__attribute__((amdgpu_waves_per_eu((NESTED && S == 1) ? 8 : 1, 8)))
+__attribute__((amdgpu_waves_per_eu(S <= 2 ? 8 : 1, 8)))
 void knn_wave_kernel(const KnnParams p) {
     __shared__ __attribute__((aligned(8))) uint8_t mark_strips[kQueriesPerBlock][kMarkCap];
     const int lane = lane_id();
