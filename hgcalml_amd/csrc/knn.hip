@@ -746,7 +746,7 @@ int launch_levels(const KnnParams &p, hipStream_t s) {
         }
         return HGC_OK;
     }
-    if constexpr (MAPPED && C == NB && NB >= 2 && NB <= 4) {  // all coordinates binned: a crowded bin has its neighbours close by
+    if constexpr (MAPPED && C == NB && NB >= 3 && NB <= 4) {  // all coordinates binned: a crowded bin has its neighbours close by
         if (p.fine_bits > 0 && p.cell_boundaries) {
             switch (levels) {
                 case 1: knn_wave_kernel<C, NB, 1, MAPPED, false, true><<<grid, block, 0, s>>>(p); break;

@@ -43,7 +43,17 @@ namespace {
 //     KnnParams::fine_bits): with it the bins themselves can be wider than a single grid would
 //     want them, which is what sparse regions like (their shells are mostly empty bins). Measured
 //     kernel times, 150,000 points in 4-D, K = 64, single grid of 20 bins -> nested grid on 18 bins:
-//     clusters + noise 450 -> 425 us, Gaussian blob 825 -> 515 us, uniform 418 -> 351 us.
+//     clusters + noise 450 -> 425 us, Gaussian blob 825 -> 515 us, uniform 418 -> 351 us. The whole
+//     call with and without it on the same bins, in ms (150,000 points; the nested grid's table is
+//     2^dimensions times larger, and few neighbours come from few candidates either way):
+//                               K = 8          16            32            64            129
+//       4-D clusters + noise  0.43 / 0.28   0.38 / 0.31   0.40 / 0.37   0.47 / 0.47   0.86 / 0.86
+//       4-D Gaussian blob     0.35 / 0.32   0.38 / 0.38   0.44 / 0.52   0.56 / 0.82   1.04 / 1.86
+//       3-D clusters + noise  0.31 / 0.23   0.30 / 0.25   0.32 / 0.30   0.36 / 0.36   0.61 / 0.64
+//       3-D uniform           0.33 / 0.21   0.29 / 0.24   0.33 / 0.29   0.35 / 0.32   0.55 / 0.53
+//       3-D Gaussian blob     0.26 / 0.25   0.29 / 0.29   0.33 / 0.36   0.37 / 0.52   0.70 / 0.96
+//       2-D clusters + noise  0.28 / 0.22   0.30 / 0.27   0.36 / 0.33   0.36 / 0.35   0.60 / 0.59
+//     so it is taken from 48 neighbours on and three binned dimensions on.
 //   * Points with more than four coordinates keep three binned dimensions, and their bins hold
 //     every point along the others: the neighbourhood is wide in bin widths however fine the
 //     grid, so a coarser one, 0.6 (points per event)^(1/3), serves better (150,000 points,
@@ -67,6 +77,8 @@ SearchGrid callers_grid(int n_coords, int n_bins_scalar, int max_bin_dims) {
 constexpr int kSmallestGridK = 32, kLargestGridK = 64;
 // a bin with more than (K - 1) / kCrowdedBinFraction points sends its queries to the nested grid
 constexpr int kCrowdedBinFraction = 4;
+// fewer neighbours than this search on the single grid (see the table above own_grid)
+constexpr int kSmallestNestedK = 48;
 
 SearchGrid own_grid(int n_vert, int n_coords, int n_rs, int n_neigh) {
     const int dims = n_coords <= 4 ? n_coords : 3;
@@ -81,7 +93,7 @@ SearchGrid own_grid(int n_vert, int n_coords, int n_rs, int n_neigh) {
         n_bins = 0.6 * std::pow(per_event, 1.0 / dims);
     }
     return {dims, std::max(2, std::min((int)std::lround(n_bins), dims >= 4 ? 40 : dims == 3 ? 128 : 1024)),
-            dims == n_coords};
+            dims == n_coords && dims >= 3 && n_neigh >= kSmallestNestedK};
 }
 
 SearchGrid search_grid(int n_vert, int n_coords, int n_rs, int n_neigh, int n_bins_scalar, int max_bin_dims) {

@@ -212,8 +212,9 @@ int hgc_binned_select_knn_fused(const float *d_coord, const int *d_bin_idx, cons
  * The neighbour sets of an exact search do not depend on the grid it walks, so
  * by default the pipeline searches on a grid of its own choice (up to four
  * binned dimensions, about one point per bin at 64 neighbours and finer for
- * fewer; where every coordinate is binned, a second grid of half the bin width
- * nested inside for the queries of crowded bins) and takes n_bins_scalar and
+ * fewer; where all of three or four coordinates are binned and 48 neighbours or
+ * more are asked for, a second grid of half the bin width nested inside for the
+ * queries of crowded bins) and takes n_bins_scalar and
  * max_bin_dims only for the reference's argument checks; hgc_set_knn_grid(1)
  * makes the calling thread's later calls bin exactly as asked
  * (n_bins_scalar bins over min(max_bin_dims, n_coords) dimensions),

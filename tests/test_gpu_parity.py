@@ -255,24 +255,22 @@ def test_knn_dense_bins_long_candidate_lists(oracle, C, n_bins):
     run_knn_case(oracle, coords, rs, 20, n_bins)
 
 
-@pytest.mark.parametrize("case", ["blob4", "blob3", "blob2", "uniform4", "clumps", "clumps_radius", "edge"])
+@pytest.mark.parametrize("case", ["blob4", "blob3", "blob4_two_registers", "blob4_few_neighbours", "clumps",
+                                  "clumps_radius", "edge"])
 def test_knn_nested_grid_cases(oracle, case):
-    """the library's own grid with every coordinate binned carries a nested grid of half the bin
-    width for the queries of crowded bins (more than (K-1)/4 points):
-    blob*: most queries walk it; uniform4: bins just above the threshold, shells of several
-    batches of segments while the list fills; clumps: tight groups of 20 points far from
-    everything else -- their walk on the nested grid gives up after a few shells and starts
-    again on the grid of bins; edge: crowded bins on the border of the grid"""
-    rng = np.random.default_rng({"blob4": 1, "blob3": 2, "blob2": 3, "uniform4": 4, "clumps": 5, "clumps_radius": 5,
-                                 "edge": 6}[case])
+    """the library's own grid with every coordinate binned (three or four) carries, from 48 neighbours on, a nested
+    grid of half the bin width for the queries of crowded bins (more than (K-1)/4 points):
+    blob*: most queries walk it, with one and with two list registers per lane (blob4_few_neighbours: K below 48,
+    the same points on the single grid); clumps: tight groups of 20 points far from everything else -- their walk on
+    the nested grid gives up after a few shells and starts again on the grid of bins; edge: crowded bins on the border
+    of the grid. Shells of several batches of segments while the list fills occur in all of them."""
+    rng = np.random.default_rng({"blob4": 1, "blob3": 2, "blob4_two_registers": 3, "blob4_few_neighbours": 1, "clumps": 5,
+                                 "clumps_radius": 5, "edge": 6}[case])
     kw = {}
     if case.startswith("blob"):
-        C = int(case[-1])
-        n, K = 30000, {4: 40, 3: 24, 2: 16}[C]
+        C = int(case[4])
+        n, K = 30000, {"blob4": 64, "blob3": 56, "blob4_two_registers": 100, "blob4_few_neighbours": 40}[case]
         coords = rng.standard_normal((n, C)).astype(np.float32)
-    elif case == "uniform4":
-        n, K = 40000, 16
-        coords = rng.random((n, 4), dtype=np.float32)
     elif case in ("clumps", "clumps_radius"):
         centres = rng.random((30, 4), dtype=np.float32)
         clumps = (centres[:, None, :] + 1e-3 * rng.standard_normal((30, 20, 4))).reshape(-1, 4).astype(np.float32)
@@ -286,7 +284,7 @@ def test_knn_nested_grid_cases(oracle, case):
         far = (1.0 - 1e-2 * rng.random((3000, 3))).astype(np.float32)                  # ... and at the upper one
         coords = np.concatenate([corner, far, rng.random((6000, 3), dtype=np.float32)])
         coords = coords[rng.permutation(len(coords))]
-        n, K = len(coords), 32
+        n, K = len(coords), 48
     rs = np.array([0, n], np.int32) if case != "blob3" else np.array([0, 9000, 9000, n], np.int32)
     run_knn_case(oracle, np.ascontiguousarray(coords), rs, K, 10, max_ties=1, **kw)
 
