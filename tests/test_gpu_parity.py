@@ -915,7 +915,7 @@ def test_push_knn_matrices_beyond_2_to_31_elements():
 
 # ------------------------------------------------------------------ ops next to the accumulation
 
-@pytest.mark.parametrize("K,C", [(16, 3), (64, 4), (5, 8)])
+@pytest.mark.parametrize("K,C", [(16, 3), (64, 4), (5, 8), (7, 2), (33, 4)])
 def test_select_knn_grad(oracle, K, C):
     rng = np.random.default_rng(50 + K)
     n = 3000
@@ -928,6 +928,12 @@ def test_select_knn_grad(oracle, K, C):
     ref = oracle.select_knn_grad_kernel(g, idx, x)
     got = torch.ops.hgcalml.select_knn_grad(t(g), t(idx), t(np.zeros_like(g)), t(x))
     # same terms in the same order as the oracle: identical bits
+    assert (bits(got.cpu().numpy()) == bits(ref)).all()
+    # a coordinate matrix that does not start on a 16-byte boundary (a view into a larger buffer)
+    buf = torch.zeros(n * C + 1, dtype=torch.float32, device=DEV)
+    shifted = buf[1:].view(n, C)
+    shifted.copy_(t(x))
+    got = torch.ops.hgcalml.select_knn_grad(t(g), t(idx), t(np.zeros_like(g)), shifted)
     assert (bits(got.cpu().numpy()) == bits(ref)).all()
 
 
