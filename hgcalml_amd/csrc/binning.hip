@@ -432,6 +432,13 @@ __global__ __launch_bounds__(256) void move_to_bin_order_kernel(
 // front of it and scans itself): a few thousand chunks at most, and no chunk waits for another
 // as in a single-pass scan with look-back (2.5 M counters: 9 us against 19 us for the library scan).
 constexpr int kScanChunk = 2048;  // 256 threads x 8 counters
+constexpr int kMaxScanChunks = 16384;
+
+__global__ __launch_bounds__(256) void strided_copy_kernel(const int *__restrict__ in, int *__restrict__ out, int n,
+                                                           int shift) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = in[(size_t)i << shift];
+}
 
 __global__ __launch_bounds__(256) void counter_chunk_sums_kernel(const int *__restrict__ counts, long long n,
                                                                  int *__restrict__ chunk_sums) {
@@ -549,10 +556,21 @@ static size_t grouping_counters(int n_bins_bound, int n_bin_dims, bool spatial) 
     return ((size_t)n_bins_bound << bin_grouping_sub_shift(n_bins_bound, n_bin_dims, spatial)) + 1;
 }
 
+// scratch of the boundary table's scan: the chunk sums, or the library scan's own for tables of more
+// than kMaxScanChunks chunks
+static size_t scan_scratch_bytes(size_t n_counters) {
+    const size_t n_chunks = (n_counters + kScanChunk - 1) / kScanChunk;
+    if (n_chunks <= (size_t)kMaxScanChunks) return n_chunks * sizeof(int);
+    size_t temp = 0;
+    (void)rocprim::exclusive_scan(nullptr, temp, (const int *)nullptr, (int *)nullptr, 0, n_counters,
+                                  rocprim::plus<int>(), (hipStream_t) nullptr);
+    return temp;
+}
+
 size_t bin_grouping_workspace_bytes(int n_vert, int n_bins_bound, int n_bin_dims, bool spatial) {
     const size_t n = std::max(n_vert, 1);
     const size_t n_counters = grouping_counters(n_bins_bound, n_bin_dims, spatial);
-    return align_up(ceil_div(n_counters, (size_t)kScanChunk) * sizeof(int)) +
+    return align_up(scan_scratch_bytes(n_counters)) +
            align_up((size_t)grouping_blocks(n_vert) * 2 * kMaxBinDims * sizeof(float)) +
            align_up(n_counters * sizeof(int)) + 2 * align_up(n * sizeof(int)) +
            align_up(n * (kMaxBinDims + 1) * sizeof(int));
@@ -577,7 +595,8 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
     int *rank = carve.take<int>(n_vert);
     int *binass = carve.take<int>((size_t)n_vert * (kMaxBinDims + 1));
     const int n_chunks = (int)ceil_div(n_counters, (size_t)kScanChunk);
-    int *chunk_sums = carve.take<int>(n_chunks);
+    size_t scan_temp_bytes = scan_scratch_bytes(n_counters);
+    int *chunk_sums = reinterpret_cast<int *>(carve.take<char>(scan_temp_bytes));
     column_minmax_kernel<<<blocks, 256, 0, s>>>(d_coords, n_coords, n_vert, n_bin_dims, partial, counts,
                                                 (long long)n_counters);
     int rc = check_launch("column_minmax");
@@ -589,10 +608,20 @@ int bin_grouping(const float *d_coords, const int *d_row_splits, const int *d_di
     rc = check_launch("bin_points_ranked");
     if (rc) return rc;
     // boundaries[b << sub_shift] = number of points in bins below b
-    counter_chunk_sums_kernel<<<n_chunks, 256, 0, s>>>(counts, (long long)n_counters, chunk_sums);
-    counter_scan_kernel<<<n_chunks, 256, 0, s>>>(counts, (long long)n_counters, chunk_sums, d_boundaries, d_bin_starts,
-                                                 sub_shift);
-    rc = check_launch("counter_scan");
+    if (n_chunks <= kMaxScanChunks) {
+        counter_chunk_sums_kernel<<<n_chunks, 256, 0, s>>>(counts, (long long)n_counters, chunk_sums);
+        counter_scan_kernel<<<n_chunks, 256, 0, s>>>(counts, (long long)n_counters, chunk_sums, d_boundaries,
+                                                     d_bin_starts, sub_shift);
+        rc = check_launch("counter_scan");
+    } else {  // every chunk adds up the sums in front of it: quadratic in the chunks, so huge tables take the library scan
+        HGC_HIP(rocprim::exclusive_scan(chunk_sums, scan_temp_bytes, counts, d_boundaries, 0, n_counters,
+                                        rocprim::plus<int>(), s));
+        if (d_bin_starts) {
+            strided_copy_kernel<<<ceil_div((long long)n_bins_bound + 1, 256), 256, 0, s>>>(d_boundaries, d_bin_starts,
+                                                                                          n_bins_bound + 1, sub_shift);
+        }
+        rc = check_launch("bin boundary table");
+    }
     if (rc) return rc;
     const int rows_aligned =
         ((reinterpret_cast<uintptr_t>(d_coords) | reinterpret_cast<uintptr_t>(d_scoords)) & 15u) == 0;

@@ -289,6 +289,25 @@ def test_knn_nested_grid_cases(oracle, case):
     run_knn_case(oracle, np.ascontiguousarray(coords), rs, K, 10, max_ties=1, **kw)
 
 
+def test_knn_bin_table_beyond_the_two_pass_scan(oracle):
+    """a caller's grid of 331^3 bins: the boundary table has more chunks than the grouping's own two-pass scan
+    takes and goes through the library scan instead; few points, so every row is checked by brute force"""
+    from hgcalml_amd import BinnedSelectKnn
+    from hgcalml_amd import globals as gl
+    from helpers import check_knn_rows
+    rng = np.random.default_rng(77)
+    n, K = 1500, 8
+    coords = rng.random((n, 3), dtype=np.float32)
+    coords[: n // 2] = 0.5 + 1e-3 * rng.standard_normal((n // 2, 3)).astype(np.float32)   # neighbours within a few bins
+    rs = np.array([0, n], np.int32)
+    gl.knn_callers_grid = True
+    try:
+        idx, dist = BinnedSelectKnn(K, t(coords), t(rs), n_bins=330, max_radius=0.02)
+    finally:
+        gl.knn_callers_grid = False
+    assert check_knn_rows(oracle, idx.cpu().numpy(), dist.cpu().numpy(), coords, rs, K, np.arange(n), radius=0.02) == 0
+
+
 def test_knn_small_events_direction_tf_compat(oracle):
     rng = np.random.default_rng(18)
     coords = rng.standard_normal((330, 3)).astype(np.float32)
