@@ -59,11 +59,10 @@ __host__ __device__ __forceinline__ uint32_t owner_reg(uint32_t f, int vec) {
 
 // ---- pass 1: records ---------------------------------------------------------
 
-// the lanes among `active` whose `digit` agrees with this lane's in its low 8 bits
-__device__ __forceinline__ uint64_t same_byte_lanes(uint32_t digit, uint64_t active) {
+// the lanes among `active` whose `digit` agrees with this lane's in its low `n_bits` bits
+__device__ __forceinline__ uint64_t same_byte_lanes(uint32_t digit, uint64_t active, int n_bits) {
     uint64_t peers = active;
-#pragma unroll
-    for (int b = 0; b < 8; ++b) {
+    for (int b = 0; b < n_bits; ++b) {
         const bool set = (digit >> b) & 1u;
         const uint64_t with = __ballot(set);
         peers &= set ? with : ~with;
@@ -102,6 +101,7 @@ __global__ __launch_bounds__(256) void hit_records_kernel(const float *__restric
     wave_lds_fence();
     const unsigned char *srow = maxslot + (size_t)v * F;
     const float *grow = g + (size_t)v * 2 * F + F;
+    const int slot_bits = 32 - __builtin_clz((unsigned)max(K - 1, 1));
     int slot[BLOCKS], rank[BLOCKS];
     float gv[BLOCKS];
 #pragma unroll
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256) void hit_records_kernel(const float *__restric
 #pragma unroll
     for (int b = 0; b < BLOCKS; ++b) {
         const bool valid = slot[b] < K;  // 255: the feature has no arg-max slot
-        const uint64_t peers = same_byte_lanes((uint32_t)slot[b], __ballot(valid));
+        const uint64_t peers = same_byte_lanes((uint32_t)slot[b], __ballot(valid), slot_bits);  // valid slots are below K
         const int among = lanes_below(peers);
         const int before = valid ? count[slot[b]] : 0;
         __builtin_amdgcn_wave_barrier();
