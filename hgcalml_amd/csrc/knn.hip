@@ -22,12 +22,17 @@
 //   * The K-1 best keys live in registers, sorted across the lanes (rank r in
 //     lane r%64, register r/64). A ballot finds the candidates that beat the
 //     current K-th key; each is inserted with one DPP wave shift and two
-//     compares, and the new K-th key is read back with a readlane. When 16 or
+//     compares, and the new K-th key is read back with a readlane. When 20 or
 //     more of a step's 64 candidates enter (the first steps of every query), the
 //     step is sorted across the lanes by a bitonic network and merged into the
 //     list in one go instead.
 //   * The shell loop stops exactly as the reference does: list full and
 //     ((bw*d)*bw)*d > K-th distance, or no bin of the shell inside the grid.
+//   * Only the rows of a shell that lie inside the grid and within reach of the
+//     search get a slot: one per row on a face of the shell (its run), one or
+//     two per inner row (its end caps).
+//   * Optionally (callers that group the points by half-bin cells) the queries of
+//     crowded bins walk a nested grid of half the bin width: walk_shells<FINE>.
 //   * The kernel is bound by vector ALU issue; LDS holds only the marks. No
 //     atomics, no barriers; every wave is its own workgroup and exits on its own.
 #include "hgc_common.hpp"
