@@ -464,7 +464,12 @@ __device__ __forceinline__ bool walk_shells(const KnnParams &p, const int q, con
             const bool runs_only = d == 0 || (d == 1 && with_own_bin);
             const int n_slots = d == 0 ? 1 : FINE ? n_rows * P : (!runs_only && low_caps && high_caps) ? n_rows + n_inner : n_rows;
 
-            for (int slot0 = 0; slot0 < n_slots; slot0 += kWave) {
+            // batches of 64 slots, from the middle of the numbering outwards: the rows with small
+            // leading offsets, the nearer ones, come first (1 to 2 % of the kernel time)
+            const int n_batches = (n_slots + kWave - 1) / kWave;
+            for (int turn = 0; turn < n_batches; ++turn) {
+                const int mid = (n_batches - 1) >> 1;
+                const int slot0 = kWave * ((turn & 1) ? mid + ((turn + 1) >> 1) : mid - (turn >> 1));
                 // ---- each lane resolves one segment of the shell ----
                 int seg_start = 0, seg_len = 0;
                 bool far_segment = false;  // walked after the near ones of its batch
