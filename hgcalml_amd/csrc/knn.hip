@@ -261,8 +261,10 @@ constexpr int kBulkInsertMin = 20;
 // lists of more runs than this would insert one by one (a merge costs 12 more steps per run)
 constexpr int kBulkInsertMaxRuns = 8;
 
-// Segments of a batch whose bins are at least sqrt(kNearFirst) * d bin widths away (shell d) are
-// walked after the nearer ones (150,000 points in 4-D, K = 64, kernel: Gaussian blob 508 us without,
+// NEAR_FIRST (the kernels of the nested grid, i.e. 48 neighbours and more: 16 events of 3-D points
+// with K = 32 and a radius ran 4 % slower with it): segments of a batch whose bins are at least
+// sqrt(kNearFirst) * d bin widths away (shell d) are walked after the nearer ones
+// (150,000 points in 4-D, K = 64, kernel: Gaussian blob 508 us without,
 // 455 / 464 / 464 / 473 us at 0.3 / 0.45 / 0.6 / 0.75; clusters + noise 409, 407 / 405 / 413 / 418;
 // uniform 347, 359 / 352 / 347 / 354)
 constexpr float kNearFirst = 0.45f;
@@ -302,7 +304,7 @@ __device__ __forceinline__ void divmod_small(int x, int w, float inv_w, int &q, 
 // being binned, that is the rule where the bin's neighbourhood is about as crowded as the bin.
 constexpr int kFineMaxShell = 3;
 
-template <int C, int NB, int S, bool MAPPED, bool WINDOW, bool FINE>
+template <int C, int NB, int S, bool MAPPED, bool WINDOW, bool FINE, bool NEAR_FIRST>
 __device__ __forceinline__ bool walk_shells(const KnnParams &p, const int q, const int lane, uint8_t *const marks,
                                             const int Kn, const uint64_t floor_key, uint64_t (&key)[S]) {
     constexpr int kDims = NB > 0 ? NB : kMaxBinDims;  // array extents
@@ -464,15 +466,18 @@ __device__ __forceinline__ bool walk_shells(const KnnParams &p, const int q, con
             const bool runs_only = d == 0 || (d == 1 && with_own_bin);
             const int n_slots = d == 0 ? 1 : FINE ? n_rows * P : (!runs_only && low_caps && high_caps) ? n_rows + n_inner : n_rows;
 
-            // batches of 64 slots, from the middle of the numbering outwards: the rows with small
-            // leading offsets, the nearer ones, come first (1 to 2 % of the kernel time)
+            // batches of 64 slots; NEAR_FIRST: from the middle of the numbering outwards, so that the rows
+            // with small leading offsets, the nearer ones, come first (1 to 2 % of the kernel time)
             const int n_batches = (n_slots + kWave - 1) / kWave;
-            for (int turn = 0; turn < n_batches; ++turn) {
-                const int mid = (n_batches - 1) >> 1;
-                const int slot0 = kWave * ((turn & 1) ? mid + ((turn + 1) >> 1) : mid - (turn >> 1));
+            for (int slot_lin = 0, turn = 0; slot_lin < n_slots; slot_lin += kWave, ++turn) {
+                int slot0 = slot_lin;
+                if constexpr (NEAR_FIRST) {
+                    const int mid = (n_batches - 1) >> 1;
+                    slot0 = kWave * ((turn & 1) ? mid + ((turn + 1) >> 1) : mid - (turn >> 1));
+                }
                 // ---- each lane resolves one segment of the shell ----
                 int seg_start = 0, seg_len = 0;
-                bool far_segment = false;  // walked after the near ones of its batch
+                [[maybe_unused]] bool far_segment = false;  // NEAR_FIRST: walked after the near ones of its batch
                 const int slot = slot0 + lane;
                 // Nothing farther than `reach2` can still enter the list (K-th distance
                 // once the list is full, the radius cut otherwise). A bin at offset o
@@ -542,7 +547,7 @@ __device__ __forceinline__ bool walk_shells(const KnnParams &p, const int q, con
                     int lo = on_face ? run_lo : cap;
                     int hi = on_face ? run_hi : cap;
                     bool too_far = on_face ? 0.999f * gap2 > reach2 : (piece > 1 || 0.999f * cap2 > reach2);
-                    far_segment = (on_face ? gap2 : cap2) > near2;
+                    if constexpr (NEAR_FIRST) far_segment = (on_face ? gap2 : cap2) > near2;
                     lo = max(lo, 0);
                     hi = min(hi, nb_last - 1);
                     if (FINE) {
@@ -582,12 +587,21 @@ __device__ __forceinline__ bool walk_shells(const KnnParams &p, const int q, con
                 // The segments whose lower bound of the distance is within near2 come first in the
                 // candidate list, the others behind them (marks 65..128, so that the prefix maximum
                 // keeps the two apart): fewer candidates enter the list only to be pushed out again.
-                const int end_near = wave_inclusive_sum(far_segment ? 0 : seg_len);
-                const int end_far = wave_inclusive_sum(far_segment ? seg_len : 0);
-                const int total_near = readlane_i32(end_near, kWave - 1);
-                const int seg_off = (far_segment ? total_near + end_far : end_near) - seg_len;
-                const int total = total_near + readlane_i32(end_far, kWave - 1);
-                const uint8_t mark = (uint8_t)(lane + (far_segment ? kWave + 1 : 1));
+                int seg_off, total;
+                uint8_t mark;
+                if constexpr (NEAR_FIRST) {
+                    const int end_near = wave_inclusive_sum(far_segment ? 0 : seg_len);
+                    const int end_far = wave_inclusive_sum(far_segment ? seg_len : 0);
+                    const int total_near = readlane_i32(end_near, kWave - 1);
+                    seg_off = (far_segment ? total_near + end_far : end_near) - seg_len;
+                    total = total_near + readlane_i32(end_far, kWave - 1);
+                    mark = (uint8_t)(lane + (far_segment ? kWave + 1 : 1));
+                } else {
+                    const int seg_end_off = wave_inclusive_sum(seg_len);
+                    seg_off = seg_end_off - seg_len;
+                    total = readlane_i32(seg_end_off, kWave - 1);
+                    mark = (uint8_t)(lane + 1);
+                }
                 // candidate position -> point index for the owning segment; kept one lane up,
                 // so that the mark (lane number + 1) is the lane to read it from
                 // (DPP wave_ror:1; lane 63's value goes to lane 0, which is where mark 64 reads)
@@ -731,14 +745,14 @@ void knn_wave_kernel(const KnnParams p) {
     if (searching) {
         if constexpr (NESTED) {
             if (!crowded) {
-                walk_shells<C, NB, S, MAPPED, WINDOW, false>(p, q, lane, marks, Kn, floor_key, key);
-            } else if (!walk_shells<C, NB, S, MAPPED, WINDOW, true>(p, q, lane, marks, Kn, floor_key, key)) {
+                walk_shells<C, NB, S, MAPPED, WINDOW, false, NESTED>(p, q, lane, marks, Kn, floor_key, key);
+            } else if (!walk_shells<C, NB, S, MAPPED, WINDOW, true, NESTED>(p, q, lane, marks, Kn, floor_key, key)) {
 #pragma unroll
                 for (int s = 0; s < S; ++s) key[s] = kEmptyKey;
-                walk_shells<C, NB, S, MAPPED, WINDOW, false>(p, q, lane, marks, Kn, floor_key, key);
+                walk_shells<C, NB, S, MAPPED, WINDOW, false, NESTED>(p, q, lane, marks, Kn, floor_key, key);
             }
         } else {
-            walk_shells<C, NB, S, MAPPED, WINDOW, false>(p, q, lane, marks, Kn, floor_key, key);
+            walk_shells<C, NB, S, MAPPED, WINDOW, false, NESTED>(p, q, lane, marks, Kn, floor_key, key);
         }
     }
 
