@@ -807,14 +807,19 @@ int launch_levels(const KnnParams &p, hipStream_t s) {
     return check_launch("knn_wave_kernel");
 }
 
-// The usual shapes (binned dimensions = min(3, coordinates), up to 8 coordinates) get kernels with
-// both numbers fixed at compile time, anything else the one that reads them.
+// The usual shapes (up to 8 coordinates; binned dimensions = min(3, coordinates), the reference
+// wrapper's default, or min(4, coordinates), the pipeline's own grid) get kernels with both
+// numbers fixed at compile time, anything else the one that reads them.
 template <bool MAPPED>
 int launch_coords(const KnnParams &p, hipStream_t s) {
     if (p.n_coords == 2 && p.n_bin_dim == 2) return launch_levels<2, 2, MAPPED>(p, s);
     if (p.n_coords == 3 && p.n_bin_dim == 3) return launch_levels<3, 3, MAPPED>(p, s);
     if (p.n_coords == 4 && p.n_bin_dim == 3) return launch_levels<4, 3, MAPPED>(p, s);
     if (p.n_coords == 4 && p.n_bin_dim == 4) return launch_levels<4, 4, MAPPED>(p, s);
+    if (p.n_coords == 5 && p.n_bin_dim == 4) return launch_levels<5, 4, MAPPED>(p, s);
+    if (p.n_coords == 6 && p.n_bin_dim == 4) return launch_levels<6, 4, MAPPED>(p, s);
+    if (p.n_coords == 7 && p.n_bin_dim == 4) return launch_levels<7, 4, MAPPED>(p, s);
+    if (p.n_coords == 8 && p.n_bin_dim == 4) return launch_levels<8, 4, MAPPED>(p, s);
     if (p.n_coords == 5 && p.n_bin_dim == 3) return launch_levels<5, 3, MAPPED>(p, s);
     if (p.n_coords == 6 && p.n_bin_dim == 3) return launch_levels<6, 3, MAPPED>(p, s);
     if (p.n_coords == 7 && p.n_bin_dim == 3) return launch_levels<7, 3, MAPPED>(p, s);

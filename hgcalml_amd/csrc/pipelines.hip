@@ -54,11 +54,12 @@ namespace {
 //       3-D Gaussian blob     0.26 / 0.25   0.29 / 0.29   0.33 / 0.36   0.37 / 0.52   0.70 / 0.96
 //       2-D clusters + noise  0.28 / 0.22   0.30 / 0.27   0.36 / 0.33   0.36 / 0.35   0.60 / 0.59
 //     so it is taken from 48 neighbours on and three binned dimensions on.
-//   * Points with more than four coordinates keep three binned dimensions, and their bins hold
-//     every point along the others: the neighbourhood is wide in bin widths however fine the
-//     grid, so a coarser one, 0.6 (points per event)^(1/3), serves better (150,000 points,
-//     K = 64, uniform / Gaussian: 5-D 2.46 / 1.81 ms at 53 bins -> 1.4 / 1.8 ms at 32; 8-D 14.7 /
-//     8.4 -> 7.9 / 8.0 ms).
+//   * Points with more than four coordinates bin the first four, on the same rule (their bins hold
+//     every point along the other coordinates, so the neighbourhood is wide in bin widths however
+//     fine the grid; a nested grid does not pay there). 150,000 points, K = 64, three binned
+//     dimensions at 32 bins -> four at 18: 5-D Gaussian 2.07 -> 1.45 ms, 6-D Gaussian 2.91 -> 2.20 ms,
+//     6-D uniform 2.24 -> 1.62 ms, 8-D Gaussian 7.40 -> 5.85 ms. (Gaussians like more bins still,
+//     uniform boxes fewer: 24 / 11 bins give 1.17 / 2.32, 2.08 / 3.71, 2.71 / 1.23, 5.95 / 7.70 ms.)
 //   * Small events want fewer bins than that (most of a small grid is boundary): 200,000 uniform
 //     4-D points in 1000 events, K = 64: 0.80 ms at 4 bins, 0.52 at 3; in 4000 events 1.07 ms at
 //     4 bins, 0.31 at 2.
@@ -81,17 +82,12 @@ constexpr int kCrowdedBinFraction = 4;
 constexpr int kSmallestNestedK = 48;
 
 SearchGrid own_grid(int n_vert, int n_coords, int n_rs, int n_neigh) {
-    const int dims = n_coords <= 4 ? n_coords : 3;
+    const int dims = std::min(n_coords, 4);
     const double per_event = std::max(1.0, (double)n_vert / std::max(1, n_rs - 1));
     // small events: 0.75 of the rule up to 5,000 points per event, rising to 1 at 50,000
     const double small = std::min(1.0, std::max(0.75, 0.75 + 0.25 * (std::log10(per_event) - 3.7)));
-    double n_bins;
-    if (n_coords <= 4) {
-        const double k = std::min(std::max(n_neigh, kSmallestGridK), kLargestGridK);
-        n_bins = 0.9 * small * std::pow(per_event * 64.0 / k, 1.0 / dims);
-    } else {
-        n_bins = 0.6 * std::pow(per_event, 1.0 / dims);
-    }
+    const double k = std::min(std::max(n_neigh, kSmallestGridK), kLargestGridK);
+    const double n_bins = 0.9 * small * std::pow(per_event * 64.0 / k, 1.0 / dims);
     return {dims, std::max(2, std::min((int)std::lround(n_bins), dims >= 4 ? 40 : dims == 3 ? 128 : 1024)),
             dims == n_coords && dims >= 3 && n_neigh >= kSmallestNestedK};
 }
