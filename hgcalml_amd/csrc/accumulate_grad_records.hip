@@ -46,9 +46,10 @@ constexpr uint32_t kNoLane = 0xffu;  // key of a hit place that is empty
 
 // Which lane of the gather pass owns feature f, and in which of its registers
 // (VEC consecutive features per lane in blocks of 64 * VEC features).
-__host__ __device__ __forceinline__ uint32_t owner_lane(uint32_t f, int vec) { return (f / vec) & (kWave - 1); }
+// (vec is 1 or 2: written with shifts, the pass that builds the records gets it at run time)
+__host__ __device__ __forceinline__ uint32_t owner_lane(uint32_t f, int vec) { return (f >> (vec - 1)) & (kWave - 1); }
 __host__ __device__ __forceinline__ uint32_t owner_reg(uint32_t f, int vec) {
-    return f / (kWave * vec) * vec + f % vec;
+    return ((f >> (5 + vec)) << (vec - 1)) + (f & (uint32_t)(vec - 1));
 }
 
 // record of flat slot s at records[2*s], records[2*s+1]:
