@@ -287,9 +287,9 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
         float mean[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; ++e) mean[e] = sum[e] / kf;
-        store_vec<VEC>(out + (size_t)v * out_cols + fb, mean);
+        store_vec_once<VEC>(out + (size_t)v * out_cols + fb, mean);
         if (MAX) {
-            store_vec<VEC>(out + (size_t)v * out_cols + F + fb, best);
+            store_vec_once<VEC>(out + (size_t)v * out_cols + F + fb, best);
             int argidx[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) argidx[e] = arg[e] < 0 ? 0 : irow[arg[e]];

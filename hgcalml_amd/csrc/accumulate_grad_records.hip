@@ -158,8 +158,8 @@ __global__ __launch_bounds__(256) void hit_records_kernel(const float *__restric
         r1.y = dense ? bits[4 * n + 2] : __float_as_uint(vv[2]);
         r1.z = dense ? bits[4 * n + 3] : __float_as_uint(vv[3]);
         r1.w = __float_as_uint(vv[4]);
-        records[2 * s] = r0;
-        records[2 * s + 1] = r1;
+        store_once(records + 2 * s, r0);  // 2 KB per vertex, read back much later by the gather
+        store_once(records + 2 * s + 1, r1);
     }
 }
 
@@ -391,7 +391,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
         lane_bytes[b] = in_row ? (uint32_t)fb * 4u : kOutOfRange;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) xo[b][e] = 0.f;
-        if (in_row) load_vec<VEC>(feat + (size_t)m * F + fb, xo[b]);
+        if (in_row) load_vec_once<VEC>(feat + (size_t)m * F + fb, xo[b]);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
             tab.own[fb + e] = xo[b][e];
@@ -485,7 +485,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
-        if (!PARTIAL || lane_bytes[b] != kOutOfRange) store_vec<VEC>(gfeat + (size_t)m * F + (lane_bytes[b] >> 2), acc[b]);
+        if (!PARTIAL || lane_bytes[b] != kOutOfRange) store_vec_once<VEC>(gfeat + (size_t)m * F + (lane_bytes[b] >> 2), acc[b]);
 }
 
 template <int VEC, int NB, bool PARTIAL>

@@ -71,6 +71,43 @@ __device__ __forceinline__ void store_vec_i(int *p, const int (&x)[VEC]) {
 
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// The same for data that is touched once (a vertex's own row, its result row): the
+// non-temporal hint keeps such lines from pushing re-used rows out of L2.
+template <int VEC>
+__device__ __forceinline__ void load_vec_once(const float *p, float (&x)[VEC]) {
+    static_assert(VEC == 1 || VEC == 2, "one or two features per lane");
+    if constexpr (VEC == 2) {
+        const f32x2 v = __builtin_nontemporal_load(reinterpret_cast<const f32x2 *>(p));
+        x[0] = v.x; x[1] = v.y;
+    } else {
+        x[0] = __builtin_nontemporal_load(p);
+    }
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_vec_once(float *p, const float (&x)[VEC]) {
+    static_assert(VEC == 1 || VEC == 2 || VEC == 4, "one, two or four features per lane");
+    if constexpr (VEC == 4) {
+        f32x4 v;
+        v.x = x[0]; v.y = x[1]; v.z = x[2]; v.w = x[3];
+        __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p));
+    } else if constexpr (VEC == 2) {
+        f32x2 v;
+        v.x = x[0]; v.y = x[1];
+        __builtin_nontemporal_store(v, reinterpret_cast<f32x2 *>(p));
+    } else {
+        __builtin_nontemporal_store(x[0], p);
+    }
+}
+
+__device__ __forceinline__ void store_once(uint4 *p, const uint4 &x) {
+    u32x4 v;
+    v.x = x.x; v.y = x.y; v.z = x.z; v.w = x.w;
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+}
 
 __device__ __forceinline__ int wave_vertex() {
     const int tile = xcd_contiguous_block(blockIdx.x, gridDim.x);
