@@ -366,7 +366,7 @@ __device__ __forceinline__ void records_group(const RowMatrix &Gm, const BatchTa
 template <int VEC, int NB, bool POW2K, bool PARTIAL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) void accumulate_grad_records_kernel(
     const float *__restrict__ g, const float *__restrict__ feat, const uint4 *__restrict__ records,
-    const int *__restrict__ inv_off, const int *__restrict__ inv_slots, float *__restrict__ gw,
+    const int *__restrict__ inv_off, const int *__restrict__ inv_slots, float *__restrict__ gw_list,
     float *__restrict__ gfeat, int n_vert, int K, int F, const FastDiv div_k, const int *__restrict__ idx,
     const int *__restrict__ order, const float kf) {
     constexpr int Q = VEC * NB;
@@ -466,6 +466,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
         const uint64_t dense_mask = __ballot(dense && lane < cnt);
         const uint64_t many_mask = __ballot(n_hits > 2u && lane < cnt);
         wave_lds_fence();
+        float dot = 0.f;  // lane L: the mean part of entry L's weight gradient
         for (int c0 = 0; c0 < cnt; c0 += kGroup) {
             float val[kGroup];
 #pragma unroll
@@ -477,11 +478,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
                 records_group<VEC, NB, POW2K, false>(Gm, tab, lane_bytes, max_col_bytes, c0, cnt, dense_mask, many_mask,
                                                      xo, xk, acc, kf, val);
             const float r = transpose_reduce_group(val);  // lane L: entry c0 + (L & (kGroup - 1))
-            const int from = c0 + (lane & (kGroup - 1));
-            const int dst = __shfl(slot_v, from, kWave);
-            const float md = __shfl(max_dot, from, kWave);
-            if (lane < kGroup && c0 + lane < cnt) gw[dst] = r + md;
+            dot = (lane & ~(kGroup - 1)) == c0 ? r : dot;
         }
+        // in the order of the inverse list: one run of 4-byte values per target instead of a
+        // scattered write per entry (weight_grad_to_table_kernel moves them to their slots)
+        if (lane < cnt) gw_list[b0 + lane] = dot + max_dot;
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -490,18 +491,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8))) voi
 
 template <int VEC, int NB, bool PARTIAL>
 int launch_records(const float *g, const float *feat, const uint4 *records, const int *inv_off, const int *inv_slots,
-                   float *gw, float *gfeat, int n_vert, int K, int F, const int *idx, const int *order, float divisor,
-                   hipStream_t s) {
+                   float *gw_list, float *gfeat, int n_vert, int K, int F, const int *idx, const int *order,
+                   float divisor, hipStream_t s) {
     const dim3 grid(ceil_div(n_vert, 4)), block(256);
     const FastDiv div_k = make_fast_div(K);
     const bool pow2k = divisor == (float)(int)divisor && is_pow2((int)divisor);
     if (pow2k)
         accumulate_grad_records_kernel<VEC, NB, true, PARTIAL><<<grid, block, 0, s>>>(
-            g, feat, records, inv_off, inv_slots, gw, gfeat, n_vert, K, F, div_k, idx, order, divisor);
+            g, feat, records, inv_off, inv_slots, gw_list, gfeat, n_vert, K, F, div_k, idx, order, divisor);
     else
         accumulate_grad_records_kernel<VEC, NB, false, PARTIAL><<<grid, block, 0, s>>>(
-            g, feat, records, inv_off, inv_slots, gw, gfeat, n_vert, K, F, div_k, idx, order, divisor);
+            g, feat, records, inv_off, inv_slots, gw_list, gfeat, n_vert, K, F, div_k, idx, order, divisor);
     return check_launch("accumulate_grad_records_kernel");
+}
+
+// ---- pass 3: weight gradients from list order to their slots -------------------
+
+// gw[inv_slots[e]] = gw_list[e] for the entries of all targets, four per thread. The
+// scattered 4-byte writes of one stretch of the list fall into the rows of the source
+// vertices around it; each XCD works on one contiguous stretch, so the lines stay in
+// its L2 until they are full.
+__global__ __launch_bounds__(256) void weight_grad_to_table_kernel(const int *__restrict__ inv_off,
+                                                                   const int *__restrict__ inv_slots,
+                                                                   const float *__restrict__ gw_list,
+                                                                   float *__restrict__ gw, int n_vert) {
+    const long long n_entries = inv_off[n_vert];
+    const long long e0 = ((long long)xcd_contiguous_block(blockIdx.x, gridDim.x) * 256 + threadIdx.x) * 4;
+    if (e0 + 4 <= n_entries) {
+        const u32x4 slots = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(inv_slots + e0));
+        const f32x4 vals = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(gw_list + e0));
+        gw[slots.x] = vals.x;
+        gw[slots.y] = vals.y;
+        gw[slots.z] = vals.z;
+        gw[slots.w] = vals.w;
+    } else {
+        for (long long e = e0; e < n_entries; ++e) gw[inv_slots[e]] = gw_list[e];
+    }
 }
 
 // features per lane and blocks of 64 lanes of the gather pass for rows of F features; false: not covered
@@ -517,12 +542,15 @@ bool records_layout(int F, uintptr_t align_or, int &vec, int &nb) {
 int launch_zero_padded_weight_grad(const int *inv_off, const int *inv_slots, float *gw, int n_vert, long long total,
                                    hipStream_t s);
 
-// Bytes of record storage the record path needs for this shape, 0 where it does not apply:
+static size_t record_bytes(int n_vert, int K) { return align_up((size_t)n_vert * K * kRecordWords * sizeof(uint32_t)); }
+
+// Bytes of storage the record path needs for this shape (the records, then the weight
+// gradients in list order), 0 where it does not apply:
 // rows of 16 to 128 features addressed through 32-bit buffer offsets, slot bytes (K <= 254).
 size_t accumulate_grad_records_bytes(int n_vert, int K, int F) {
     if (n_vert <= 0 || K < 1 || K > 254 || F < 16 || F > 2 * kWave) return 0;
     if ((unsigned long long)n_vert * (unsigned long long)(2 * F) * 4ull >= (1ull << 32)) return 0;
-    return align_up((size_t)n_vert * K * kRecordWords * sizeof(uint32_t));
+    return record_bytes(n_vert, K) + align_up((size_t)n_vert * K * sizeof(float));
 }
 
 // Where the record pass has measured faster than the gather with the slot table (MI355X; kNN
@@ -540,7 +568,7 @@ int launch_accumulate_grad_records(const float *g, const float *w, const float *
                                    size_t records_bytes, hipStream_t s) {
     const size_t need = accumulate_grad_records_bytes(n_vert, K, F);
     if (need == 0 || !records || records_bytes < need || !maxslot || !gw || !gfeat) return 1;
-    if ((reinterpret_cast<uintptr_t>(records) & 15u) != 0) return 1;
+    if (((reinterpret_cast<uintptr_t>(records) | reinterpret_cast<uintptr_t>(inv_slots)) & 15u) != 0) return 1;
     const uintptr_t align_or = reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(feat) |
                                reinterpret_cast<uintptr_t>(gfeat);
     int vec, nb;
@@ -548,6 +576,7 @@ int launch_accumulate_grad_records(const float *g, const float *w, const float *
     const bool partial = F % kWave != 0;
 
     uint4 *rec = static_cast<uint4 *>(records);
+    float *gw_list = reinterpret_cast<float *>(static_cast<char *>(records) + record_bytes(n_vert, K));
     const size_t lds = (size_t)4 * K * (5 + 2 * kRecordHits) * sizeof(int);
     const dim3 grid(ceil_div(n_vert, 4));
     if (F <= kWave) hit_records_kernel<1><<<grid, 256, lds, s>>>(g, w, maxslot, rec, n_vert, K, F, vec);
@@ -556,11 +585,16 @@ int launch_accumulate_grad_records(const float *g, const float *w, const float *
     if (rc) return rc;
     rc = launch_zero_padded_weight_grad(inv_off, inv_slots, gw, n_vert, (long long)n_vert * K, s);
     if (rc) return rc;
-#define HGC_ARGS g, feat, rec, inv_off, inv_slots, gw, gfeat, n_vert, K, F, idx, order, divisor, s
-    if (partial) return nb == 1 ? launch_records<1, 1, true>(HGC_ARGS) : launch_records<1, 2, true>(HGC_ARGS);
-    if (vec == 2) return launch_records<2, 1, false>(HGC_ARGS);
-    return nb == 1 ? launch_records<1, 1, false>(HGC_ARGS) : launch_records<1, 2, false>(HGC_ARGS);
+#define HGC_ARGS g, feat, rec, inv_off, inv_slots, gw_list, gfeat, n_vert, K, F, idx, order, divisor, s
+    if (partial) rc = nb == 1 ? launch_records<1, 1, true>(HGC_ARGS) : launch_records<1, 2, true>(HGC_ARGS);
+    else if (vec == 2) rc = launch_records<2, 1, false>(HGC_ARGS);
+    else rc = nb == 1 ? launch_records<1, 1, false>(HGC_ARGS) : launch_records<1, 2, false>(HGC_ARGS);
 #undef HGC_ARGS
+    if (rc) return rc;
+    // the list has at most n_vert * K entries (fewer where slots are padded)
+    const long long blocks = ceil_div((long long)n_vert * K, 1024ll);
+    weight_grad_to_table_kernel<<<dim3((unsigned)blocks), 256, 0, s>>>(inv_off, inv_slots, gw_list, gw, n_vert);
+    return check_launch("weight_grad_to_table_kernel");
 }
 
 }  // namespace hgc

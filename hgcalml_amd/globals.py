@@ -21,8 +21,8 @@ reference would: `n_bins` (or its default formula, which reads the first event's
 size) over `max_bin_dims` dimensions.
 
 `acc_grad_hit_records` (no counterpart): the accumulation's gradient can first
-build one 32-byte record per (vertex, slot) in scratch memory (N*K*32 bytes) that
-hands the max part to the gather pass. None: where the library says it pays (wide
+build one 32-byte record per (vertex, slot) in scratch memory (N*K*36 bytes with
+the weight gradients in list order) that hands the max part to the gather pass. None: where the library says it pays (wide
 rows of large tables); True: wherever the shape allows; False: never. The results
 are the same (the weight gradient to the last bits of its tolerance)."""
 

@@ -354,12 +354,14 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
                                   int n_vert, int n_neigh, int n_feat, int n_grad_from_out_feat,
                                   int n_moments, int mean_and_max, hgc_stream_t stream);
 
-/* hgc_accumulate_knn_grad_slots with scratch memory for one 32-byte record per
- * (vertex, slot): a streaming pass over the vertices first collects, for every
- * slot, the weight, which features have their maximum there (from d_max_slots)
- * and their upstream gradients; the gather over the inverse index then reads
- * one record per entry instead of a weight, a line of slot bytes and scattered
- * pieces of the max half of the gradient row. Same results as
+/* hgc_accumulate_knn_grad_slots with scratch memory for one 32-byte record and
+ * one 4-byte result per (vertex, slot): a streaming pass over the vertices first
+ * collects, for every slot, the weight, which features have their maximum there
+ * (from d_max_slots) and their upstream gradients; the gather over the inverse
+ * index then reads one record per entry instead of a weight, a line of slot
+ * bytes and scattered pieces of the max half of the gradient row, and writes the
+ * weight gradients in the order of the inverse list; a last streaming pass moves
+ * them to their slots. Same results as
  * hgc_accumulate_knn_grad_slots (feature gradient bit for bit; the weight
  * gradient's max part is added after the mean part instead of inside it). Has
  * no counterpart in the reference. The workspace query returns 0 for shapes the
@@ -368,7 +370,7 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
  * hgc_accumulate_knn_grad_slots and accepts a NULL workspace, as it does when
  * d_max_slots is NULL. hgc_accumulate_knn_grad_records_pays says where the
  * record pass has measured faster (n_feat <= 2 n_neigh and n_vert * n_feat of
- * 12 Mi elements or more: cfg4 5.8 -> 5.2 ms); elsewhere
+ * 12 Mi elements or more: cfg4 5.8 -> 4.7 ms); elsewhere
  * hgc_accumulate_knn_grad_slots is the better call. */
 size_t hgc_accumulate_knn_grad_records_workspace_bytes(int n_vert, int n_neigh, int n_feat,
                                                        int mean_and_max);

@@ -573,7 +573,8 @@ def test_accumulate_gradient_hit_records_workspace_rules():
     """the C entry point: workspace sizes, where the record pass applies and where it pays, refusal of a
     workspace that is too small, and the fall-back to the slot-byte gather where it does not apply"""
     from hgcalml_amd._lib import lib
-    assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 64, 128, 1) == 1000 * 64 * 32
+    # a 32-byte record and a 4-byte weight gradient in list order per table entry
+    assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 64, 128, 1) == 1000 * 64 * (32 + 4)
     assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 64, 128, 0) == 0      # mean only: nothing to record
     assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 255, 128, 1) == 0     # slots are bytes
     assert lib.hgc_accumulate_knn_grad_records_workspace_bytes(1000, 64, 192, 1) == 0      # rows beyond 128 features
