@@ -397,8 +397,9 @@ def main():
         "accumulate_fwd_grad_GBps": round(achieved, 1),
         # the dominant kernel of the graded path: one launch of the one-pass gradient kernel
         "roofline": {"bound": "hbm",
-                     "kernel": "hit_records_kernel + accumulate_grad_records_kernel: one call of the accumulate_knn "
-                               "gradient (weights + features), cfg4 (N=%d, K=%d, F=%d)" % (n4, K4, F4),
+                     "kernel": "hit_records_kernel + accumulate_grad_records_kernel + weight_grad_to_table_kernel: one "
+                               "call of the accumulate_knn gradient (weights + features), cfg4 (N=%d, K=%d, F=%d)"
+                               % (n4, K4, F4),
                      "achieved": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(bytes_bwd / (grad_ms[0] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "traffic": traffic["gradient"] if traffic else None,

@@ -553,12 +553,15 @@ size_t accumulate_grad_records_bytes(int n_vert, int K, int F) {
     return record_bytes(n_vert, K) + align_up((size_t)n_vert * K * sizeof(float));
 }
 
-// Where the record pass has measured faster than the gather with the slot table (MI355X; kNN
-// tables of 150 k vertices and banded tables of 1 M, K = 16..64, F = 32..128): slots that hold
-// two hits or fewer on average, and gathered rows that add up to more than the L2 caches keep
-// (below that the streaming pass costs more than the gather saves).
+// Where the record pass has measured faster than the gather with the slot table (MI355X; banded
+// tables and kNN tables of 100 k to 1 M vertices, K = 16..64, F = 32..128): rows wider than K
+// features with two hits or fewer per slot on average, 48 neighbours or more, and gathered rows
+// that add up to more than the L2 caches keep. (Measured ratios of the two, records / slot bytes:
+// K = 64, F = 128: 0.81 on a banded table of 200 k to 1 M vertices, 0.99 on a kNN table of 1 M;
+// K = 64, F = 64: 0.93 banded, 1.30 kNN; K = 32: 0.99 to 1.26.)
 bool accumulate_grad_records_pays(int n_vert, int K, int F) {
-    return accumulate_grad_records_bytes(n_vert, K, F) != 0 && F <= 2 * K && (long long)n_vert * F >= (12ll << 20);
+    return accumulate_grad_records_bytes(n_vert, K, F) != 0 && K >= 48 && F > K && F <= 2 * K &&
+           (long long)n_vert * F >= (12ll << 20);
 }
 
 // Returns 1 when the shape is not covered (the caller then takes another path).

@@ -369,8 +369,8 @@ int hgc_accumulate_knn_grad_slots(const float *d_grad_from_out_features, const f
  * matrix of 4 GiB or more, !mean_and_max); the call then behaves exactly like
  * hgc_accumulate_knn_grad_slots and accepts a NULL workspace, as it does when
  * d_max_slots is NULL. hgc_accumulate_knn_grad_records_pays says where the
- * record pass has measured faster (n_feat <= 2 n_neigh and n_vert * n_feat of
- * 12 Mi elements or more: cfg4 5.8 -> 4.7 ms); elsewhere
+ * record pass has measured faster (n_neigh >= 48, n_neigh < n_feat <= 2 n_neigh
+ * and n_vert * n_feat of 12 Mi elements or more: cfg4 5.8 -> 4.7 ms); elsewhere
  * hgc_accumulate_knn_grad_slots is the better call. */
 size_t hgc_accumulate_knn_grad_records_workspace_bytes(int n_vert, int n_neigh, int n_feat,
                                                        int mean_and_max);

@@ -581,6 +581,8 @@ def test_accumulate_gradient_hit_records_workspace_rules():
     assert lib.hgc_accumulate_knn_grad_records_pays(1000000, 64, 128, 1) == 1
     assert lib.hgc_accumulate_knn_grad_records_pays(150000, 64, 64, 1) == 0
     assert lib.hgc_accumulate_knn_grad_records_pays(1000000, 16, 128, 1) == 0
+    assert lib.hgc_accumulate_knn_grad_records_pays(1000000, 64, 64, 1) == 0    # measured slower on kNN tables
+    assert lib.hgc_accumulate_knn_grad_records_pays(1000000, 32, 64, 1) == 0
     from hgcalml_amd import ops
     from hgcalml_amd._lib import p, stream
     rng = np.random.default_rng(5)
