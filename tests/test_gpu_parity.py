@@ -259,7 +259,7 @@ def test_knn_dense_bins_long_candidate_lists(oracle, C, n_bins):
                                   "clumps_radius", "edge"])
 def test_knn_nested_grid_cases(oracle, case):
     """the library's own grid with every coordinate binned (three or four) carries, from 48 neighbours on, a nested
-    grid of half the bin width for the queries of crowded bins (more than (K-1)/4 points):
+    grid of half the bin width for the queries of crowded bins (more than (K-1)/3 points):
     blob*: most queries walk it, with one and with two list registers per lane (blob4_few_neighbours: K below 48,
     the same points on the single grid); clumps: tight groups of 20 points far from everything else -- their walk on
     the nested grid gives up after a few shells and starts again on the grid of bins; edge: crowded bins on the border
