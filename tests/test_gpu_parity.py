@@ -1284,6 +1284,45 @@ def test_knn_and_accumulate_replay_from_a_hip_graph():
             assert all(torch.equal(a, b) for a, b in zip(eager, ref))
 
 
+@pytest.mark.parametrize("records", [False, True])
+def test_accumulate_gradient_replays_from_a_hip_graph(records):
+    """inverse neighbour index + gradient (either formulation) captured into a HIP graph:
+    every replay, with eager calls and synchronisations in between, returns the eager bits"""
+    from hgcalml_amd import globals as gl, ops
+    cfg = workloads.cfg4(scale=0.02)
+    idx, w = t(cfg["indices"]), t(np.exp(-cfg["distsq"]))
+    x, g = t(cfg["features"]), t(cfg["grad_out"])
+    out, arg, slots = torch.ops.hgcalml.accumulate_knn_slots(w, x, idx, 0, True)
+
+    def step():
+        inv = ops.inverse_neighbour_index(idx)
+        return torch.ops.hgcalml.accumulate_knn_grad_slots(g, w, x, idx, arg, slots, *inv)
+
+    gl.acc_grad_hit_records = records
+    try:
+        with torch.no_grad():
+            ref = [a.clone() for a in step()]
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                outs = step()
+            for _ in range(4):
+                for a in outs:
+                    a.zero_()
+                graph.replay()
+                torch.cuda.synchronize()
+                assert all(torch.equal(a, b) for a, b in zip(outs, ref))
+                eager = step()
+                torch.cuda.synchronize()
+                assert all(torch.equal(a, b) for a, b in zip(eager, ref))
+    finally:
+        gl.acc_grad_hit_records = None
+
+
 def test_vertex_processing_order_changes_nothing(oracle):
     """the kNN hands its bin order to the accumulation as a processing order:
     same bits with it, without it and with an arbitrary permutation"""
