@@ -49,7 +49,14 @@ def test_random_configuration(oracle, seed):
         # which member of an exactly tied K-th group survives is open; the distances are not
         assert (np.sort(bits(gd), 1) == np.sort(bits(rd), 1)).all()
     else:
-        assert (gi == ri).all() and (bits(gd) == bits(rd)).all()
+        # random floats: rows may differ from the oracle's only where the K-th boundary is an exact tie
+        # (which member of the tied group survives is open), and such a row is still a valid kNN set
+        differ = np.nonzero((gi != ri).any(1) | (bits(gd) != bits(rd)).any(1))[0]
+        assert len(differ) <= max(2, n // 500), differ[:10]
+        if len(differ):
+            from helpers import check_knn_rows
+            assert check_knn_rows(oracle, gi, gd, coords, rs, K, differ, direction=direction, tf_compatible=tfc,
+                                  radius=radius) == len(differ)
 
     if kind != 2 and K >= 2:      # the accumulation needs rows of distinct neighbours
         F = int(rng.choice([3, 8, 32, 64, 96, 128, 192, 256]))
