@@ -42,6 +42,7 @@ _SIGNATURES = {
     "hgc_index_replacer": (_c_int, [_ptr, _ptr, _ptr, _c_int, _c_int, _ptr]),
     "hgc_accumulate_knn": (_c_int, [_ptr] * 5 + [_c_int] * 6 + [_ptr]),
     "hgc_accumulate_knn_slots": (_c_int, [_ptr] * 7 + [_c_int] * 6 + [_ptr]),
+    "hgc_accumulate_knn_exp_slots": (_c_int, [_ptr] * 8 + [_c_int] * 6 + [_ptr]),
     "hgc_inverse_neighbour_index_workspace_bytes": (_c_size, [_c_int, _c_int]),
     "hgc_inverse_neighbour_index": (_c_int, [_ptr, _c_int, _c_int, _ptr, _ptr, _ptr, _c_size, _ptr]),
     "hgc_inverse_index_without_first_column_workspace_bytes": (_c_size, [_c_int]),

@@ -31,6 +31,28 @@ class _AccumulateFn(torch.autograd.Function):
         return gw, gx, None, None
 
 
+class _AccumulateExpFn(torch.autograd.Function):
+    """AccumulateKnn as one op each way: exp(-distances) is taken inside the accumulation kernel
+    (modules/accknn_op.py:52 + :71-89), the gradient w.r.t. the distances is -(gw * w)"""
+
+    @staticmethod
+    def forward(ctx, distances, features, indices, mean_and_max):
+        out, maxidx, slots, weights = torch.ops.hgcalml.accumulate_knn_exp_slots(distances, features, indices, 0,
+                                                                                 mean_and_max)
+        ctx.save_for_backward(weights, features, indices, maxidx, slots)
+        ctx.indices_ref = indices
+        ctx.mark_non_differentiable(maxidx)
+        return out, maxidx
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_maxidx):
+        weights, features, indices, maxidx, slots = ctx.saved_tensors
+        inv_off, inv_slots = ops.cached_inverse_neighbour_index(ctx.indices_ref)
+        gw, gx = torch.ops.hgcalml.accumulate_knn_grad_slots(grad_out.contiguous(), weights, features, indices,
+                                                             maxidx, slots, inv_off, inv_slots)
+        return ops.exp_neg_grad(gw, weights), gx, None, None
+
+
 class _ExpNegFn(torch.autograd.Function):
     """weights = exp(-distances) (modules/accknn_op.py:86) and its chain rule, one kernel each"""
 
@@ -73,8 +95,9 @@ def AccumulateKnn(distances, features, indices, mean_and_max=True, force_tf=Fals
     Returns (out [N, 2F] (mean | max) or [N, F], arg-max neighbour index [N, F]).
     """
     if (not gl.acc_ops_use_tf_gradients) and (not force_tf):
-        weights = _ExpNegFn.apply(distances) if distances.dtype == torch.float32 else torch.exp(-distances)
-        return _AccumulateFn.apply(weights, features, indices, bool(mean_and_max))
+        if distances.dtype == torch.float32:
+            return _AccumulateExpFn.apply(distances, features, indices, bool(mean_and_max))
+        return _AccumulateFn.apply(torch.exp(-distances), features, indices, bool(mean_and_max))
     return _torch_composition(torch.exp(-distances), features, indices, mean_and_max)
 
 

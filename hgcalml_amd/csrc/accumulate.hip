@@ -183,14 +183,16 @@ __device__ __forceinline__ void fwd_slot(const float (&x)[VEC], float wn, int sl
 // lane l and are broadcast with v_readlane (no arrays of scalars to keep alive),
 // all rows are in flight together, a slot without a neighbour fetches row 0 and
 // is skipped. Returns n_begin so that the caller's loop advances as for a full chunk.
-template <int VEC, bool MAX, int U>
+// (EXPW: the row's weights are already in the lanes of w_row, slot n in lane n.)
+template <int VEC, bool MAX, int U, bool EXPW>
 __device__ __forceinline__ int partial_chunk(const RowMatrix &X, const int *__restrict__ irow,
-                                             const float *__restrict__ wrow, int n_begin, int n_end, int n_vert,
-                                             uint32_t lane_bytes, float (&sum)[VEC], float (&best)[VEC], int (&arg)[VEC]) {
+                                             const float *__restrict__ wrow, float w_row, int n_begin, int n_end,
+                                             int n_vert, uint32_t lane_bytes, float (&sum)[VEC], float (&best)[VEC],
+                                             int (&arg)[VEC]) {
     const int lane = lane_id();
     const int n_mine = min(n_begin + lane, n_end - 1);
     const int j_lane = n_begin + lane < n_end ? irow[n_mine] : -1;
-    const float w_lane = wrow[n_mine];
+    const float w_lane = EXPW ? 0.f : wrow[n_mine];
     const uint64_t valid = __ballot((uint32_t)j_lane < (uint32_t)n_vert);  // bit l: slot n_begin + l has a neighbour
     float x[U][VEC];
 #pragma unroll
@@ -201,7 +203,8 @@ __device__ __forceinline__ int partial_chunk(const RowMatrix &X, const int *__re
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         if (!((valid >> u) & 1ull)) continue;  // wave-uniform
-        const float w = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(w_lane), u));
+        const float w = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
+            (int)__float_as_uint(EXPW ? w_row : w_lane), EXPW ? n_begin + u : u));
         if (n_begin + u == 0)
             fwd_slot<VEC, MAX, true>(x[u], w, 0, sum, best, arg);
         else
@@ -210,19 +213,32 @@ __device__ __forceinline__ int partial_chunk(const RowMatrix &X, const int *__re
     return n_begin;
 }
 
-template <int VEC, bool MAX>
+// EXPW (rows of 64 slots or fewer): `w` holds distances; lane n turns the distance of slot n into
+// the weight exp(-d) (modules/accknn_op.py:52, there a framework op of its own in front of the
+// kernel), writes it to w_out for the gradient, and the slots' weights reach the scalar side by
+// v_readlane instead of scalar loads.
+template <int VEC, bool MAX, bool EXPW>
 __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *__restrict__ w,
                                                                   const float *__restrict__ feat,
                                                                   const int *__restrict__ idx, float *__restrict__ out,
                                                                   int *__restrict__ out_maxidx,
                                                                   unsigned char *__restrict__ out_maxslot, int n_vert,
                                                                   int K, int F, int out_cols, float kf,
-                                                                  const int *__restrict__ order) {
+                                                                  const int *__restrict__ order,
+                                                                  float *__restrict__ w_out) {
     constexpr int U = VEC == 4 ? 8 : 16;
     const int v = wave_vertex(order, n_vert);
     if (v >= n_vert) return;
     const int *irow = idx + (size_t)v * K;
     const float *wrow = w + (size_t)v * K;
+    float w_row = 0.f;
+    if (EXPW) {
+        const int n = lane_id();
+        if (n < K) {
+            w_row = expf(-wrow[n]);
+            w_out[(size_t)v * K + n] = w_row;
+        }
+    }
     const RowMatrix X(feat, n_vert, F);
     int first_self = -1;  // first slot that names the vertex itself (wave-uniform, scalar ALU)
 
@@ -245,7 +261,8 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 j[u] = irow[n0 + u];
-                wn[u] = wrow[n0 + u];
+                wn[u] = EXPW ? __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(w_row), n0 + u))
+                             : wrow[n0 + u];
                 j_max = max(j_max, (uint32_t)j[u]);
             }
             const bool all_valid = j_max < (uint32_t)n_vert;
@@ -268,7 +285,8 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                     for (int u = 0; u < U; ++u) fwd_slot<VEC, MAX, false>(x[u], wn[u], n0 + u, sum, best, arg);
                 }
             } else {
-                n0 = partial_chunk<VEC, MAX, U>(X, irow, wrow, n0, n0 + U, n_vert, lane_bytes, sum, best, arg);
+                n0 = partial_chunk<VEC, MAX, U, EXPW>(X, irow, wrow, w_row, n0, n0 + U, n_vert, lane_bytes, sum, best,
+                                                      arg);
             }
         }
         if (n0 < K) {  // K not a multiple of U
@@ -278,11 +296,11 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                 if (first_self < 0 && self) first_self = n0 + __builtin_ctzll(self);
             }
             if (K - n0 <= 4)
-                partial_chunk<VEC, MAX, 4>(X, irow, wrow, n0, K, n_vert, lane_bytes, sum, best, arg);
+                partial_chunk<VEC, MAX, 4, EXPW>(X, irow, wrow, w_row, n0, K, n_vert, lane_bytes, sum, best, arg);
             else if (K - n0 <= 8 || U == 8)
-                partial_chunk<VEC, MAX, 8>(X, irow, wrow, n0, K, n_vert, lane_bytes, sum, best, arg);
+                partial_chunk<VEC, MAX, 8, EXPW>(X, irow, wrow, w_row, n0, K, n_vert, lane_bytes, sum, best, arg);
             else
-                partial_chunk<VEC, MAX, 16>(X, irow, wrow, n0, K, n_vert, lane_bytes, sum, best, arg);
+                partial_chunk<VEC, MAX, 16, EXPW>(X, irow, wrow, w_row, n0, K, n_vert, lane_bytes, sum, best, arg);
         }
         float mean[VEC];
 #pragma unroll
@@ -759,9 +777,12 @@ namespace hgc {
 
 // Forward pass shared by accumulate_knn (divisor = K) and the feature gradient of
 // push_knn (divisor = 1): out = (sum over the slots of w * feat[idx]) / divisor.
+// d_out_weights == nullptr: d_distances are the weights. Otherwise they are distances, the weights
+// exp(-d) are used and written to d_out_weights.
 int accumulate_forward(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
                        int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat,
-                       int n_out_feat, int mean_and_max, float divisor, const int *d_order, hgc_stream_t stream) {
+                       int n_out_feat, int mean_and_max, float divisor, const int *d_order, float *d_out_weights,
+                       hgc_stream_t stream) {
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_feat >= 1, "bad sizes");
     HGC_REQUIRE(n_out_feat == n_feat * (mean_and_max ? 2 : 1), "n_out_feat must be n_feat * (mean_and_max ? 2 : 1)");
     // slots are numbered with 32 bits; matrices of any size (beyond 4 GiB: the thread-per-element kernels with
@@ -776,18 +797,28 @@ int accumulate_forward(const float *d_distances, const float *d_feat, const int 
                               reinterpret_cast<uintptr_t>(d_out_maxidxs);
     // the wave kernels address rows through 32-bit buffer offsets
     const bool fits_32bit = (unsigned long long)n_vert * (unsigned long long)n_out_feat * 4ull < (1ull << 32);
-    if (n_feat >= 16 && fits_32bit) {  // one wave per vertex (lanes beyond a short row stay idle)
+    const bool wave_kernel = n_feat >= 16 && fits_32bit;
+    const bool exp_in_kernel = d_out_weights && wave_kernel && n_neigh <= kWave;
+    if (d_out_weights && !exp_in_kernel) {  // the weights in a pass of their own, then as if they had been given
+        const int rc = hgc_exp_neg(d_distances, d_out_weights, (long long)n_vert * n_neigh, stream);
+        if (rc) return rc;
+        d_distances = d_out_weights;
+    }
+    if (wave_kernel) {  // one wave per vertex (lanes beyond a short row stay idle)
         const int vec = wave_vec(n_feat, align_or);
         const dim3 grid(ceil_div(n_vert, 4)), block(256);
-#define HGC_FWD(VEC, MAX)                                                                                         \
-    accumulate_fwd_wave_kernel<VEC, MAX><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, \
-                                                               d_out_maxslots, n_vert, n_neigh, n_feat, n_out_feat, divisor, \
-                                                               d_order)
+#define HGC_FWD(VEC, MAX, EXPW)                                                                                     \
+    accumulate_fwd_wave_kernel<VEC, MAX, EXPW><<<grid, block, 0, s>>>(d_distances, d_feat, d_idxs, d_out_feat,         \
+                                                                     d_out_maxidxs, d_out_maxslots, n_vert, n_neigh, \
+                                                                     n_feat, n_out_feat, divisor, d_order, d_out_weights)
+#define HGC_FWD_VEC(MAX, EXPW)                                                                                      \
+    if (vec == 4) HGC_FWD(4, MAX, EXPW); else if (vec == 2) HGC_FWD(2, MAX, EXPW); else HGC_FWD(1, MAX, EXPW)
         if (mean_and_max) {
-            if (vec == 4) HGC_FWD(4, true); else if (vec == 2) HGC_FWD(2, true); else HGC_FWD(1, true);
+            if (exp_in_kernel) { HGC_FWD_VEC(true, true); } else { HGC_FWD_VEC(true, false); }
         } else {
-            if (vec == 4) HGC_FWD(4, false); else if (vec == 2) HGC_FWD(2, false); else HGC_FWD(1, false);
+            if (exp_in_kernel) { HGC_FWD_VEC(false, true); } else { HGC_FWD_VEC(false, false); }
         }
+#undef HGC_FWD_VEC
 #undef HGC_FWD
         return check_launch("accumulate_fwd_wave_kernel");
     }
@@ -824,7 +855,19 @@ int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, cons
                              hgc_stream_t stream) {
     (void)n_moments;  // carried by the reference op, never used by its kernels
     return accumulate_forward(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, d_out_maxslots, n_vert, n_neigh,
-                              n_feat, n_out_feat, mean_and_max, (float)n_neigh, d_vertex_order, stream);
+                              n_feat, n_out_feat, mean_and_max, (float)n_neigh, d_vertex_order, nullptr, stream);
+}
+
+int hgc_accumulate_knn_exp_slots(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
+                                 int *d_out_maxidxs, unsigned char *d_out_maxslots, float *d_out_weights,
+                                 const int *d_vertex_order, int n_vert, int n_neigh, int n_feat, int n_out_feat,
+                                 int n_moments, int mean_and_max, hgc_stream_t stream) {
+    (void)n_moments;
+    HGC_REQUIRE(n_vert <= 0 || d_out_weights, "null pointer");
+    HGC_REQUIRE(((reinterpret_cast<uintptr_t>(d_distances) | reinterpret_cast<uintptr_t>(d_out_weights)) & 15u) == 0,
+                "distances and weights must start on 16-byte boundaries");
+    return accumulate_forward(d_distances, d_feat, d_idxs, d_out_feat, d_out_maxidxs, d_out_maxslots, n_vert, n_neigh,
+                              n_feat, n_out_feat, mean_and_max, (float)n_neigh, d_vertex_order, d_out_weights, stream);
 }
 
 int hgc_accumulate_knn(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,

@@ -20,7 +20,8 @@ namespace hgc {
 // accumulate.hip
 int accumulate_forward(const float *d_distances, const float *d_feat, const int *d_idxs, float *d_out_feat,
                        int *d_out_maxidxs, unsigned char *d_out_maxslots, int n_vert, int n_neigh, int n_feat,
-                       int n_out_feat, int mean_and_max, float divisor, const int *d_order, hgc_stream_t stream);
+                       int n_out_feat, int mean_and_max, float divisor, const int *d_order, float *d_out_weights,
+                       hgc_stream_t stream);
 int accumulate_gradient(const float *d_grad_from_out_features, const float *d_distances, const float *d_feat,
                         const int *d_max_feat_indices, const unsigned char *d_max_slots, const int *d_neigh_indices,
                         const int *d_inv_offsets, const int *d_inv_slots, float *d_out_grad_distances,
@@ -432,7 +433,7 @@ int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *
     }
     // feat_grad[v, f] = sum_n grad[idx[v,n], f] * w[v,n]: the mean-only forward over `grad`, not divided by K
     int rc = accumulate_forward(d_weights, d_grad, d_idxs, d_feat_grad, nullptr, nullptr, n_vert, n_neigh, n_feat,
-                                n_feat, 0, 1.f, nullptr, stream);
+                                n_feat, 0, 1.f, nullptr, nullptr, stream);
     if (rc) return rc;
     // w_grad[v, n] = sum_f grad[idx[v,n], f] * feat[v, f]: the weight gradient with the roles of the
     // vertex's own row (feat) and the gathered rows (grad) as in the accumulation's

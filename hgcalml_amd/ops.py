@@ -258,7 +258,8 @@ def share_vertex_order(source_indices, derived_indices):
         set_vertex_order(derived_indices, order)
 
 
-def _accumulate_forward(distances, features, indices, n_moments, mean_and_max, with_slots):
+def _accumulate_forward(distances, features, indices, n_moments, mean_and_max, with_slots, exp_weights=False):
+    """exp_weights: `distances` are distances, the weights exp(-d) are used and returned as a fourth value"""
     dev = require_device(distances, features, indices)
     w, x, idx = f32(distances), f32(features), i32(indices)
     # modules/compiled/accumulate_knn_kernel.cc:107-111
@@ -275,6 +276,12 @@ def _accumulate_forward(distances, features, indices, n_moments, mean_and_max, w
     slots = None
     if with_slots and mean_and_max and k <= 254:
         slots = torch.empty((n, f), dtype=torch.uint8, device=dev)
+    if exp_weights:
+        weights = torch.empty_like(w)
+        check(lib.hgc_accumulate_knn_exp_slots(p(w), p(x), p(idx), p(out), p(maxidx), p(slots), p(weights),
+                                               p(vertex_order_of(indices)), n, k, f, out.shape[1], int(n_moments),
+                                               int(mean_and_max), stream()))
+        return out, maxidx, slots, weights
     check(lib.hgc_accumulate_knn_slots(p(w), p(x), p(idx), p(out), p(maxidx), p(slots), p(vertex_order_of(indices)),
                                        n, k, f, out.shape[1], int(n_moments), int(mean_and_max), stream()))
     return out, maxidx, slots
@@ -286,6 +293,20 @@ def accumulate_knn(distances: torch.Tensor, features: torch.Tensor, indices: tor
     """modules/compiled/accumulate_knn_module.cc:7-14 (`distances` are the weights)"""
     out, maxidx, _ = _accumulate_forward(distances, features, indices, n_moments, mean_and_max, False)
     return out, maxidx
+
+
+@torch.library.custom_op("hgcalml::accumulate_knn_exp_slots", mutates_args=())
+def accumulate_knn_exp_slots(distances: torch.Tensor, features: torch.Tensor, indices: torch.Tensor, n_moments: int,
+                             mean_and_max: bool) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """accumulate_knn_slots with the weights exp(-distances) of the AccumulateKnn wrapper
+    (modules/accknn_op.py:52) taken inside the kernel; the weights are the fourth result."""
+    if distances.data_ptr() % 16:
+        distances = distances.clone()
+    out, maxidx, slots, weights = _accumulate_forward(distances, features, indices, n_moments, mean_and_max, True,
+                                                      exp_weights=True)
+    if slots is None:
+        slots = torch.empty((0,), dtype=torch.uint8, device=out.device)
+    return out, maxidx, slots, weights
 
 
 @torch.library.custom_op("hgcalml::accumulate_knn_slots", mutates_args=())
@@ -657,6 +678,15 @@ def _(distances, features, indices, n_moments, mean_and_max):
     n, f = features.shape
     with_slots = mean_and_max and indices.shape[1] <= 254
     return out, maxidx, features.new_empty((n, f) if with_slots else (0,), dtype=torch.uint8)
+
+
+@accumulate_knn_exp_slots.register_fake
+def _(distances, features, indices, n_moments, mean_and_max):
+    out, maxidx = _accumulate_shapes(features, indices, mean_and_max)
+    n, f = features.shape
+    with_slots = mean_and_max and indices.shape[1] <= 254
+    return (out, maxidx, features.new_empty((n, f) if with_slots else (0,), dtype=torch.uint8),
+            _f32_like(indices.shape, features))
 
 
 def _accumulate_grad_shapes(features, neigh_indices):

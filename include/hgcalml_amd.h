@@ -302,6 +302,23 @@ int hgc_accumulate_knn_slots(const float *d_distances, const float *d_feat, cons
                              int n_vert, int n_neigh, int n_feat, int n_out_feat,
                              int n_moments, int mean_and_max, hgc_stream_t stream);
 
+/* hgc_accumulate_knn_slots for the AccumulateKnn wrapper: d_distances are
+ * distances, the weights are exp(-d) (modules/accknn_op.py:52, there a
+ * framework op of its own in front of the kernel) and are also written to
+ * d_out_weights [n_vert, n_neigh], which the gradient calls take as their
+ * d_distances. For rows of 64 slots or fewer and 16 features or more the
+ * exponential is taken inside the accumulation kernel, otherwise by hgc_exp_neg
+ * first; the results are the same bits as hgc_exp_neg followed by
+ * hgc_accumulate_knn_slots. d_distances and d_out_weights on 16-byte
+ * boundaries. No single counterpart in the reference (its wrapper's op and
+ * its kernel in one call). */
+int hgc_accumulate_knn_exp_slots(const float *d_distances, const float *d_feat, const int *d_idxs,
+                                 float *d_out_feat, int *d_out_maxidxs,
+                                 unsigned char *d_out_maxslots, float *d_out_weights,
+                                 const int *d_vertex_order,
+                                 int n_vert, int n_neigh, int n_feat, int n_out_feat,
+                                 int n_moments, int mean_and_max, hgc_stream_t stream);
+
 /* Inverse neighbour index: for every vertex m the list of (vertex, slot)
  * pairs that name m, ascending. Built once per neighbour table and reused by
  * every gradient call on it.

@@ -1449,6 +1449,42 @@ def test_inverse_index_without_first_column(n, k):
     assert ops.cached_inverse_neighbour_index(whole.view(n, k))[0] is ops.cached_inverse_neighbour_index(whole)[0]
 
 
+@pytest.mark.parametrize("n,K,F", [(3000, 64, 64), (2000, 10, 32), (1500, 33, 128), (700, 65, 64), (900, 16, 8),
+                                   (500, 1, 16), (1200, 64, 256)])
+def test_accumulate_knn_with_the_exponential_inside(n, K, F):
+    """AccumulateKnn's weights exp(-d) taken inside the accumulation kernel (rows of up to 64 slots and
+    16 or more features; the other shapes run the two passes): the bits of the two-pass route for the
+    weights, both outputs, the arg-max and the slot table, with padded rows and in either mode; and the
+    wrapper's gradients are those of the two autograd functions it replaces"""
+    from hgcalml_amd import AccumulateKnn, ops
+    from hgcalml_amd.accknn_op import _AccumulateFn, _ExpNegFn
+    rng = np.random.default_rng(900 + K + F)
+    d, x, idx = make_acc_case(rng, n, K, F)
+    d = (np.abs(d) * 3).astype(np.float32)
+    td, tx, ti = t(d), t(x), t(idx)
+    for mm in (True, False):
+        w = ops.exp_neg(td)
+        out0, arg0, slots0 = torch.ops.hgcalml.accumulate_knn_slots(w, tx, ti, 0, mm)
+        out1, arg1, slots1, w1 = torch.ops.hgcalml.accumulate_knn_exp_slots(td, tx, ti, 0, mm)
+        assert torch.equal(w1.view(torch.int32), w.view(torch.int32))
+        assert torch.equal(out1.view(torch.int32), out0.view(torch.int32))
+        assert torch.equal(arg1, arg0) and torch.equal(slots1, slots0)
+        a = [td.clone().requires_grad_(True), tx.clone().requires_grad_(True)]
+        b = [td.clone().requires_grad_(True), tx.clone().requires_grad_(True)]
+        oa, _ = AccumulateKnn(a[0], a[1], ti, mean_and_max=mm)
+        ob, _ = _AccumulateFn.apply(_ExpNegFn.apply(b[0]), b[1], ti, mm)
+        assert torch.equal(oa, ob)
+        g = torch.from_numpy(rng.standard_normal(tuple(oa.shape)).astype(np.float32)).to(DEV)
+        oa.backward(g)
+        ob.backward(g)
+        assert torch.equal(a[0].grad, b[0].grad) and torch.equal(a[1].grad, b[1].grad)
+    # distances that do not start on a 16-byte boundary
+    flat = torch.cat([td.new_zeros(1), td.flatten()])
+    shifted = flat[1:].view(n, K)
+    out2, _, _, w2 = torch.ops.hgcalml.accumulate_knn_exp_slots(shifted, tx, ti, 0, True)
+    assert torch.equal(w2, ops.exp_neg(td)) and torch.equal(out2, torch.ops.hgcalml.accumulate_knn_slots(w2, tx, ti, 0, True)[0])
+
+
 def test_accumulate_knn_weights_and_their_gradient_in_one_pass():
     """exp(-d) and -(g*w) of the AccumulateKnn wrapper: the library's one-pass kernels return the
     bits of the framework's elementwise ops, for sizes that are no multiple of four and views that

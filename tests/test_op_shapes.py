@@ -37,6 +37,8 @@ def test_fake_implementations_give_the_reference_output_shapes(ops):
     assert describe(h.accumulate_knn_slots(m(N, K), m(N, F), m(N, K, dtype=i32), 0, True)) == \
         [((N, 2 * F), f32, "meta"), ((N, F), i32, "meta"), ((N, F), u8, "meta")]
     assert describe(h.accumulate_knn_slots(m(N, 300), m(N, F), m(N, 300, dtype=i32), 0, True))[2] == ((0,), u8, "meta")
+    assert describe(h.accumulate_knn_exp_slots(m(N, K), m(N, F), m(N, K, dtype=i32), 0, True)) == \
+        [((N, 2 * F), f32, "meta"), ((N, F), i32, "meta"), ((N, F), u8, "meta"), ((N, K), f32, "meta")]
     grads = [((N, K), f32, "meta"), ((N, F), f32, "meta")]
     assert describe(h.accumulate_knn_grad(m(N, 2 * F), m(N, K), m(N, F), m(N, K, dtype=i32), m(N, F, dtype=i32),
                                           m(N + 1, dtype=i32), m(N * K, dtype=i32))) == grads
