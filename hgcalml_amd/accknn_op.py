@@ -54,7 +54,7 @@ class _AccumulateExpFn(torch.autograd.Function):
 
 
 class _ExpNegFn(torch.autograd.Function):
-    """weights = exp(-distances) (modules/accknn_op.py:86) and its chain rule, one kernel each"""
+    """weights = exp(-distances) (modules/accknn_op.py:52) and its chain rule, one kernel each"""
 
     @staticmethod
     def forward(ctx, distances):

@@ -220,7 +220,7 @@ using namespace hgc;
 
 namespace {
 
-// weights of AccumulateKnn, w = exp(-d) (modules/accknn_op.py:86), and the chain rule back to
+// weights of AccumulateKnn, w = exp(-d) (modules/accknn_op.py:52), and the chain rule back to
 // the distances, gd = -(gw * w): one pass each instead of two framework kernels
 __global__ __launch_bounds__(256) void exp_neg_kernel(const float *__restrict__ d, float *__restrict__ w,
                                                       long long n) {

@@ -475,7 +475,7 @@ int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *
                       const int *d_idxs, float *d_feat_grad, float *d_w_grad,
                       int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
 
-/* The elementwise glue of the AccumulateKnn wrapper (modules/accknn_op.py:86,
+/* The elementwise glue of the AccumulateKnn wrapper (modules/accknn_op.py:52,
  * `tf.exp(-distsq)`) and of its gradient, one pass each: d_weights[i] =
  * exp(-d_distances[i]); d_distance_grad[i] = -(d_weight_grad[i] * d_weights[i]).
  * Arrays of n_values floats on 16-byte boundaries. */
