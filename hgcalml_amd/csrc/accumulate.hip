@@ -183,10 +183,10 @@ __device__ __forceinline__ void fwd_slot(const float (&x)[VEC], float wn, int sl
 // lane l and are broadcast with v_readlane (no arrays of scalars to keep alive),
 // all rows are in flight together, a slot without a neighbour fetches row 0 and
 // is skipped. Returns n_begin so that the caller's loop advances as for a full chunk.
-// (EXPW: the row's weights are already in the lanes of w_row, slot n in lane n.)
+// (EXPW: the row's weights wait in LDS, w_lds[n] for slot n.)
 template <int VEC, bool MAX, int U, bool EXPW>
 __device__ __forceinline__ int partial_chunk(const RowMatrix &X, const int *__restrict__ irow,
-                                             const float *__restrict__ wrow, float w_row, int n_begin, int n_end,
+                                             const float *__restrict__ wrow, const float *w_lds, int n_begin, int n_end,
                                              int n_vert, uint32_t lane_bytes, float (&sum)[VEC], float (&best)[VEC],
                                              int (&arg)[VEC]) {
     const int lane = lane_id();
@@ -203,8 +203,8 @@ __device__ __forceinline__ int partial_chunk(const RowMatrix &X, const int *__re
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         if (!((valid >> u) & 1ull)) continue;  // wave-uniform
-        const float w = __uint_as_float((uint32_t)__builtin_amdgcn_readlane(
-            (int)__float_as_uint(EXPW ? w_row : w_lane), EXPW ? n_begin + u : u));
+        const float w = EXPW ? w_lds[n_begin + u]
+                             : __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(w_lane), u));
         if (n_begin + u == 0)
             fwd_slot<VEC, MAX, true>(x[u], w, 0, sum, best, arg);
         else
@@ -215,8 +215,8 @@ __device__ __forceinline__ int partial_chunk(const RowMatrix &X, const int *__re
 
 // EXPW (rows of 64 slots or fewer): `w` holds distances; lane n turns the distance of slot n into
 // the weight exp(-d) (modules/accknn_op.py:52, there a framework op of its own in front of the
-// kernel), writes it to w_out for the gradient, and the slots' weights reach the scalar side by
-// v_readlane instead of scalar loads.
+// kernel), writes it to w_out for the gradient and to LDS, from where every lane reads the slots'
+// weights (same address in all lanes) instead of the scalar loads.
 template <int VEC, bool MAX, bool EXPW>
 __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *__restrict__ w,
                                                                   const float *__restrict__ feat,
@@ -231,13 +231,17 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
     if (v >= n_vert) return;
     const int *irow = idx + (size_t)v * K;
     const float *wrow = w + (size_t)v * K;
-    float w_row = 0.f;
+    __shared__ float s_weights[EXPW ? 4 : 1][kWave];
+    const float *w_lds = s_weights[EXPW ? threadIdx.x >> 6 : 0];
     if (EXPW) {
         const int n = lane_id();
+        float w_n = 0.f;
         if (n < K) {
-            w_row = expf(-wrow[n]);
-            w_out[(size_t)v * K + n] = w_row;
+            w_n = expf(-wrow[n]);
+            w_out[(size_t)v * K + n] = w_n;
         }
+        s_weights[threadIdx.x >> 6][n] = w_n;
+        wave_lds_fence();
     }
     const RowMatrix X(feat, n_vert, F);
     int first_self = -1;  // first slot that names the vertex itself (wave-uniform, scalar ALU)
@@ -261,8 +265,7 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 j[u] = irow[n0 + u];
-                wn[u] = EXPW ? __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(w_row), n0 + u))
-                             : wrow[n0 + u];
+                wn[u] = EXPW ? w_lds[n0 + u] : wrow[n0 + u];
                 j_max = max(j_max, (uint32_t)j[u]);
             }
             const bool all_valid = j_max < (uint32_t)n_vert;
@@ -285,7 +288,7 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                     for (int u = 0; u < U; ++u) fwd_slot<VEC, MAX, false>(x[u], wn[u], n0 + u, sum, best, arg);
                 }
             } else {
-                n0 = partial_chunk<VEC, MAX, U, EXPW>(X, irow, wrow, w_row, n0, n0 + U, n_vert, lane_bytes, sum, best,
+                n0 = partial_chunk<VEC, MAX, U, EXPW>(X, irow, wrow, w_lds, n0, n0 + U, n_vert, lane_bytes, sum, best,
                                                       arg);
             }
         }
@@ -296,11 +299,11 @@ __global__ __launch_bounds__(256) void accumulate_fwd_wave_kernel(const float *_
                 if (first_self < 0 && self) first_self = n0 + __builtin_ctzll(self);
             }
             if (K - n0 <= 4)
-                partial_chunk<VEC, MAX, 4, EXPW>(X, irow, wrow, w_row, n0, K, n_vert, lane_bytes, sum, best, arg);
+                partial_chunk<VEC, MAX, 4, EXPW>(X, irow, wrow, w_lds, n0, K, n_vert, lane_bytes, sum, best, arg);
             else if (K - n0 <= 8 || U == 8)
-                partial_chunk<VEC, MAX, 8, EXPW>(X, irow, wrow, w_row, n0, K, n_vert, lane_bytes, sum, best, arg);
+                partial_chunk<VEC, MAX, 8, EXPW>(X, irow, wrow, w_lds, n0, K, n_vert, lane_bytes, sum, best, arg);
             else
-                partial_chunk<VEC, MAX, 16, EXPW>(X, irow, wrow, w_row, n0, K, n_vert, lane_bytes, sum, best, arg);
+                partial_chunk<VEC, MAX, 16, EXPW>(X, irow, wrow, w_lds, n0, K, n_vert, lane_bytes, sum, best, arg);
         }
         float mean[VEC];
 #pragma unroll
