@@ -158,8 +158,29 @@ __global__ __launch_bounds__(256) void hit_records_kernel(const float *__restric
         r1.y = dense ? bits[4 * n + 2] : __float_as_uint(vv[2]);
         r1.z = dense ? bits[4 * n + 3] : __float_as_uint(vv[3]);
         r1.w = __float_as_uint(vv[4]);
-        store_once(records + 2 * s, r0);  // 2 KB per vertex, read back much later by the gather
-        store_once(records + 2 * s + 1, r1);
+        // (2 KB per 64 slots, read back much later by the gather)
+        if (n - lane + kWave <= K) {  // wave-uniform: 64 records, written as whole lines --
+            // lane i holds bytes [16 i, 16 i + 16) of either half of the 2 KB
+            uint4 *block = records + 2 * (s - lane);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int src = 32 * h + (lane >> 1);
+                const bool odd = lane & 1;
+                uint4 o;
+                const uint32_t a0 = __shfl(r0.x, src, kWave), b0 = __shfl(r1.x, src, kWave);
+                const uint32_t a1 = __shfl(r0.y, src, kWave), b1 = __shfl(r1.y, src, kWave);
+                const uint32_t a2 = __shfl(r0.z, src, kWave), b2 = __shfl(r1.z, src, kWave);
+                const uint32_t a3 = __shfl(r0.w, src, kWave), b3 = __shfl(r1.w, src, kWave);
+                o.x = odd ? b0 : a0;
+                o.y = odd ? b1 : a1;
+                o.z = odd ? b2 : a2;
+                o.w = odd ? b3 : a3;
+                store_once(block + kWave * h + lane, o);
+            }
+        } else {
+            store_once(records + 2 * s, r0);
+            store_once(records + 2 * s + 1, r1);
+        }
     }
 }
 
