@@ -310,17 +310,18 @@ def main():
     try:
         c3 = workloads.cfg3()
         co3, rs3 = torch.from_numpy(c3["coords"]).to(dev), torch.from_numpy(c3["row_splits"]).to(dev)
-        m3 = event_ms(lambda: BinnedSelectKnn(c3["K"], co3, rs3, n_bins=c3["n_bins"], max_radius=c3["max_radius"]), 5, 2)
+        # sub-millisecond, instruction-bound calls: warmed up like the headline loop (see --warmup)
+        m3 = event_ms(lambda: BinnedSelectKnn(c3["K"], co3, rs3, n_bins=c3["n_bins"], max_radius=c3["max_radius"]), 30, 100)
         extra["cfg3_knn_ms"] = round(m3[0], 3)
         extra["cfg3_queries_per_s"] = round(len(c3["coords"]) / (m3[0] * 1e-3), 1)
         # a 4-D Gaussian blob (the shape of a learned coordinate space): N=150k, K=65
         blob = torch.from_numpy(np.random.default_rng(5).standard_normal((150000, 4)).astype(np.float32)).to(dev)
-        mb = event_ms(lambda: BinnedSelectKnn(65, blob, rs, n_bins=30), 5, 2)
+        mb = event_ms(lambda: BinnedSelectKnn(65, blob, rs, n_bins=30), 30, 150)
         extra["knn_gaussian_blob_4d_N150k_K65_ms"] = round(mb[0], 3)
         c5 = workloads.cfg5(ragged=True)
         a5 = [torch.from_numpy(c5[k]).to(dev) for k in ("ccoords", "betas", "dist", "row_splits")]
         for mode in (True, False):
-            m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode), 5, 2)
+            m5 = event_ms(lambda: BuildAndAssignCondensatesBinned(*a5, c5["beta_threshold"], assign_by_max_beta=mode), 30, 100)
             extra["cfg5_condensates_ms_max_beta" if mode else "cfg5_condensates_ms_min_dist"] = round(m5[0], 3)
         # PushKnn forward / gradient over the cfg4 neighbour table (F=128)
         from hgcalml_amd import PushKnn
@@ -338,7 +339,7 @@ def main():
             out, _, _, dist = layer(xg, rs2)
             (out.sum() + dist.sum()).backward()
             xg.grad = None
-        mg = event_ms(gravnet_step, 5, 2)
+        mg = event_ms(gravnet_step, 20, 40)
         extra["gravnet_block_fwd_bwd_ms_N150k_K64_F64"] = round(mg[0], 3)
     except Exception as e:  # information only; never hide the headline numbers
         extra["info_error"] = repr(e)
