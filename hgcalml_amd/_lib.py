@@ -53,6 +53,7 @@ _SIGNATURES = {
     "hgc_accumulate_knn_grad_records_pays": (_c_int, [_c_int] * 4),
     "hgc_accumulate_knn_grad_records": (_c_int, [_ptr] * 11 + [_c_int] * 6 + [_ptr, _c_size, _ptr]),
     "hgc_select_knn_grad": (_c_int, [_ptr] * 7 + [_c_int] * 3 + [_ptr]),
+    "hgc_select_knn_grad_ordered": (_c_int, [_ptr] * 8 + [_c_int] * 3 + [_ptr]),
     "hgc_local_distance": (_c_int, [_ptr] * 3 + [_c_int] * 4 + [_ptr]),
     "hgc_neighbour_covariance": (_c_int, [_ptr] * 8 + [_c_int] * 4 + [_ptr]),
     "hgc_push_knn": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),

@@ -34,18 +34,24 @@ namespace {
 // One thread per (vertex i, coordinate c). d(dist_ik)/d(x_i) summed over the
 // vertex's own neighbours first, in slot order, then the terms of every (v, n)
 // that names i, in ascending (v, n) order. Each term is formed in double and
-// rounded once, as the reference's `2. * g * (x_k - x_i)` is.
+// rounded once, as the reference's `2. * g * (x_k - x_i)` is. With a processing
+// order (a permutation of the vertices, e.g. the kNN's bin order) neighbouring
+// threads work on vertices that share neighbours, whose coordinates then come
+// from the first-level cache; the results do not depend on it.
 __global__ __launch_bounds__(256) void select_knn_grad_kernel(const float *__restrict__ grad_dist,
                                                               const int *__restrict__ idx,
                                                               const float *__restrict__ coord,
                                                               const int *__restrict__ inv_off,
                                                               const int *__restrict__ inv_slots,
                                                               float *__restrict__ grad_coord, int n_vert, int K, int C,
-                                                              const acc::FastDiv div_k) {
+                                                              const acc::FastDiv div_k,
+                                                              const int *__restrict__ order) {
     const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    const int i = (int)(t / C);
-    if (i >= n_vert) return;
-    const int c = (int)(t - (long long)i * C);
+    const int r = (int)(t / C);
+    if (r >= n_vert) return;
+    const int c = (int)(t - (long long)r * C);
+    const int i = order ? order[r] : r;
+    if ((uint32_t)i >= (uint32_t)n_vert) return;  // not a permutation: that vertex is left out
     const float xi = coord[(size_t)i * C + c];
 
     // loads of U slots are issued together; the additions stay in slot / list order
@@ -380,9 +386,10 @@ int hgc_neighbour_covariance(const float *d_coords, const float *d_weights, cons
     return HGC_ERR_UNSUPPORTED;
 }
 
-int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const float *d_dist, const float *d_coord,
-                        const int *d_inv_offsets, const int *d_inv_slots, float *d_grad_coord, int n_vert, int n_neigh,
-                        int n_coords, hgc_stream_t stream) {
+int hgc_select_knn_grad_ordered(const float *d_grad_dist, const int *d_indices, const float *d_dist,
+                                const float *d_coord, const int *d_inv_offsets, const int *d_inv_slots,
+                                const int *d_vertex_order, float *d_grad_coord, int n_vert, int n_neigh, int n_coords,
+                                hgc_stream_t stream) {
     (void)d_dist;  // carried by the reference op, not used by its kernels
     HGC_REQUIRE(n_vert >= 0 && n_neigh >= 1 && n_coords >= 1, "bad sizes");
     HGC_REQUIRE((long long)n_vert * std::max(n_neigh, n_coords) < (1ll << 31), "tensor too large for int32 indexing");
@@ -391,8 +398,15 @@ int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const fl
     const long long threads = (long long)n_vert * n_coords;
     select_knn_grad_kernel<<<ceil_div(threads, 256), 256, 0, as_stream(stream)>>>(
         d_grad_dist, d_indices, d_coord, d_inv_offsets, d_inv_slots, d_grad_coord, n_vert, n_neigh, n_coords,
-        acc::make_fast_div(n_neigh));
+        acc::make_fast_div(n_neigh), d_vertex_order);
     return check_launch("select_knn_grad_kernel");
+}
+
+int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const float *d_dist, const float *d_coord,
+                        const int *d_inv_offsets, const int *d_inv_slots, float *d_grad_coord, int n_vert, int n_neigh,
+                        int n_coords, hgc_stream_t stream) {
+    return hgc_select_knn_grad_ordered(d_grad_dist, d_indices, d_dist, d_coord, d_inv_offsets, d_inv_slots, nullptr,
+                                       d_grad_coord, n_vert, n_neigh, n_coords, stream);
 }
 
 int hgc_local_distance(const int *d_neigh_idxs, const float *d_coords, float *d_distances, int n_coords, int n_in_vert,

@@ -483,8 +483,8 @@ def select_knn_grad(grad_distances: torch.Tensor, indices: torch.Tensor, distanc
     n, k = idx.shape
     inv_offsets, inv_slots = cached_inverse_neighbour_index(indices if indices is idx else idx)
     out = torch.empty_like(x)
-    check(lib.hgc_select_knn_grad(p(g), p(idx), p(d), p(x), p(inv_offsets), p(inv_slots), p(out), n, k, x.shape[1],
-                                  stream()))
+    check(lib.hgc_select_knn_grad_ordered(p(g), p(idx), p(d), p(x), p(inv_offsets), p(inv_slots),
+                                          p(vertex_order_of(indices)), p(out), n, k, x.shape[1], stream()))
     return out
 
 

@@ -957,6 +957,21 @@ def test_select_knn_grad(oracle, K, C):
     shifted.copy_(t(x))
     got = torch.ops.hgcalml.select_knn_grad(t(g), t(idx), t(np.zeros_like(g)), shifted)
     assert (bits(got.cpu().numpy()) == bits(ref)).all()
+    # a processing order of the vertices changes nothing; an order that is no permutation leaves out the
+    # vertices it does not name and touches nothing else
+    from hgcalml_amd import ops
+    from hgcalml_amd._lib import check, lib, p, stream
+    tg, ti, tx = t(g), t(idx), t(x)
+    inv = ops.inverse_neighbour_index(ti)
+    perm = rng.permutation(n).astype(np.int32)
+    broken = perm.copy()
+    broken[:10] = [-1, n, n + 7, -5, 2**30, -2**31, n, -1, n, n]
+    for order, named in ((perm, np.ones(n, bool)), (broken, np.isin(np.arange(n), broken[10:]))):
+        out = torch.full((n, C), 777.0, device=DEV)
+        check(lib.hgc_select_knn_grad_ordered(p(tg), p(ti), None, p(tx), p(inv[0]), p(inv[1]), p(t(order)), p(out), n, K, C,
+                                              stream()))
+        out = out.cpu().numpy()
+        assert (bits(out[named]) == bits(ref[named])).all() and (out[~named] == 777.0).all()
 
 
 def test_knn_distance_gradient_through_wrapper(oracle):
