@@ -55,8 +55,10 @@ _SIGNATURES = {
     "hgc_select_knn_grad": (_c_int, [_ptr] * 7 + [_c_int] * 3 + [_ptr]),
     "hgc_select_knn_grad_ordered": (_c_int, [_ptr] * 8 + [_c_int] * 3 + [_ptr]),
     "hgc_local_distance": (_c_int, [_ptr] * 3 + [_c_int] * 4 + [_ptr]),
+    "hgc_local_distance_ordered": (_c_int, [_ptr] * 4 + [_c_int] * 4 + [_ptr]),
     "hgc_neighbour_covariance": (_c_int, [_ptr] * 8 + [_c_int] * 4 + [_ptr]),
     "hgc_push_knn": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),
+    "hgc_push_knn_ordered": (_c_int, [_ptr] * 7 + [_c_int] * 3 + [_ptr]),
     "hgc_push_knn_grad": (_c_int, [_ptr] * 6 + [_c_int] * 3 + [_ptr]),
     "hgc_exp_neg": (_c_int, [_ptr, _ptr, ctypes.c_longlong, _ptr]),
     "hgc_exp_neg_grad": (_c_int, [_ptr, _ptr, _ptr, ctypes.c_longlong, _ptr]),

@@ -102,14 +102,21 @@ __global__ __launch_bounds__(256) void select_knn_grad_kernel(const float *__res
 }
 
 // one thread per (vertex, slot): serial fp32 sum over the coordinates, 0 for a
-// missing neighbour and for the vertex itself
+// missing neighbour and for the vertex itself (order: see select_knn_grad_kernel)
 __global__ __launch_bounds__(256) void local_distance_kernel(const int *__restrict__ idx,
                                                              const float *__restrict__ coord,
                                                              float *__restrict__ dist, int C, int n_in_vert,
-                                                             long long total, int K) {
-    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+                                                             long long total, int K, const int *__restrict__ order,
+                                                             int n_out_vert) {
+    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= total) return;
-    const int i = (int)(t / K);
+    int i = (int)(t / K);
+    if (order) {
+        const int n = (int)(t - (long long)i * K);
+        i = order[i];
+        if ((uint32_t)i >= (uint32_t)n_out_vert) return;  // not a permutation: that vertex is left out
+        t = (long long)i * K + n;
+    }
     const int j = idx[t];
     float dsq = 0.f;
     if (j >= 0 && j < n_in_vert && j != i) {
@@ -409,27 +416,42 @@ int hgc_select_knn_grad(const float *d_grad_dist, const int *d_indices, const fl
                                        d_grad_coord, n_vert, n_neigh, n_coords, stream);
 }
 
-int hgc_local_distance(const int *d_neigh_idxs, const float *d_coords, float *d_distances, int n_coords, int n_in_vert,
-                       int n_out_vert, int n_neigh, hgc_stream_t stream) {
+int hgc_local_distance_ordered(const int *d_neigh_idxs, const float *d_coords, const int *d_vertex_order,
+                               float *d_distances, int n_coords, int n_in_vert, int n_out_vert, int n_neigh,
+                               hgc_stream_t stream) {
     HGC_REQUIRE(n_in_vert >= 0 && n_out_vert >= 0 && n_out_vert <= n_in_vert && n_neigh >= 1 && n_coords >= 1,
                 "bad sizes");
     HGC_REQUIRE((long long)n_out_vert * n_neigh < (1ll << 31), "tensor too large for int32 indexing");
     if (n_out_vert == 0) return HGC_OK;
     HGC_REQUIRE(d_neigh_idxs && d_coords && d_distances, "null pointer");
     const long long total = (long long)n_out_vert * n_neigh;
-    local_distance_kernel<<<ceil_div(total, 256), 256, 0, as_stream(stream)>>>(d_neigh_idxs, d_coords, d_distances,
-                                                                              n_coords, n_in_vert, total, n_neigh);
+    local_distance_kernel<<<ceil_div(total, 256), 256, 0, as_stream(stream)>>>(
+        d_neigh_idxs, d_coords, d_distances, n_coords, n_in_vert, total, n_neigh, d_vertex_order, n_out_vert);
     return check_launch("local_distance_kernel");
 }
 
-int hgc_push_knn(const float *d_weights, const float *d_feat, const int *d_idxs, const int *d_inv_offsets,
-                 const int *d_inv_slots, float *d_out_feat, int n_vert, int n_neigh, int n_feat, hgc_stream_t stream) {
+int hgc_local_distance(const int *d_neigh_idxs, const float *d_coords, float *d_distances, int n_coords, int n_in_vert,
+                       int n_out_vert, int n_neigh, hgc_stream_t stream) {
+    return hgc_local_distance_ordered(d_neigh_idxs, d_coords, nullptr, d_distances, n_coords, n_in_vert, n_out_vert,
+                                      n_neigh, stream);
+}
+
+int hgc_push_knn_ordered(const float *d_weights, const float *d_feat, const int *d_idxs, const int *d_inv_offsets,
+                         const int *d_inv_slots, const int *d_vertex_order, float *d_out_feat, int n_vert, int n_neigh,
+                         int n_feat, hgc_stream_t stream) {
     (void)d_idxs;  // the inverse index carries all the op needs of the neighbour table
     HGC_REQUIRE(n_vert <= 0 || d_out_feat, "null pointer");
     // out[m, f] = sum over (v, n) naming m of feat[v, f] * w[v, n]: the mean-only
     // feature gradient of the accumulation with `feat` as upstream gradient, not divided by K
     return accumulate_gradient(d_feat, d_weights, nullptr, nullptr, nullptr, nullptr, d_inv_offsets, d_inv_slots,
-                               nullptr, d_out_feat, n_vert, n_neigh, n_feat, n_feat, 0, 1.f, nullptr, nullptr, 0, stream);
+                               nullptr, d_out_feat, n_vert, n_neigh, n_feat, n_feat, 0, 1.f, d_vertex_order, nullptr, 0,
+                               stream);
+}
+
+int hgc_push_knn(const float *d_weights, const float *d_feat, const int *d_idxs, const int *d_inv_offsets,
+                 const int *d_inv_slots, float *d_out_feat, int n_vert, int n_neigh, int n_feat, hgc_stream_t stream) {
+    return hgc_push_knn_ordered(d_weights, d_feat, d_idxs, d_inv_offsets, d_inv_slots, nullptr, d_out_feat, n_vert,
+                                n_neigh, n_feat, stream);
 }
 
 int hgc_push_knn_grad(const float *d_grad, const float *d_weights, const float *d_feat, const int *d_idxs,

@@ -496,7 +496,11 @@ def local_distance(coordinates: torch.Tensor, neighbour_idxs: torch.Tensor) -> t
     if x.dim() != 2 or idx.dim() != 2 or idx.shape[0] > x.shape[0]:
         raise ValueError("LocalDistanceOp expects coordinates [N,C] and neighbour indices [M<=N,K]")
     out = torch.empty(idx.shape, dtype=torch.float32, device=dev)
-    check(lib.hgc_local_distance(p(idx), p(x), p(out), x.shape[1], x.shape[0], idx.shape[0], idx.shape[1], stream()))
+    order = vertex_order_of(neighbour_idxs)
+    if order is not None and order.numel() != idx.shape[0]:
+        order = None
+    check(lib.hgc_local_distance_ordered(p(idx), p(x), p(order), p(out), x.shape[1], x.shape[0], idx.shape[0],
+                                         idx.shape[1], stream()))
     return out
 
 
@@ -519,7 +523,8 @@ def push_knn(weights: torch.Tensor, features: torch.Tensor, indices: torch.Tenso
     n, k = idx.shape
     inv_offsets, inv_slots = cached_inverse_neighbour_index(indices if indices is idx else idx)
     out = torch.empty_like(x)
-    check(lib.hgc_push_knn(p(w), p(x), p(idx), p(inv_offsets), p(inv_slots), p(out), n, k, x.shape[1], stream()))
+    check(lib.hgc_push_knn_ordered(p(w), p(x), p(idx), p(inv_offsets), p(inv_slots), p(vertex_order_of(indices)), p(out),
+                                   n, k, x.shape[1], stream()))
     return out
 
 

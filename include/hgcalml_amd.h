@@ -439,6 +439,13 @@ int hgc_select_knn_grad_ordered(const float *d_grad_dist, const int *d_indices, 
 int hgc_local_distance(const int *d_neigh_idxs, const float *d_coords, float *d_distances,
                        int n_coords, int n_in_vert, int n_out_vert, int n_neigh,
                        hgc_stream_t stream);
+/* The same with a processing order of the n_out_vert vertices (may be NULL), as
+ * for hgc_select_knn_grad_ordered: same results, 0.16 -> 0.12 ms at N=150k,
+ * K=64, C=4 on shuffled points. No counterpart in the reference. */
+int hgc_local_distance_ordered(const int *d_neigh_idxs, const float *d_coords,
+                               const int *d_vertex_order, float *d_distances,
+                               int n_coords, int n_in_vert, int n_out_vert, int n_neigh,
+                               hgc_stream_t stream);
 
 /* Feature-weighted mean and covariance of the neighbours' coordinates, as the
  * wrapper modules/neighbour_covariance_op.py:8-62 composes them from three
@@ -473,6 +480,13 @@ int hgc_neighbour_covariance(const float *d_coords, const float *d_weights, cons
 int hgc_push_knn(const float *d_weights, const float *d_feat, const int *d_idxs,
                  const int *d_inv_offsets, const int *d_inv_slots, float *d_out_feat,
                  int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
+/* The same with a processing order of the target vertices (may be NULL), as
+ * for hgc_accumulate_knn_slots: same bits, 0.49 -> 0.24 ms at N=150k, K=64,
+ * F=64 on shuffled points. No counterpart in the reference. */
+int hgc_push_knn_ordered(const float *d_weights, const float *d_feat, const int *d_idxs,
+                         const int *d_inv_offsets, const int *d_inv_slots,
+                         const int *d_vertex_order, float *d_out_feat,
+                         int n_vert, int n_neigh, int n_feat, hgc_stream_t stream);
 
 /* Gradients of hgc_push_knn. Replaces PushKnnGradOpFunctor
  * (modules/compiled/push_knn_grad_kernel.h, _kernel.cc:23-71):

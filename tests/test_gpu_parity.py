@@ -1016,6 +1016,15 @@ def test_push_knn_and_gradient(oracle, K, F):
     scale = (np.abs(g[np.maximum(idx, 0)]) * np.abs(x)[:, None, :]).sum(-1)
     assert (np.abs(tw.grad.cpu().numpy() - rwg) <= 1e-5 * scale + 1e-30).all()
     assert (tw.grad.cpu().numpy()[idx < 0] == 0).all()
+    # with a processing order of the target vertices: the same bits
+    from hgcalml_amd import ops
+    from hgcalml_amd._lib import check, lib, p, stream
+    ti, tw0, tx0 = t(idx), t(w), t(x)
+    inv = ops.inverse_neighbour_index(ti)
+    ordered = torch.empty((n, F), device=DEV)
+    check(lib.hgc_push_knn_ordered(p(tw0), p(tx0), p(ti), p(inv[0]), p(inv[1]), p(t(rng.permutation(n).astype(np.int32))),
+                                   p(ordered), n, K, F, stream()))
+    assert (bits(ordered.cpu().numpy()) == bits(ref)).all()
 
 
 @pytest.mark.parametrize("linear", [True, False])
@@ -1173,6 +1182,13 @@ def test_local_distance_and_gradient(oracle):
     # fewer index rows than coordinates (forward only)
     d_part = torch.ops.hgcalml.local_distance(t(x), t(idx[:700]))
     assert torch.equal(d_part, dist.detach()[:700])
+    # with a processing order of the vertices: the same bits
+    from hgcalml_amd._lib import check, lib, p, stream
+    ti, txx = t(idx), t(x)
+    out = torch.empty((n, K), device=DEV)
+    check(lib.hgc_local_distance_ordered(p(ti), p(txx), p(t(rng.permutation(n).astype(np.int32))), p(out), C, n, n, K,
+                                         stream()))
+    assert torch.equal(out, dist.detach())
 
 
 def test_neighbour_covariance(oracle):
